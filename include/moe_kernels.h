@@ -1,0 +1,118 @@
+/*
+ * moe_kernels.h — C ABI of the MoE-layer compute kernels (gfx950 / MI355X).
+ *
+ * These entry points are what a host (the patched MoE module of the reference,
+ * or llama.cpp through the reference's libmoe_cache.so) binds instead of the
+ * per-expert kernels the reference outsources to cuBLAS / exllama / HQQ / ggml.
+ * The reference itself has no source for them: its MoE module contract is only
+ * visible through its stand-in
+ *   eval/demo-simulate/transformers-deepseek-moe.py:36-49  (SimulateMoeLayer.forward)
+ * and the hook sites src/sparse_llm_cache/utils/__init__.py:82-96.
+ *
+ * Conventions: every function returns 0 on success or a negative MOE_E* code and
+ * never aborts (the reference aborts on any failed check, logging.cc:77-81).
+ * All pointers are DEVICE pointers unless the name ends in _host.  `stream` is a
+ * hipStream_t passed as void* (NULL = the null stream).  Nothing here allocates.
+ */
+#ifndef MOE_KERNELS_H
+#define MOE_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_OK 0
+#define MOE_EINVAL (-1)   /* bad argument / unsupported shape */
+#define MOE_EHIP (-2)     /* a HIP runtime call failed: see moe_last_error() */
+#define MOE_ESTATE (-3)   /* call not valid in the current engine state */
+#define MOE_ENOMEM (-4)
+#define MOE_ENOTRESIDENT (-5)
+
+/* gating conventions (k1) */
+#define MOE_ROUTE_SOFTMAX_TOPK 0        /* DeepSeek-MoE / Qwen-MoE: softmax over E, top-k, no renorm */
+#define MOE_ROUTE_SOFTMAX_TOPK_RENORM 1 /* same, weights divided by their sum */
+#define MOE_ROUTE_TOPK_SOFTMAX 2        /* Mixtral: top-k of logits, softmax over the k */
+
+/* weight formats of an expert (all weights [out,in]) */
+#define MOE_FMT_INT4_G128 0 /* tiled int4, group 128 along K, fp16 scales, uint4 zeros */
+#define MOE_FMT_BF16 1      /* row-major bf16: w13 [2I,H] (gate rows then up rows), w2 [H,I] */
+
+const char *moe_last_error(void);
+
+/*
+ * Byte layout of ONE int4 expert inside a cache slot (or inside the resident
+ * shared-expert buffer).  Section offsets are from the expert's base address.
+ *
+ *  w13 = gate_proj and up_proj [I,H] interleaved in 16-row blocks: row-block 2b
+ *        holds gate rows 16b..16b+15, row-block 2b+1 the up rows 16b..16b+15.
+ *  w2  = down_proj [H,I].
+ *  A matrix W[N,K] is stored as tiles (rb = n/16, g = k/128), tile (rb,g) at
+ *  q + (rb*G + g)*1024 bytes: 64 lanes x 4 dwords; lane l holds row 16rb + (l&15),
+ *  k = 128g + 32(l>>4) + 8j + 0..7 in dword j, with element k+i at bit
+ *  (i even ? 2i : 16 + 2(i-1)) (so (dword >> 4m) & 0x000f000f is the pair
+ *  (k+2m, k+2m+1)).  scales: fp16 [N/16][G][16]; zeros: 4 bit [N/16][G][16]
+ *  (8 bytes per tile, row r in byte r/2, low nibble first).  w = (q - z) * s.
+ */
+typedef struct moe_int4_layout {
+  int64_t off13_q, off13_s, off13_z;
+  int64_t off2_q, off2_s, off2_z;
+  int64_t total_bytes; /* = 3*I*H/2 + 3*I*H/128*2 + 3*I*H/128/2 */
+} moe_int4_layout;
+
+/* H, I multiples of 128 and 16.  Reference counterpart: the per-param chunk list
+ * registered through ModelLoader::add_one_expert_param (model_loader.hpp:282-288),
+ * laid end to end as ExpertMemHanlderTensorUnified does (model_loader.cpp:208-234). */
+int moe_int4_layout_make(int H, int I, moe_int4_layout *out);
+
+/* k1a: logits[t*ldl + e] = sum_k x[t,k]*wg[e,k] (+ bias[e]); bf16 inputs, fp32 result.
+ * Summation order is fixed (64 lane partials over k = c*512 + 8*lane + i, then an
+ * xor butterfly 32..1) so the result is bit-reproducible.  H % 8 == 0. */
+int moe_gate_logits(const void *x_bf16, const void *wg_bf16, const float *bias, float *logits,
+                    int T, int H, int E, int ldl, void *stream);
+
+/* k1b: top-k routing.  Selection on the logits, ties toward the lower expert index.
+ * idx [T,k] int32, w [T,k] fp32.  E <= 256, k <= 32. */
+int moe_topk(const float *logits, int T, int E, int ldl, int k, int mode, int *idx, float *w,
+             void *stream);
+
+/* one active routed expert of a layer call */
+typedef struct moe_unit {
+  int32_t expert; /* expert id, -1 = unused entry */
+  int32_t m;      /* tokens routed to it */
+  int32_t row0;   /* first row in the sorted pair order */
+  int32_t pad;
+} moe_unit;
+
+/* k2: stable dispatch of the P = T*k (token,slot) pairs (pair p = t*k + j).
+ * counts[E], offsets[E+1], sorted_pair[P], pos_of_pair[P], sorted_tok[P] (= p / k),
+ * units[max_units] (active experts ascending id, rest m = 0), n_active[1],
+ * active_ids[max_units] int64 (the `unique expert ids` list the reference's module
+ * hands to report_experts, utils/__init__.py:84-88). */
+int moe_dispatch(const int *idx, int T, int k, int E, int *counts, int *offsets, int *sorted_pair,
+                 int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
+                 int64_t *active_ids, int max_units, void *stream);
+
+/* k3 (decode): int4 grouped SwiGLU expert product through the slot table.
+ *   expert_ptr[e] : device address of expert e's slot (0 = not resident -> *err |= 1)
+ *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL
+ *   h_r [P, I] bf16, h_s [T, I_sh] bf16, part_r [P, H] fp32, part_s [T, H] fp32: workspaces
+ * Rows of the routed buffers follow the sorted pair order of moe_dispatch.
+ * Covers tokens-per-expert of any size by chunks of <=16 rows; meant for T <= 16. */
+int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, int k,
+                            const moe_unit *units, int max_units, const int *sorted_tok,
+                            const uint64_t *expert_ptr, const void *shared_ptr, void *h_r,
+                            void *h_s, float *part_r, float *part_s, int *err, void *stream);
+
+/* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
+ * g_t = sigmoid(shared_gate_logit[t]) when shared_gate_logit != NULL, else 1;
+ * part_s may be NULL (no shared expert). */
+int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
+                const int *pos_of_pair, const float *shared_gate_logit, void *y_bf16, int T, int H,
+                int k, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

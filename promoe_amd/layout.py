@@ -1,0 +1,92 @@
+"""Host-side repacking of expert weights into the engine's cache-slot layout.
+
+The exchange format a caller hands over for an int4 matrix W[N,K] is the plain one
+(`qweight` int32 [N,K/8] low-nibble-first along K, `scales` fp16 [N,K/128], `qzeros`
+uint4 packed 8 per int32 over the flat index n*G+g).  The slot layout (see
+include/moe_kernels.h) tiles it 16 rows x 128 k so that one 64-lane dwordx4 load is
+one tile and interleaves the nibbles so that a shift+mask yields bf16 pairs.
+
+Reference counterpart: the reference copies whatever tensors the quantisation
+backend registered, chunk by chunk (worker.cpp:84-105); the repack replaces
+AutoGPTQ's exllama `post_init` shuffle that the reference has to drive through
+temp_move_expert_to_gpu (prefetcher.cpp:663-697, utils/hooks.py:402-440).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+GROUP = 128
+
+# bit position of element i (0..7) of a dword in the slot layout
+_NIB_SHIFT = np.array([0, 16, 4, 20, 8, 24, 12, 28], dtype=np.uint32)
+
+
+def int4_layout(H: int, I: int) -> dict:
+    """Section offsets of one int4 expert (mirror of moe_int4_layout_make)."""
+    assert H % 128 == 0 and I % 128 == 0
+    n13, g13, n2, g2 = 2 * I, H // 128, H, I // 128
+    o = 0
+    out = {}
+    for name, sz in (("off13_q", n13 * H // 2), ("off13_s", n13 * g13 * 2), ("off13_z", n13 * g13 // 2),
+                     ("off2_q", n2 * I // 2), ("off2_s", n2 * g2 * 2), ("off2_z", n2 * g2 // 2)):
+        out[name] = o
+        o += sz
+    out["total_bytes"] = o
+    return out
+
+
+def _unpack_exchange(qweight, scales, qzeros, N, K):
+    G = K // GROUP
+    qw = np.ascontiguousarray(qweight).view(np.uint32).reshape(N, K // 8)
+    q = np.stack([(qw >> np.uint32(4 * j)) & np.uint32(0xF) for j in range(8)], axis=2).reshape(N, K)
+    qz = np.ascontiguousarray(qzeros).view(np.uint32).reshape(-1)
+    z = np.stack([(qz >> np.uint32(4 * j)) & np.uint32(0xF) for j in range(8)], axis=1).reshape(-1)[: N * G]
+    s = np.ascontiguousarray(scales).view(np.float16).reshape(N, G)
+    return q.astype(np.uint32), s, z.reshape(N, G).astype(np.uint8)
+
+
+def tile_int4(q: np.ndarray, s: np.ndarray, z: np.ndarray):
+    """q[N,K] (0..15), s[N,G] fp16, z[N,G] (0..15) -> (qtiles u8, stiles u8, ztiles u8)."""
+    N, K = q.shape
+    assert N % 16 == 0 and K % GROUP == 0
+    G = K // GROUP
+    # [rb, r, g, qd, j, i] -> tile order [rb, g, qd, r, j] with i packed into a dword
+    q6 = q.astype(np.uint32).reshape(N // 16, 16, G, 4, 4, 8)
+    dw = np.zeros(q6.shape[:-1], np.uint32)
+    for i in range(8):
+        dw |= q6[..., i] << _NIB_SHIFT[i]
+    dw = dw.transpose(0, 2, 3, 1, 4)          # [rb, g, qd, r, j]; lane = qd*16 + r
+    qt = np.ascontiguousarray(dw).view(np.uint8).reshape(-1)
+    st = np.ascontiguousarray(s.astype(np.float16).reshape(N // 16, 16, G).transpose(0, 2, 1)).view(np.uint8).reshape(-1)
+    z3 = z.astype(np.uint8).reshape(N // 16, 16, G).transpose(0, 2, 1).reshape(N // 16, G, 8, 2)
+    zt = np.ascontiguousarray(z3[..., 0] | (z3[..., 1] << 4)).reshape(-1)
+    return qt, st, zt
+
+
+def pack_expert_int4(gate, up, down, H: int, I: int) -> np.ndarray:
+    """gate/up/down: (qweight, scales, qzeros) in the exchange format for W_gate[I,H],
+    W_up[I,H], W_down[H,I].  Returns the slot image (uint8, total_bytes)."""
+    lay = int4_layout(H, I)
+    qg, sg, zg = _unpack_exchange(*gate, I, H)
+    qu, su, zu = _unpack_exchange(*up, I, H)
+    qd, sd, zd = _unpack_exchange(*down, H, I)
+
+    def interleave(a, b):  # 16-row blocks: gate block, up block, gate block, ...
+        nb = a.shape[0] // 16
+        return np.stack([a.reshape(nb, 16, -1), b.reshape(nb, 16, -1)], axis=1).reshape(2 * a.shape[0], -1)
+
+    q13, s13, z13 = interleave(qg, qu), interleave(sg, su), interleave(zg, zu)
+    buf = np.zeros(lay["total_bytes"], np.uint8)
+    for off, arr in zip(("off13_q", "off13_s", "off13_z"), tile_int4(q13, s13, z13)):
+        buf[lay[off]: lay[off] + arr.size] = arr
+    for off, arr in zip(("off2_q", "off2_s", "off2_z"), tile_int4(qd, sd, zd)):
+        buf[lay[off]: lay[off] + arr.size] = arr
+    return buf
+
+
+def split_chunks_int4(H: int, I: int):
+    """(name, offset, nbytes) of the six copy chunks of an int4 expert, in slot order."""
+    lay = int4_layout(H, I)
+    names = ["off13_q", "off13_s", "off13_z", "off2_q", "off2_s", "off2_z"]
+    ends = [lay[n] for n in names[1:]] + [lay["total_bytes"]]
+    return [(n.replace("off", "w"), lay[n], e - lay[n]) for n, e in zip(names, ends)]

@@ -1,0 +1,97 @@
+"""Thin torch-tensor wrappers over the kernel entry points of the C ABI.
+
+torch is used for device memory and streams only; every op below runs a
+hand-written HIP kernel from libmoe_engine.so on torch's current stream.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib as L
+from ._lib import lib, ptr, cur_stream, check
+
+
+def _dev(t):
+    assert t.is_cuda and t.is_contiguous(), "expected a contiguous device tensor"
+    return t
+
+
+def gate_logits(x: torch.Tensor, wg: torch.Tensor, bias: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """x [T,H] bf16, wg [E,H] bf16 -> logits [T,E] fp32 (fixed summation order)."""
+    T, H = x.shape
+    E = wg.shape[0]
+    assert x.dtype == torch.bfloat16 and wg.dtype == torch.bfloat16 and wg.shape[1] == H
+    if out is None:
+        out = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    check(lib.moe_gate_logits(ptr(_dev(x)), ptr(_dev(wg)), ptr(bias), ptr(out), T, H, E,
+                              out.stride(0), cur_stream()), "moe_gate_logits")
+    return out
+
+
+def topk(logits: torch.Tensor, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK, E: int | None = None):
+    T = logits.shape[0]
+    E = logits.shape[1] if E is None else E
+    idx = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    check(lib.moe_topk(ptr(_dev(logits)), T, E, logits.stride(0), k, mode, ptr(idx), ptr(w),
+                       cur_stream()), "moe_topk")
+    return idx, w
+
+
+class Dispatch:
+    """Device buffers produced by moe_dispatch."""
+
+    def __init__(self, T: int, k: int, E: int, max_units: int, device):
+        P = T * k
+        i32 = dict(dtype=torch.int32, device=device)
+        self.T, self.k, self.E, self.max_units = T, k, E, max_units
+        self.counts = torch.empty(E, **i32)
+        self.offsets = torch.empty(E + 1, **i32)
+        self.sorted_pair = torch.empty(max(P, 1), **i32)
+        self.pos_of_pair = torch.empty(max(P, 1), **i32)
+        self.sorted_tok = torch.empty(max(P, 1), **i32)
+        self.units = torch.empty(max(max_units, 1), 4, **i32)
+        self.n_active = torch.empty(1, **i32)
+        self.active_ids = torch.empty(max(max_units, 1), dtype=torch.int64, device=device)
+
+
+def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispatch | None = None) -> Dispatch:
+    T, k = idx.shape
+    if max_units is None:
+        max_units = min(E, T * k)
+    d = out if out is not None else Dispatch(T, k, E, max_units, idx.device)
+    check(lib.moe_dispatch(ptr(_dev(idx)), T, k, E, ptr(d.counts), ptr(d.offsets), ptr(d.sorted_pair),
+                           ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units), ptr(d.n_active),
+                           ptr(d.active_ids), max_units, cur_stream()), "moe_dispatch")
+    return d
+
+
+def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
+                        H: int, I: int, I_sh: int):
+    """Returns (part_r [P,H] fp32, part_s [T,H] fp32 or None, err int32[1])."""
+    T, k = d.T, d.k
+    P = T * k
+    dev = x.device
+    h_r = torch.empty(max(P, 1), max(I, 1), dtype=torch.bfloat16, device=dev)
+    part_r = torch.empty(max(P, 1), H, dtype=torch.float32, device=dev)
+    h_s = part_s = None
+    if shared is not None:
+        h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
+        part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    check(lib.moe_experts_decode_int4(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
+                                      ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
+                                      ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
+                                      ptr(err), cur_stream()), "moe_experts_decode_int4")
+    return part_r, part_s, err, h_r, h_s
+
+
+def combine(part_r, part_s, topk_w, pos_of_pair, shared_gate_logit, T: int, H: int, k: int,
+            out: torch.Tensor | None = None):
+    dev = (part_r if part_r is not None else part_s).device
+    if out is None:
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    check(lib.moe_combine(ptr(part_r), ptr(part_s), ptr(topk_w), ptr(pos_of_pair),
+                          ptr(shared_gate_logit), ptr(out), T, H, k, cur_stream()), "moe_combine")
+    return out

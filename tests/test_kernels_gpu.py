@@ -1,0 +1,157 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.synth import Int4Layer
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2  # max |y - ref| / max |ref|  (stated output tolerance of the path)
+
+
+def bf16_dev(a, dev):
+    return torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16).to(dev)
+
+
+@pytest.mark.parametrize("T,H,E", [(1, 2048, 64), (4, 2048, 64), (16, 2048, 64), (5, 4096, 8),
+                                   (3, 3584, 65), (7, 256, 60), (2, 2048, 61)])
+def test_gate_logits_bit_exact(cuda, T, H, E):
+    from promoe_amd import ops
+    print(f"case gate_logits T={T} H={H} E={E}", flush=True)
+    x = O.synth_acts(T, H, seed=1)
+    wg = O.round_bf16(O.synth_weights((E, H), seed=0))
+    bias = O.zipf_gate_bias(E, 1.2)
+    got = ops.gate_logits(bf16_dev(x, cuda), bf16_dev(wg, cuda)).cpu().numpy()
+    ref = O.gate_logits_ordered(x, wg)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    got_b = ops.gate_logits(bf16_dev(x, cuda), bf16_dev(wg, cuda), torch.from_numpy(bias).to(cuda)).cpu().numpy()
+    assert np.array_equal(got_b.view(np.uint32), (ref + bias[None, :]).astype(np.float32).view(np.uint32))
+    # and the order-free product agrees to fp32 rounding
+    assert np.allclose(got, (x.astype(np.float64) @ wg.astype(np.float64).T), rtol=0, atol=1e-4)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("T,E,k", [(1, 64, 6), (16, 64, 6), (33, 60, 4), (5, 8, 2), (9, 64, 8), (4, 200, 8)])
+def test_topk_routing(cuda, T, E, k, mode):
+    from promoe_amd import ops
+    print(f"case topk T={T} E={E} k={k} mode={mode}", flush=True)
+    rng = np.random.default_rng(T * 1000 + E + k)
+    logits = rng.normal(0, 2, (T, E)).astype(np.float32)
+    # constructed ties: duplicate values inside rows, including at the k-th boundary
+    logits[:, E // 2] = logits[:, 1]
+    if T > 2:
+        logits[2, :] = 0.5
+    idx, w = ops.topk(torch.from_numpy(logits).to(cuda), k, mode)
+    ridx, rw = O.topk_route(logits, k, mode)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("T,k,E", [(1, 6, 64), (4, 6, 64), (16, 6, 64), (2048, 4, 60), (4096, 2, 8),
+                                   (515, 8, 64), (300, 3, 200), (0, 6, 64)])
+def test_dispatch_bit_exact(cuda, T, k, E):
+    from promoe_amd import ops
+    print(f"case dispatch T={T} k={k} E={E}", flush=True)
+    rng = np.random.default_rng(T + k + E)
+    # distinct experts per token, skewed popularity
+    p = 1.0 / np.arange(1, E + 1) ** 1.2
+    p /= p.sum()
+    idx = np.stack([rng.choice(E, size=k, replace=False, p=p) for _ in range(T)]).astype(np.int32) \
+        if T else np.zeros((0, k), np.int32)
+    d = ops.dispatch(torch.from_numpy(idx).to(cuda).reshape(T, k), E)
+    counts, offsets, sp, pp = O.dispatch(idx, E)
+    P = T * k
+    assert np.array_equal(d.counts.cpu().numpy(), counts)
+    assert np.array_equal(d.offsets.cpu().numpy(), offsets)
+    assert np.array_equal(d.sorted_pair.cpu().numpy()[:P], sp)
+    assert np.array_equal(d.pos_of_pair.cpu().numpy()[:P], pp)
+    assert np.array_equal(d.sorted_tok.cpu().numpy()[:P], sp // k)
+    act = np.nonzero(counts)[0]
+    n_act = int(d.n_active.cpu()[0])
+    assert n_act == min(len(act), d.max_units)
+    units = d.units.cpu().numpy()[:n_act]
+    assert np.array_equal(units[:, 0], act[:n_act])
+    assert np.array_equal(units[:, 1], counts[act[:n_act]])
+    assert np.array_equal(units[:, 2], offsets[act[:n_act]])
+    assert np.array_equal(d.active_ids.cpu().numpy()[:n_act], act[:n_act])
+    assert np.all(d.units.cpu().numpy()[n_act:d.max_units, 1] == 0)
+
+
+def run_layer_gpu(layer, x, k, mode, dev, resident=None):
+    """gate -> topk -> dispatch -> int4 decode experts -> combine, all on the GPU."""
+    from promoe_amd import ops
+    H, I, E, I_sh = layer.H, layer.I, layer.E, layer.I_sh
+    T = x.shape[0]
+    xd = bf16_dev(x, dev)
+    wg = layer.wg
+    if layer.shared_gate is not None:
+        wg = np.concatenate([wg, layer.shared_gate[None, :]], axis=0)
+    logits = ops.gate_logits(xd, bf16_dev(wg, dev),
+                             None if layer.bias is None else torch.from_numpy(
+                                 np.concatenate([layer.bias, np.zeros(wg.shape[0] - E, np.float32)])).to(dev))
+    idx, w = ops.topk(logits, k, mode, E=E)
+    d = ops.dispatch(idx, E)
+    slots = [torch.from_numpy(s).to(dev) for s in layer.slots]
+    table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
+                          for e in range(E)], dtype=torch.int64, device=dev)
+    shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
+    part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh)
+    sg = logits[:, E].contiguous() if layer.shared_gate is not None else None
+    y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
+    torch.cuda.synchronize()
+    return dict(y=y.float().cpu().numpy(), idx=idx.cpu().numpy(), w=w.cpu().numpy(),
+                logits=logits.cpu().numpy(), err=int(err.cpu()[0]), d=d)
+
+
+def check_layer(layer, T, k, mode, dev, seed=1):
+    x = O.synth_acts(T, layer.H, seed=seed)
+    got = run_layer_gpu(layer, x, k, mode, dev)
+    lg = O.gate_logits_ordered(x, layer.wg)
+    if layer.bias is not None:
+        lg = (lg + layer.bias[None, :]).astype(np.float32)
+    ref = O.moe_forward(x, layer.wg, layer.experts_fp32, k, mode, shared=layer.shared_fp32,
+                        shared_gate=layer.shared_gate, logits=lg)
+    assert got["err"] == 0
+    assert np.array_equal(got["logits"][:, :layer.E].view(np.uint32), lg.view(np.uint32))
+    assert np.array_equal(got["idx"], ref["idx"])          # routing bit-exact
+    counts, offsets, sp, pp = O.dispatch(ref["idx"], layer.E)
+    assert np.array_equal(got["d"].sorted_pair.cpu().numpy()[:T * k], sp)  # permutation bit-exact
+    err = np.abs(got["y"] - ref["out"]).max() / np.abs(ref["out"]).max()
+    print(f"  T={T} k={k} mode={mode} max-rel-err={err:.3e}", flush=True)
+    assert err <= TOL
+    return err
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 7, 16, 21])
+def test_decode_layer_small(cuda, T):
+    print(f"case decode_small T={T}", flush=True)
+    layer = Int4Layer(H=256, I=384, E=8, I_sh=256, seed=3)
+    check_layer(layer, T, 2, 0, cuda)
+
+
+def test_decode_layer_small_variants(cuda):
+    print("case decode_small_variants", flush=True)
+    # no shared expert, Mixtral routing
+    check_layer(Int4Layer(H=512, I=128, E=8, I_sh=0, seed=4), 5, 2, 2, cuda)
+    # sigmoid-gated shared expert, renormalised routing, Zipf bias
+    check_layer(Int4Layer(H=256, I=256, E=60, I_sh=512, seed=5, shared_gate=True, zipf=1.1), 6, 4, 1, cuda)
+    # odd group counts per wave (G = 3 and 5)
+    check_layer(Int4Layer(H=384, I=640, E=4, I_sh=128, seed=6), 3, 2, 0, cuda)
+
+
+@pytest.mark.parametrize("T", [1, 4, 16])
+def test_decode_layer_deepseek_shape(cuda, T):
+    print(f"case decode_deepseek T={T}", flush=True)
+    # DeepSeek-MoE-16B layer shape; 16 experts instead of 64 keeps host-side quantisation short
+    layer = Int4Layer(H=2048, I=1408, E=16, I_sh=2816, seed=0, zipf=1.2)
+    check_layer(layer, T, 6, 0, cuda)
+
+
+def test_non_resident_expert_is_reported(cuda):
+    print("case non_resident", flush=True)
+    layer = Int4Layer(H=256, I=128, E=4, I_sh=0, seed=7)
+    x = O.synth_acts(2, 256)
+    got = run_layer_gpu(layer, x, 2, 0, cuda, resident=set())
+    assert got["err"] == 1
