@@ -106,11 +106,11 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
                             void *h_s, float *part_r, float *part_s, int *err, void *stream);
 
 /* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
- * g_t = sigmoid(shared_gate_logit[t]) when shared_gate_logit != NULL, else 1;
+ * g_t = sigmoid(shared_gate_logit[t*sg_stride]) when shared_gate_logit != NULL, else 1;
  * part_s may be NULL (no shared expert). */
 int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
-                const int *pos_of_pair, const float *shared_gate_logit, void *y_bf16, int T, int H,
-                int k, void *stream);
+                const int *pos_of_pair, const float *shared_gate_logit, int sg_stride, void *y_bf16,
+                int T, int H, int k, void *stream);
 
 #ifdef __cplusplus
 }

@@ -48,7 +48,7 @@ _sig("moe_gate_logits", [vp, vp, vp, vp, i32, i32, i32, i32, vp])
 _sig("moe_topk", [vp, i32, i32, i32, i32, i32, vp, vp, vp])
 _sig("moe_dispatch", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp])
-_sig("moe_combine", [vp, vp, vp, vp, vp, vp, i32, i32, i32, vp])
+_sig("moe_combine", [vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, vp])
 
 
 def check(rc: int, what: str = ""):
@@ -63,3 +63,66 @@ def ptr(t) -> int:
 
 def cur_stream() -> int:
     return torch.cuda.current_stream().cuda_stream
+
+# ---- engine (include/moe_engine.h) ----
+BACKEND_HIP, BACKEND_HOST = 0, 1
+sz = C.c_size_t
+pp = C.POINTER(vp)
+
+
+class Counters(C.Structure):
+    _fields_ = [(n, u64) for n in ("hit", "miss", "ready", "unready", "prefetch_hit", "prefetch_miss",
+                                   "activated", "wait_us", "h2d_bytes", "h2d_copies", "evictions",
+                                   "forwards")]
+
+    def as_dict(self):
+        return {n: int(getattr(self, n)) for n, _ in self._fields_}
+
+
+class LayerDesc(C.Structure):
+    _fields_ = [("H", i32), ("I", i32), ("I_sh", i32), ("top_k", i32), ("route_mode", i32), ("fmt", i32),
+                ("shared_gated", i32), ("gate_w", vp), ("gate_bias", vp), ("shared", vp)]
+
+
+_sig("moe_cfg_create", [i32, i32], vp)
+_sig("moe_cfg_destroy", [vp], None)
+_sig("moe_cfg_set", [vp, C.c_char_p, C.c_char_p])
+_sig("moe_cfg_set_params", [vp, C.POINTER(C.c_char_p), i32])
+_sig("moe_cfg_finalize", [vp])
+_sig("moe_cfg_get", [vp, C.c_char_p, C.c_char_p, i32])
+_sig("moe_engine_create", [vp, i32, vp, pp])
+_sig("moe_engine_destroy", [vp], None)
+_sig("moe_host_alloc", [sz], vp)
+_sig("moe_host_free", [vp], None)
+_sig("moe_register_param", [vp, i32, i32, i32, vp, sz, sz])
+_sig("moe_pin_host", [vp, C.POINTER(i32)])
+_sig("moe_init_slots", [vp])
+_sig("moe_slot_distribution", [i64, i32, C.POINTER(i64)])
+_sig("moe_slot_info", [vp, i32, C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)])
+_sig("moe_launch", [vp])
+_sig("moe_expert_param_ptr", [vp, i32, i32, i32, pp])
+_sig("moe_expert_ptr_table", [vp, i32, pp])
+_sig("moe_flush_table", [vp, i32, vp])
+_sig("moe_expert_status", [vp, i32, i32])
+_sig("moe_is_in_cache", [vp, i32, i32])
+_sig("moe_expert_num_ready", [vp, i32, i32])
+_sig("moe_report_layer_logits", [vp, i32, vp, i32, i32, i32])
+_sig("moe_report_one_layer", [vp, i32, vp, i64])
+_sig("moe_wait_expert", [vp, i32, i32])
+_sig("moe_expert_launched", [vp, i32, i32])
+_sig("moe_layer_done", [vp, i32])
+_sig("moe_acquire_layer", [vp, i32, vp, i64])
+_sig("moe_release_layer", [vp, i32])
+_sig("moe_prefetch_layer", [vp, i32, vp, i64, i32])
+_sig("moe_attach_predictor", [vp, i32])
+_sig("moe_update_priority", [vp, vp, i32, i32])
+_sig("moe_oracle_load", [vp, vp, i64, vp, i64, vp, i64, vp, i64])
+_sig("moe_set_seq", [vp, u64])
+_sig("moe_streams", [vp, pp, pp])
+_sig("moe_drain", [vp])
+_sig("moe_get_counters", [vp, C.POINTER(Counters)])
+_sig("moe_report", [vp, i32, C.c_char_p, i32])
+_sig("moe_set_layer", [vp, i32, C.POINTER(LayerDesc)])
+_sig("moe_forward_prepare", [vp, i32])
+_sig("moe_forward", [vp, i32, vp, i32, vp])
+_sig("moe_last_routing", [vp, pp, pp, pp])

@@ -1,0 +1,221 @@
+// Fused MoE-layer forward on top of the cache engine: the patched MoE module's
+// forward (contract: eval/demo-simulate/transformers-deepseek-moe.py:36-49 of the
+// reference) as one call.  gate -> top-k -> dispatch run on the device; the active
+// expert list comes back to the host once (the reference's `unique().cpu()` sync
+// point), the cache hooks run in the reference's order, experts that are already
+// resident go out as ONE grouped launch, missed experts follow one by one as their
+// copies land (the returned order of report_one_layer), then combine.
+#include <algorithm>
+#include <cstring>
+
+#include "engine_internal.h"
+
+struct LayerState {
+  int max_tokens = 0, max_k = 0, max_units = 0;
+  int E = 0, H = 0, I = 0, I_sh = 0;
+  float *logits = nullptr, *topk_w = nullptr, *part_r = nullptr, *part_s = nullptr;
+  int *idx = nullptr, *counts = nullptr, *offsets = nullptr, *sorted_pair = nullptr, *pos_of_pair = nullptr,
+      *sorted_tok = nullptr, *n_active = nullptr, *err = nullptr;
+  moe_unit *units = nullptr, *units_sub = nullptr;
+  int64_t *active_ids = nullptr;
+  void *h_r = nullptr, *h_s = nullptr;
+  // pinned host mirrors
+  moe_unit *units_host = nullptr, *units_sub_host = nullptr;
+  int *n_active_host = nullptr, *err_host = nullptr;
+  std::vector<void *> dev_allocs, host_allocs;
+  hipEvent_t ev = nullptr;
+  int sub_cursor = 0;
+};
+
+void moe_forward_free(LayerState *s) {
+  if (!s) return;
+  for (auto p : s->dev_allocs) (void)hipFree(p);
+  for (auto p : s->host_allocs) (void)hipHostFree(p);
+  if (s->ev) (void)hipEventDestroy(s->ev);
+  delete s;
+}
+
+#define HIPC(call)                                          \
+  do {                                                      \
+    if (int rc_ = moe_check_hip((call), #call)) return rc_; \
+  } while (0)
+
+extern "C" int moe_set_layer(moe_engine *eng, int layer, const moe_layer_desc *d) {
+  if (!eng || !d) { moe_set_error("moe_set_layer: null"); return MOE_EINVAL; }
+  if (layer < 0 || layer >= eng->cfg.num_layer) { moe_set_error("moe_set_layer: bad layer %d", layer); return MOE_EINVAL; }
+  if (d->H <= 0 || d->H % 128 || d->I <= 0 || d->I % 128 || d->I_sh < 0 || d->I_sh % 128 || d->top_k <= 0 ||
+      d->top_k > eng->cfg.num_expert || d->route_mode < 0 || d->route_mode > 2 || !d->gate_w ||
+      (d->I_sh > 0 && !d->shared) || (d->shared_gated && d->I_sh == 0)) {
+    moe_set_error("moe_set_layer: bad descriptor (H=%d I=%d I_sh=%d k=%d)", d->H, d->I, d->I_sh, d->top_k);
+    return MOE_EINVAL;
+  }
+  if (d->fmt != MOE_FMT_INT4_G128) { moe_set_error("moe_set_layer: weight format %d not supported by this entry point", d->fmt); return MOE_EINVAL; }
+  eng->layer_desc[layer] = *d;
+  return MOE_OK;
+}
+
+template <typename T>
+static int dalloc(LayerState *s, T **p, size_t n) {
+  void *q = nullptr;
+  HIPC(hipMalloc(&q, (n ? n : 1) * sizeof(T)));
+  s->dev_allocs.push_back(q);
+  *p = (T *)q;
+  return MOE_OK;
+}
+template <typename T>
+static int halloc(LayerState *s, T **p, size_t n) {
+  void *q = nullptr;
+  HIPC(hipHostMalloc(&q, (n ? n : 1) * sizeof(T), hipHostMallocDefault));
+  s->host_allocs.push_back(q);
+  *p = (T *)q;
+  return MOE_OK;
+}
+
+extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
+  if (!eng || max_tokens <= 0) { moe_set_error("moe_forward_prepare: bad argument"); return MOE_EINVAL; }
+  if (eng->be->compute_stream() == nullptr && eng->be->copy_stream() == nullptr) {
+    moe_set_error("moe_forward_prepare: the host backend has no compute path");
+    return MOE_ESTATE;
+  }
+  int H = 0, I = 0, I_sh = 0, k = 0;
+  for (auto &d : eng->layer_desc) {
+    if (!d.gate_w) continue;
+    H = std::max(H, d.H); I = std::max(I, d.I); I_sh = std::max(I_sh, d.I_sh); k = std::max(k, d.top_k);
+  }
+  if (H == 0) { moe_set_error("moe_forward_prepare: no layer described (moe_set_layer)"); return MOE_ESTATE; }
+  if (eng->fw) { moe_forward_free(eng->fw); eng->fw = nullptr; }
+  LayerState *s = new LayerState();
+  eng->fw = s;
+  const int E = eng->cfg.num_expert, T = max_tokens;
+  const size_t P = (size_t)T * k;
+  s->max_tokens = T; s->max_k = k; s->E = E; s->H = H; s->I = I; s->I_sh = I_sh;
+  s->max_units = (int)std::min<size_t>(E, P);
+  int rc = 0;
+  rc |= dalloc(s, &s->logits, (size_t)T * (E + 1));
+  rc |= dalloc(s, &s->topk_w, P);
+  rc |= dalloc(s, &s->idx, P);
+  rc |= dalloc(s, &s->counts, E);
+  rc |= dalloc(s, &s->offsets, E + 1);
+  rc |= dalloc(s, &s->sorted_pair, P);
+  rc |= dalloc(s, &s->pos_of_pair, P);
+  rc |= dalloc(s, &s->sorted_tok, P);
+  rc |= dalloc(s, &s->n_active, 1);
+  rc |= dalloc(s, &s->err, 1);
+  rc |= dalloc(s, &s->units, s->max_units);
+  rc |= dalloc(s, &s->units_sub, (size_t)s->max_units * 2);
+  rc |= dalloc(s, &s->active_ids, s->max_units);
+  rc |= dalloc(s, (uint16_t **)&s->h_r, P * I);
+  rc |= dalloc(s, (uint16_t **)&s->h_s, (size_t)T * I_sh);
+  rc |= dalloc(s, &s->part_r, P * H);
+  rc |= dalloc(s, &s->part_s, (size_t)T * H);
+  rc |= halloc(s, &s->units_host, s->max_units);
+  rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
+  rc |= halloc(s, &s->n_active_host, 1);
+  rc |= halloc(s, &s->err_host, 1);
+  if (rc) return MOE_EHIP;
+  HIPC(hipMemset(s->err, 0, sizeof(int)));
+  HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
+  return MOE_OK;
+}
+
+static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
+                     const moe_unit *units_dev, int n_units, bool with_shared, const uint64_t *table,
+                     hipStream_t st) {
+  return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
+                                 s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
+                                 s->part_r, s->part_s, s->err, st);
+}
+
+extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
+  if (!eng) { moe_set_error("null engine"); return MOE_EINVAL; }
+  if (!eng->fatal.empty()) { moe_set_error("engine is in a failed state: %s", eng->fatal.c_str()); return MOE_ESTATE; }
+  if (layer < 0 || layer >= eng->cfg.num_layer || !x || !y || T <= 0) { moe_set_error("moe_forward: bad argument"); return MOE_EINVAL; }
+  LayerState *s = eng->fw;
+  const moe_layer_desc &d = eng->layer_desc[layer];
+  if (!s || !d.gate_w) { moe_set_error("moe_forward: layer %d not described or workspace not prepared", layer); return MOE_ESTATE; }
+  if (T > s->max_tokens) { moe_set_error("moe_forward: T=%d exceeds the prepared workspace (%d)", T, s->max_tokens); return MOE_EINVAL; }
+  if (!eng->launched) { moe_set_error("engine not launched"); return MOE_ESTATE; }
+  const int E = eng->cfg.num_expert, k = d.top_k;
+  hipStream_t st = (hipStream_t)eng->be->compute_stream();
+  const int n_gate_rows = E + (d.shared_gated ? 1 : 0);
+  const int ldl = E + 1;
+  int rc;
+  // hook order of the reference (utils/hooks.py:216-223)
+  if (layer == 0 && (rc = moe_report_layer_logits(eng, 0, x, 1, T, d.H))) return rc;
+  if (!d.gate_bias) {
+    if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+  } else {
+    // the bias covers the routed experts only; the shared-gate row (row E) has none
+    if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+    if (d.shared_gated &&
+        (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+      return rc;
+  }
+  if ((rc = moe_topk(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, st))) return rc;
+  const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
+  if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
+                         s->units, s->n_active, s->active_ids, max_units, st)))
+    return rc;
+  // the active expert list comes back to the host
+  HIPC(hipMemcpyAsync(s->units_host, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
+  HIPC(hipMemcpyAsync(s->n_active_host, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
+  HIPC(hipEventRecord(s->ev, st));
+  HIPC(hipEventSynchronize(s->ev));
+  const int n_act = *s->n_active_host;
+  std::vector<int64_t> ids(n_act);
+  std::unordered_map<int, moe_unit> unit_of;
+  for (int u = 0; u < n_act; ++u) { ids[u] = s->units_host[u].expert; unit_of[s->units_host[u].expert] = s->units_host[u]; }
+  // report_experts (utils/__init__.py:84-88): in-place reorder, hits -> launching, misses queued
+  if ((rc = moe_report_one_layer(eng, layer, ids.data(), n_act))) return rc;
+  const uint64_t *table = nullptr;
+  if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+  // resident experts: one grouped launch, together with the shared expert
+  std::vector<int64_t> later;
+  int n_now = 0;
+  s->sub_cursor = 0;
+  moe_unit *sub_h = s->units_sub_host;
+  {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    for (int i = 0; i < n_act; ++i) {
+      Expert *e = eng->ex(layer, (int)ids[i]);
+      if (eng->cfg.early_preempt && e->status.load() == kLaunching) sub_h[n_now++] = unit_of[(int)ids[i]];
+      else later.push_back(ids[i]);
+    }
+    eng->ctr.ready += (uint64_t)n_now;
+  }
+  if ((rc = moe_flush_table(eng, layer, st))) return rc;
+  const moe_unit *units_now = s->units;
+  if (!later.empty() || n_now != n_act) {
+    if (n_now) HIPC(hipMemcpyAsync(s->units_sub, sub_h, sizeof(moe_unit) * n_now, hipMemcpyHostToDevice, st));
+    units_now = s->units_sub;
+    s->sub_cursor = n_now;
+  }
+  if (n_now > 0 || d.I_sh > 0)
+    if ((rc = run_units(eng, d, s, x, T, units_now, n_now, d.I_sh > 0, table, st))) return rc;
+  // missed experts in the returned order, one at a time as their copies land
+  for (int64_t id : later) {
+    if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
+    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
+    *slot_h = unit_of[(int)id];
+    HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
+    if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, 1, false, table, st))) return rc;
+    s->sub_cursor++;
+    if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
+  }
+  const float *sg = d.shared_gated ? s->logits + E : nullptr;
+  if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k, st)))
+    return rc;
+  if ((rc = moe_release_layer(eng, layer))) return rc;
+  // MoeLayerHook.post_forward (utils/hooks.py:220-223)
+  if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+  return moe_layer_done(eng, layer);
+}
+
+extern "C" int moe_last_routing(moe_engine *eng, const int **idx, const float **w, const int **sorted_pair) {
+  if (!eng || !eng->fw) { moe_set_error("moe_last_routing: no forward workspace"); return MOE_ESTATE; }
+  if (idx) *idx = eng->fw->idx;
+  if (w) *w = eng->fw->topk_w;
+  if (sorted_pair) *sorted_pair = eng->fw->sorted_pair;
+  return MOE_OK;
+}

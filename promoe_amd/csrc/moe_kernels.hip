@@ -428,7 +428,8 @@ __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_
                                                   const float *__restrict__ topk_w,
                                                   const int *__restrict__ pos_of_pair,
                                                   const float *__restrict__ sg_logit,
-                                                  uint16_t *__restrict__ y, int H, int k) {
+                                                  int sg_stride, uint16_t *__restrict__ y, int H,
+                                                  int k) {
   const int t = blockIdx.y;
   const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   if (n >= H) return;
@@ -441,7 +442,7 @@ __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_
     acc.z = fmaf(wj, v.z, acc.z); acc.w = fmaf(wj, v.w, acc.w);
   }
   if (part_s) {
-    const float g = sg_logit ? 1.f / (1.f + expf(-sg_logit[t])) : 1.f;
+    const float g = sg_logit ? 1.f / (1.f + expf(-sg_logit[(size_t)t * sg_stride])) : 1.f;
     const float4 v = *(const float4 *)(part_s + (size_t)t * H + n);
     acc.x = fmaf(g, v.x, acc.x); acc.y = fmaf(g, v.y, acc.y);
     acc.z = fmaf(g, v.z, acc.z); acc.w = fmaf(g, v.w, acc.w);
@@ -605,8 +606,8 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
 }
 
 extern "C" int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
-                           const int *pos_of_pair, const float *sg_logit, void *y, int T, int H,
-                           int k, void *stream) {
+                           const int *pos_of_pair, const float *sg_logit, int sg_stride, void *y,
+                           int T, int H, int k, void *stream) {
   if (!y || T < 0 || H <= 0 || H % 4 || k < 0 || (k > 0 && (!part_r || !topk_w || !pos_of_pair)) ||
       T > 65535) {
     moe_set_error("moe_combine: bad argument (T=%d H=%d k=%d)", T, H, k);
@@ -615,6 +616,6 @@ extern "C" int moe_combine(const float *part_r, const float *part_s, const float
   if (T == 0) return MOE_OK;
   dim3 grid((H / 4 + 255) / 256, T);
   hipLaunchKernelGGL(k_combine, grid, dim3(256), 0, (hipStream_t)stream, part_r, part_s, topk_w,
-                     pos_of_pair, sg_logit, (uint16_t *)y, H, k);
+                     pos_of_pair, sg_logit, sg_stride, (uint16_t *)y, H, k);
   return moe_check_launch("k_combine");
 }

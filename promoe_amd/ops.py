@@ -92,6 +92,7 @@ def combine(part_r, part_s, topk_w, pos_of_pair, shared_gate_logit, T: int, H: i
     dev = (part_r if part_r is not None else part_s).device
     if out is None:
         out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    sg_stride = shared_gate_logit.stride(0) if shared_gate_logit is not None else 0
     check(lib.moe_combine(ptr(part_r), ptr(part_s), ptr(topk_w), ptr(pos_of_pair),
-                          ptr(shared_gate_logit), ptr(out), T, H, k, cur_stream()), "moe_combine")
+                          ptr(shared_gate_logit), sg_stride, ptr(out), T, H, k, cur_stream()), "moe_combine")
     return out

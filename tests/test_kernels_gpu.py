@@ -98,7 +98,7 @@ def run_layer_gpu(layer, x, k, mode, dev, resident=None):
                           for e in range(E)], dtype=torch.int64, device=dev)
     shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
     part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh)
-    sg = logits[:, E].contiguous() if layer.shared_gate is not None else None
+    sg = logits[:, E] if layer.shared_gate is not None else None
     y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
     torch.cuda.synchronize()
     return dict(y=y.float().cpu().numpy(), idx=idx.cpu().numpy(), w=w.cpu().numpy(),
