@@ -120,8 +120,12 @@ int moe_layer_done(moe_engine *eng, int layer);
 /* fused form of the three calls above for a whole layer: report_one_layer, wait for
  * every id, flush the slot table on the compute stream. */
 int moe_acquire_layer(moe_engine *eng, int layer, int64_t *ids, int64_t n);
-/* one event for the layer on the compute stream; every launching expert -> using */
+/* one event for the layer on the compute stream; every launching expert -> using.
+ * Only valid when every expert acquired for the layer has been launched
+ * (after moe_acquire_layer). */
 int moe_release_layer(moe_engine *eng, int layer);
+/* same for an explicit list of launched experts (one shared event) */
+int moe_release_experts(moe_engine *eng, int layer, const int64_t *ids, int64_t n);
 
 /* ---- prefetch request hook: PrefetchLayerTask (prefetcher.hpp:52-58, worker.cpp:41-68) ---- */
 /* Queue speculative copies of `ids` (ranked) for a future layer.  Takes one unit of

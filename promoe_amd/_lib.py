@@ -113,6 +113,7 @@ _sig("moe_expert_launched", [vp, i32, i32])
 _sig("moe_layer_done", [vp, i32])
 _sig("moe_acquire_layer", [vp, i32, vp, i64])
 _sig("moe_release_layer", [vp, i32])
+_sig("moe_release_experts", [vp, i32, vp, i64])
 _sig("moe_prefetch_layer", [vp, i32, vp, i64, i32])
 _sig("moe_attach_predictor", [vp, i32])
 _sig("moe_update_priority", [vp, vp, i32, i32])

@@ -352,9 +352,12 @@ static int cache_miss(moe_engine *eng, Expert *in, bool precise, Expert **victim
     v->status = kIdle;  // a partially fetched expert
   }
   ENG_CHECK(eng, v->slot == slot, "slot bookkeeping mismatch");
-  set_table(eng, v, false);
-  v->slot = -1;
   v->num_ready = 0;
+  if (*victim_wait == nullptr) {
+    set_table(eng, v, false);
+    v->slot = -1;
+  }  // else: the victim keeps its slot address until the fetch thread has waited for it,
+     // as the reference's logical tensor keeps its mapping until the copy starts (worker.cpp:98-101)
   in->slot = slot;
   return 0;
 }
@@ -530,7 +533,10 @@ static void fetch_thread_main(moe_engine *eng) {
     }
     Expert *e = eng->current.e;
     const int start = eng->current.start, stop = eng->current.stop;
-    if (eng->current.wait_victim) resolve_using(eng, eng->current.wait_victim, lk);
+    if (Expert *v = eng->current.wait_victim) {
+      resolve_using(eng, v, lk);
+      if (v->slot == e->slot && !in_cache(eng, v)) { set_table(eng, v, false); v->slot = -1; }
+    }
     char *dst = (char *)eng->pool_base + (size_t)e->slot * eng->slot_stride;
     lk.unlock();
     int rc = 0;
@@ -900,6 +906,29 @@ extern "C" int moe_acquire_layer(moe_engine *eng, int layer, int64_t *ids, int64
     }
   }
   return moe_flush_table(eng, layer, eng->be->compute_stream());
+}
+
+extern "C" int moe_release_experts(moe_engine *eng, int layer, const int64_t *ids, int64_t n) {
+  ENG_GUARD(eng);
+  if (int rc = check_le(eng, layer, 0)) return rc;
+  if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_release_experts: bad ids"); return MOE_EINVAL; }
+  std::lock_guard<std::mutex> lk(eng->mu);
+  void *ev = nullptr;
+  for (int64_t i = 0; i < n; ++i) {
+    if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
+    Expert *x = eng->ex(layer, (int)ids[i]);
+    ENG_CHECK(eng, x->status.load() == kLaunching, "transfer launching->using, but expert %d.%d is in state %d", layer,
+              (int)ids[i], x->status.load());
+    if (!ev) {
+      if (!eng->layer_event[layer]) eng->layer_event[layer] = eng->be->event_create();
+      ev = eng->layer_event[layer];
+      if (ev) eng->be->event_record(ev, eng->be->compute_stream());
+    }
+    x->event = ev;
+    x->status = kUsing;
+  }
+  eng->cv_state.notify_all();
+  return MOE_OK;
 }
 
 extern "C" int moe_release_layer(moe_engine *eng, int layer) {

@@ -170,7 +170,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   const uint64_t *table = nullptr;
   if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
   // resident experts: one grouped launch, together with the shared expert
-  std::vector<int64_t> later;
+  std::vector<int64_t> later, now_ids;
   int n_now = 0;
   s->sub_cursor = 0;
   moe_unit *sub_h = s->units_sub_host;
@@ -178,7 +178,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     std::lock_guard<std::mutex> lk(eng->mu);
     for (int i = 0; i < n_act; ++i) {
       Expert *e = eng->ex(layer, (int)ids[i]);
-      if (eng->cfg.early_preempt && e->status.load() == kLaunching) sub_h[n_now++] = unit_of[(int)ids[i]];
+      if (eng->cfg.early_preempt && e->status.load() == kLaunching) { sub_h[n_now++] = unit_of[(int)ids[i]]; now_ids.push_back(ids[i]); }
       else later.push_back(ids[i]);
     }
     eng->ctr.ready += (uint64_t)n_now;
@@ -192,6 +192,9 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   }
   if (n_now > 0 || d.I_sh > 0)
     if ((rc = run_units(eng, d, s, x, T, units_now, n_now, d.I_sh > 0, table, st))) return rc;
+  // launching -> using right away: the demand copies queued for the missed experts may
+  // pick these slots as victims and must only wait for this launch, not for the whole layer
+  if (n_now > 0 && (rc = moe_release_experts(eng, layer, now_ids.data(), n_now))) return rc;
   // missed experts in the returned order, one at a time as their copies land
   for (int64_t id : later) {
     if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
@@ -206,7 +209,6 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   const float *sg = d.shared_gated ? s->logits + E : nullptr;
   if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k, st)))
     return rc;
-  if ((rc = moe_release_layer(eng, layer))) return rc;
   // MoeLayerHook.post_forward (utils/hooks.py:220-223)
   if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
   return moe_layer_done(eng, layer);

@@ -185,6 +185,10 @@ class PrefetchMngr:
     def release_layer(self, layer_id: int):
         check(lib.moe_release_layer(self._h, layer_id), "release_layer")
 
+    def release_experts(self, layer_id: int, experts):
+        ids = np.ascontiguousarray(np.asarray(experts, dtype=np.int64))
+        check(lib.moe_release_experts(self._h, layer_id, ids.ctypes.data, ids.size), "release_experts")
+
     def prefetch_layer(self, layer_id: int, experts, blocking: bool = True) -> bool:
         ids = np.ascontiguousarray(np.asarray(experts, dtype=np.int64))
         rc = lib.moe_prefetch_layer(self._h, layer_id, ids.ctypes.data, ids.size, 1 if blocking else 0)

@@ -391,3 +391,40 @@ def test_concurrent_fetch_keeps_data_and_bounds(monkeypatch):
             assert sum(pm.is_in_cache(l, e) for e in range(E)) <= pm.slot_info(l)[0]
     pm.drain()
     pm.close()
+
+
+@pytest.mark.timeout(60)
+def test_forward_protocol_with_more_active_experts_than_slots():
+    """The order the fused forward drives the hooks in: resident experts launched and
+    released as one group, then each missed expert waited for, launched and marked.
+    More active experts than slots must stream through without blocking."""
+    Lyr, E, k, P = 1, 16, 4, 2
+    rng = np.random.default_rng(21)
+    pm, bufs = make_engine(Lyr, E, k, P=P, cache_rate=0.25, cache_policy="lru")   # 4 slots
+    sim = CO.CacheSim(Lyr, E, P, k, cache_rate=0.25, policy="lru")
+    for step in range(20):
+        n = int(rng.integers(1, 13))
+        ids = np.sort(rng.choice(E, size=n, replace=False)).astype(np.int64)
+        ref = sim.report_one_layer(0, ids)
+        pm.report_one_layer(0, ids)
+        assert list(ids) == ref
+        now = [int(e) for e in ids if pm.expert_status(0, int(e)) == "launching"]
+        later = [int(e) for e in ids if int(e) not in now]
+        pm.release_experts(0, now)
+        for e in ref:
+            if e in now:
+                sim.wait_expert(0, e); sim.expert_launched(0, e)
+        for e in later:
+            pm.report_one_expert(0, e)
+            for p in range(P):
+                assert np.array_equal(slot_bytes(pm, 0, e, p, 64), bufs[(0, e, p)])
+            pm.one_expert_done(0, e)
+        for e in ref:
+            if e not in now:
+                sim.wait_expert(0, e); sim.expert_launched(0, e)
+        pm.one_moe_layer_done(0); sim.layer_done(0)
+        pm.drain(); sim.drain()
+        assert [e for e in range(E) if pm.is_in_cache(0, e)] == sim.resident(0)
+    c = pm.counters()
+    assert c["miss"] == sim.ctr["miss"] and c["hit"] == sim.ctr["hit"] and c["evictions"] == sim.ctr["evictions"]
+    pm.close()
