@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""MoE-layer decode benchmark on one MI355X.
+
+Workload (BASELINE.json configs[1]): one DeepSeek-MoE-16B-shaped MoE layer in decode,
+int4-g128 experts (hidden 2048, 64 routed experts of intermediate 1408, top-6 softmax
+without renormalisation, shared expert of intermediate 2816), bf16 activations, gate
+logits biased to Zipf(1.2) popularity.  A step is one layer forward (gate -> top-k ->
+dispatch -> cache hooks -> grouped int4 SwiGLU experts -> combine) over T tokens; steps
+walk a stack of 27 such layers (7.8 GB of expert images) so that no step finds its
+weights in a cache left warm by the previous one.
+
+value      tokens/s with every routed expert resident in its HBM slot (steady-state hits)
+roofline   HBM roofline of the dominant kernel (int4 w13 + SwiGLU GEMV)
+cache_run  the same stack at cache rate 0.375 (24 of 64 experts per layer resident, LRU);
+           PCIe-inclusive, reported beside `value`, never as it
+cpu_baseline  the fp32 CPU restatement (per-expert F.linear loop) timed on this host
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import statistics
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2700)
+    ap.add_argument("--warmup", type=int, default=270)
+    ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch): 1, 4 or 16")
+    ap.add_argument("--layers", type=int, default=27)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cache-run", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    return ap.parse_args()
+
+
+def timed_steps(pm, xs, L_, steps, torch):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        pm.forward(i % L_, xs[i % len(xs)], out=xs_out)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def kernel_times(lib):
+    names = ["gate_logits", "topk", "dispatch", "gemv_w13_swiglu", "gemv_w2", "combine"]
+    out = {}
+    for kid, name in enumerate(names):
+        tot, n = C.c_double(), C.c_int()
+        lib.moe_kernel_timing_read(kid, C.byref(tot), C.byref(n))
+        if n.value:
+            out[name] = {"avg_us": tot.value * 1e3 / n.value, "calls": n.value}
+    return out
+
+
+def cpu_baseline(T, H, I, E, I_sh, k, threads):
+    """The oracle's fp32 forward in the reference's structure (per-expert loop), on host cores."""
+    import numpy as np
+    import torch
+    from oracle import moe_oracle as O
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    mk = lambda n, kk: (torch.randn(n, kk, generator=g) * 0.02).numpy()
+    experts = [(mk(I, H), mk(I, H), mk(H, I)) for _ in range(E)]
+    shared = (mk(I_sh, H), mk(I_sh, H), mk(H, I_sh))
+    wg = O.round_bf16(mk(E, H))
+    bias = O.zipf_gate_bias(E, 1.2)
+    times = []
+    for rep in range(7):
+        x = O.synth_acts(T, H, seed=rep + 1)
+        t0 = time.perf_counter()
+        lg = (O.gate_logits(x, wg) + bias[None, :]).astype(np.float32)
+        O.moe_forward(x, wg, experts, k, 0, shared=shared, logits=lg)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times[2:])
+    return T / med, med
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)" % a.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from promoe_amd import synth, layout as LY
+    from promoe_amd._lib import lib
+
+    global xs_out
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    H, I, E, I_sh, k, L_ = 2048, 1408, 64, 2816, 6, a.layers
+    T = a.tokens
+    t_setup = time.perf_counter()
+    stack = synth.Int4Stack(L_, E, H, I, I_sh, k, dev, zipf=1.2, seed=0)
+    print("[bench] stack of %d layers x %d experts (%.2f GB of images) built in %.1f s" %
+          (L_, E, stack.expert_bytes * L_ * E / 1e9, time.perf_counter() - t_setup), file=sys.stderr, flush=True)
+
+    # ---- steady-state hits: every expert resident -------------------------------------
+    pm = stack.engine(16, cache_rate=1.0, cache_policy="lru")
+    import numpy as np
+    for l in range(L_):                      # bring every expert into its slot
+        pm.acquire_layer(l, np.arange(E, dtype=np.int64))
+        pm.release_layer(l)
+    pm.drain()
+    base_ctr = pm.counters()
+
+    def run(Tn, steps, warmup):
+        global xs_out
+        xs = stack.acts(Tn, 8, seed=1)
+        xs_out = torch.empty_like(xs[0])
+        timed_steps(pm, xs, L_, warmup, torch)
+        return timed_steps(pm, xs, L_, steps, torch)
+
+    dt = run(T, a.steps, a.warmup)
+    c1 = pm.counters()
+    assert c1["miss"] == base_ctr["miss"], "steady-state run took cache misses"
+    value = T * a.steps / dt
+
+    # per-kernel durations (HIP events on the launch stream), separate short pass
+    lib.moe_kernel_timing(1)
+    xs = stack.acts(T, 8, seed=1)
+    timed_steps(pm, xs, L_, min(a.steps, 20 * L_), torch)
+    kt = kernel_times(lib)
+    lib.moe_kernel_timing(0)
+    # distinct routed experts per step (D) for the algorithmic byte count
+    d_steps = min(a.steps, 20 * L_)
+    act0 = c1["activated"]
+    D = (pm.counters()["activated"] - act0) / d_steps
+    lay_r, lay_s = LY.int4_layout(H, I), LY.int4_layout(H, I_sh)
+    w13_bytes = D * lay_r["off2_q"] + lay_s["off2_q"] + 2 * T * H       # w13 sections + x
+    layer_bytes = D * lay_r["total_bytes"] + lay_s["total_bytes"] + E * H * 2 + 2 * T * H * 2
+    w13_us = kt["gemv_w13_swiglu"]["avg_us"]
+    achieved = w13_bytes / (w13_us * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "k_gemv_int4<T,true> (w13 + SwiGLU)", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                "algorithmic_bytes_per_launch": w13_bytes, "avg_launch_us": w13_us,
+                "distinct_routed_experts_per_step": D}
+    chain_us = sum(v["avg_us"] for v in kt.values())
+    layer = {"algorithmic_bytes_per_step": layer_bytes, "kernel_chain_us": chain_us,
+             "chain_GBps": layer_bytes / (chain_us * 1e-6) / 1e9,
+             "wall_GBps": layer_bytes / (dt / a.steps) / 1e9}
+
+    sweep = {}
+    if not a.no_sweep:
+        for Tn in (1, 4, 16):
+            if Tn == T:
+                sweep[str(Tn)] = value
+                continue
+            d2 = run(Tn, 20 * L_, 2 * L_)
+            sweep[str(Tn)] = Tn * 20 * L_ / d2
+    pm.close()
+
+    # ---- the configured cache rate: 24 of 64 experts per layer resident, LRU ------------
+    cache_run = None
+    if not a.no_cache_run:
+        pm2 = stack.engine(16, cache_rate=0.375, cache_policy="lru", num_predict_expert_per_layer=0,
+                           reorder_experts=True, early_preempt=True)
+        xs = stack.acts(T, 64, seed=3)
+        xs_out = torch.empty_like(xs[0])
+        n2 = 40 * L_
+        for i in range(10 * L_):              # fill the slots along the Zipf popularity
+            pm2.forward(i % L_, xs[(i // L_) % len(xs)], out=xs_out)
+        torch.cuda.synchronize()
+        c0 = pm2.counters()
+        t0 = time.perf_counter()
+        for i in range(n2):
+            pm2.forward(i % L_, xs[(10 + i // L_) % len(xs)], out=xs_out)
+        torch.cuda.synchronize()
+        d3 = time.perf_counter() - t0
+        c2 = pm2.counters()
+        hit, miss = c2["hit"] - c0["hit"], c2["miss"] - c0["miss"]
+        cache_run = {"cache_rate": 0.375, "policy": "lru", "tokens_per_s": T * n2 / d3, "ms_per_step": d3 / n2 * 1e3,
+                     "hit_rate": hit / max(hit + miss, 1), "h2d_GB": (c2["h2d_bytes"] - c0["h2d_bytes"]) / 1e9,
+                     "h2d_GBps": (c2["h2d_bytes"] - c0["h2d_bytes"]) / d3 / 1e9, "steps": n2}
+        pm2.close()
+
+    cpu = None
+    if not a.no_cpu:
+        threads = 8   # the reference's own torch.set_num_threads(8) (utils/__init__.py:343)
+        v, med = cpu_baseline(T, H, I, E, I_sh, k, threads)
+        cpu = {"value": v, "unit": "tokens/s", "cores": threads, "kind": "port",
+               "sample": "fp32 per-expert F.linear forward of one layer, T=%d, median of 5 after 2 warm-ups "
+                         "(%.1f ms/step); host has %d logical cores" % (T, med * 1e3, os.cpu_count())}
+
+    out = {"metric": "moe_layer_decode_tokens_per_s", "value": value, "unit": "tokens/s", "n_gpus": 1,
+           "steps": a.steps, "warmup": a.warmup, "ms_per_step": dt / a.steps * 1e3, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "DeepSeek-MoE-16B-shaped MoE layer, int4-g128 experts, decode T=%d, "
+                                  "steady-state hits (all routed experts resident), %d-layer stack" % (T, L_),
+                      "hidden": H, "experts": E, "intermediate": I, "shared_intermediate": I_sh, "top_k": k,
+                      "tokens_per_step": T, "layers": L_, "zipf": 1.2},
+           "roofline": roofline, "cpu_baseline": cpu, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
+           "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

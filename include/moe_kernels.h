@@ -112,6 +112,13 @@ int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
                 const int *pos_of_pair, const float *shared_gate_logit, int sg_stride, void *y_bf16,
                 int T, int H, int k, void *stream);
 
+/* Per-kernel timing with HIP events recorded on the launch stream around every kernel
+ * the launchers below start (no reference counterpart; used by the benchmark to report
+ * kernel durations).  kernel_id: 0 gate logits, 1 top-k, 2 dispatch, 3 decode w13+SwiGLU,
+ * 4 decode w2, 5 combine, 6 prefill w13, 7 prefill w2.  enable=1 clears earlier records. */
+int moe_kernel_timing(int enable);
+int moe_kernel_timing_read(int kernel_id, double *total_ms, int *calls);
+
 #ifdef __cplusplus
 }
 #endif

@@ -7,3 +7,9 @@
 void moe_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 int moe_check_launch(const char *what);
 int moe_check_hip(hipError_t e, const char *what);
+
+// Optional per-kernel timing with HIP events on the launch stream (moe_kernel_timing*).
+enum MoeKernelId { MOE_K_GATE = 0, MOE_K_TOPK, MOE_K_DISPATCH, MOE_K_W13, MOE_K_W2, MOE_K_COMBINE,
+                   MOE_K_PREFILL_W13, MOE_K_PREFILL_W2, MOE_K_COUNT };
+void moe_ktimer_begin(int kid, hipStream_t s);
+void moe_ktimer_end(int kid, hipStream_t s);

@@ -481,8 +481,10 @@ extern "C" int moe_gate_logits(const void *x, const void *wg, const float *bias,
   }
   if (T == 0) return MOE_OK;
   dim3 grid((E + 3) / 4, T);
+  moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_gate_logits, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
                      (const uint16_t *)wg, bias, logits, H, E, ldl);
+  moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
   return moe_check_launch("k_gate_logits");
 }
 
@@ -494,8 +496,10 @@ extern "C" int moe_topk(const float *logits, int T, int E, int ldl, int k, int m
     return MOE_EINVAL;
   }
   if (T == 0) return MOE_OK;
+  moe_ktimer_begin(MOE_K_TOPK, (hipStream_t)stream);
   hipLaunchKernelGGL(k_topk, dim3((T + 3) / 4), dim3(256), 0, (hipStream_t)stream, logits, T, E,
                      ldl, k, mode, idx, w);
+  moe_ktimer_end(MOE_K_TOPK, (hipStream_t)stream);
   return moe_check_launch("k_topk");
 }
 
@@ -511,9 +515,11 @@ extern "C" int moe_dispatch(const int *idx, int T, int k, int E, int *counts, in
   int nbits = 0;
   while ((1 << nbits) < E) ++nbits;
   const size_t lds = (size_t)16 * E * sizeof(int);
+  moe_ktimer_begin(MOE_K_DISPATCH, (hipStream_t)stream);
   hipLaunchKernelGGL(k_dispatch, dim3(1), dim3(DISP_THREADS), lds, (hipStream_t)stream, idx,
                      T * k, k, E, nbits, counts, offsets, sorted_pair, pos_of_pair, sorted_tok,
                      units, n_active, (long long *)active_ids, max_units);
+  moe_ktimer_end(MOE_K_DISPATCH, (hipStream_t)stream);
   return moe_check_launch("k_dispatch");
 }
 
@@ -529,7 +535,9 @@ static int launch_gemv(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
     }
     attr_set = true;
   }
+  moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
   hipLaunchKernelGGL((k_gemv_int4<TMAX, SW>), dim3(grid), dim3(256), lds, s, a);
+  moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4");
 }
 
@@ -615,7 +623,9 @@ extern "C" int moe_combine(const float *part_r, const float *part_s, const float
   }
   if (T == 0) return MOE_OK;
   dim3 grid((H / 4 + 255) / 256, T);
+  moe_ktimer_begin(MOE_K_COMBINE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_combine, grid, dim3(256), 0, (hipStream_t)stream, part_r, part_s, topk_w,
                      pos_of_pair, sg_logit, sg_stride, (uint16_t *)y, H, k);
+  moe_ktimer_end(MOE_K_COMBINE, (hipStream_t)stream);
   return moe_check_launch("k_combine");
 }
