@@ -99,11 +99,16 @@ int moe_dispatch(const int *idx, int T, int k, int E, int *counts, int *offsets,
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL
  *   h_r [P, I] bf16, h_s [T, I_sh] bf16, part_r [P, H] fp32, part_s [T, H] fp32: workspaces
  * Rows of the routed buffers follow the sorted pair order of moe_dispatch.
- * Covers tokens-per-expert of any size by chunks of <=16 rows; meant for T <= 16. */
+ * Covers tokens-per-expert of any size by chunks of <=16 rows; meant for T <= 16.
+ * units_host / expert_ptr_host (HOST copies of the unit list and of the slot table row,
+ * both optional): when given and max_units <= 64 the units travel in the kernel arguments
+ * and the kernels read neither `units` nor `expert_ptr`. */
 int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, int k,
                             const moe_unit *units, int max_units, const int *sorted_tok,
                             const uint64_t *expert_ptr, const void *shared_ptr, void *h_r,
-                            void *h_s, float *part_r, float *part_s, int *err, void *stream);
+                            void *h_s, float *part_r, float *part_s, int *err,
+                            const moe_unit *units_host, const uint64_t *expert_ptr_host,
+                            void *stream);
 
 /* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
  * g_t = sigmoid(shared_gate_logit[t*sg_stride]) when shared_gate_logit != NULL, else 1;

@@ -22,7 +22,7 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("MOE_EXTRA_HIPFLAGS", "").split()
 
 
 def _hipcc() -> str:

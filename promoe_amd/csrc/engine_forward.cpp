@@ -119,11 +119,13 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
 }
 
 static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
-                     const moe_unit *units_dev, int n_units, bool with_shared, const uint64_t *table,
-                     hipStream_t st) {
+                     const moe_unit *units_dev, const moe_unit *units_host, int n_units, bool with_shared,
+                     int layer, const uint64_t *table, hipStream_t st) {
+  // the host knows the units and the slot addresses: they travel in the kernel arguments
+  const uint64_t *table_host = eng->h_table + (size_t)layer * eng->cfg.num_expert;
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
-                                 s->part_r, s->part_s, s->err, st);
+                                 s->part_r, s->part_s, s->err, units_host, table_host, st);
 }
 
 extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
@@ -191,7 +193,9 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     s->sub_cursor = n_now;
   }
   if (n_now > 0 || d.I_sh > 0)
-    if ((rc = run_units(eng, d, s, x, T, units_now, n_now, d.I_sh > 0, table, st))) return rc;
+    if ((rc = run_units(eng, d, s, x, T, units_now, units_now == s->units ? s->units_host : sub_h, n_now, d.I_sh > 0,
+                        layer, table, st)))
+      return rc;
   // launching -> using right away: the demand copies queued for the missed experts may
   // pick these slots as victims and must only wait for this launch, not for the whole layer
   if (n_now > 0 && (rc = moe_release_experts(eng, layer, now_ids.data(), n_now))) return rc;
@@ -202,7 +206,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
     *slot_h = unit_of[(int)id];
     HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
-    if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, 1, false, table, st))) return rc;
+    if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
     s->sub_cursor++;
     if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
   }

@@ -241,147 +241,208 @@ __global__ __launch_bounds__(DISP_THREADS) void k_dispatch(
 
 // ---------------------------------------------------------------------------
 // k3 int4 grouped GEMV (decode).  One workgroup (4 waves) owns two adjacent
-// 16-row blocks of one unit's matrix; the waves split the K groups.
+// 16-row blocks of one unit's matrix; wave w takes the K groups w, w+4, w+8, ...
 //   SWIGLU: blocks are (gate rows, up rows) -> out = silu(g)*u, bf16, 16 values
 //   else  : plain product, fp32, 32 values
+// The load section is straight-line code (clamped addresses instead of branches):
+// activations and scale/zero sections first, then the weight tiles, so that the small
+// loads can be staged in LDS while the tiles are still in flight.
 // ---------------------------------------------------------------------------
 struct GemvClass {
-  const uint16_t *act;  // bf16 activations [rows, act_stride]
+  const uint16_t *act;  // bf16 activations [rows, act_stride] (act_stride 0: one shared row)
   const int *gather;    // row -> activation row (NULL = identity)
   void *out;            // bf16 (SWIGLU) or fp32
   long long off_q, off_s, off_z;
-  int K, G, act_stride, out_stride, nblk;
+  int K, G, act_stride, out_stride, nblk, pad;
 };
+#define GEMV_MAX_KUNITS 64
+struct KUnit { unsigned long long base; int m, row0; };
 struct GemvArgs {
   GemvClass cls[2];  // 0 = shared expert, 1 = routed experts
-  const moe_unit *units;
-  const unsigned long long *expert_ptr;
+  const moe_unit *units;                 // device-built unit list (NULL: use ku[])
+  const unsigned long long *expert_ptr;  // device slot table, indexed by expert id
   const unsigned char *shared_base;
   int n_sh_blocks, T;
   int *err;
+  KUnit ku[GEMV_MAX_KUNITS];             // units resolved on the host, passed by value: the
+                                         // weight loads then depend on no global load
 };
 
-template <int TMAX, bool SWIGLU>
-__global__ __launch_bounds__(256) void k_gemv_int4(const GemvArgs a) {
+// global-address-space loads (pointers that come out of the slot table are generic
+// to the compiler and would otherwise become flat_load)
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const u32x4_t g_uint4;
+typedef __attribute__((address_space(1))) const unsigned int g_u32;
+static __device__ __forceinline__ uint4 ldg_u4(const void *p) {
+  const u32x4_t v = *(g_uint4 *)(unsigned long long)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+static __device__ __forceinline__ u32 ldg_u32(const void *p) { return *(g_u32 *)(unsigned long long)p; }
+static __device__ __forceinline__ float sum8_bf16(const uint4 &v) {
+  return bf16lo(v.x) + bf16hi(v.x) + bf16lo(v.y) + bf16hi(v.y) + bf16lo(v.z) + bf16hi(v.z) + bf16lo(v.w) +
+         bf16hi(v.w);
+}
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
+static __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
+}
+static __device__ __forceinline__ uint4 bload16(rsrc_t r, int voff, int soff) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+static __device__ __forceinline__ u32 bload4(rsrc_t r, int voff, int soff) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+
+template <int TMAX, bool SWIGLU, int CH>
+__global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  int ci, b, m, row0;
+  // all kernel arguments are fetched in one batch (both classes, then selected): the
+  // scalar loads do not depend on one another
+  const GemvClass c0 = a.cls[0], c1 = a.cls[1];
+  const int n_sh = a.n_sh_blocks;
+  const bool sh = (int)blockIdx.x < n_sh;
+  GemvClass c;
+  c.act = sh ? c0.act : c1.act; c.gather = sh ? c0.gather : c1.gather; c.out = sh ? c0.out : c1.out;
+  c.off_q = sh ? c0.off_q : c1.off_q; c.off_s = sh ? c0.off_s : c1.off_s; c.off_z = sh ? c0.off_z : c1.off_z;
+  c.K = sh ? c0.K : c1.K; c.G = sh ? c0.G : c1.G; c.act_stride = sh ? c0.act_stride : c1.act_stride;
+  c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk;
+  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
+  const int u = sh ? 0 : rr / c.nblk;
+  const int b = rr - u * c.nblk;
+  int m, row0;
   const unsigned char *base;
-  if ((int)blockIdx.x < a.n_sh_blocks) {
-    ci = 0; b = blockIdx.x; m = a.T; row0 = 0; base = a.shared_base;
-  } else {
-    ci = 1;
-    const int rr = blockIdx.x - a.n_sh_blocks;
-    const int u = rr / a.cls[1].nblk;
-    b = rr - u * a.cls[1].nblk;
+  if (a.units && !sh) {
     const moe_unit ud = a.units[u];
     m = ud.m; row0 = ud.row0;
-    if (m <= 0) return;
-    base = (const unsigned char *)a.expert_ptr[ud.expert];
-    if (base == nullptr) {
-      if (tid == 0) atomicOr(a.err, 1);
-      return;
-    }
+    base = m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
+  } else {
+    const KUnit ku = a.ku[u];
+    m = sh ? a.T : ku.m; row0 = sh ? 0 : ku.row0;
+    base = sh ? a.shared_base : (const unsigned char *)ku.base;
   }
-  const GemvClass &c = a.cls[ci];
+  if (m <= 0) return;
+  if (base == nullptr) {
+    if (tid == 0) atomicOr(a.err, 1);
+    return;
+  }
   const int K = c.K, G = c.G, KS = K >> 5;
-  uint16_t *xs = (uint16_t *)smem;                                // [TMAX][K]
-  float *xsum = (float *)(smem + (size_t)TMAX * K * 2);          // [TMAX][K/32]
-  float *red = xsum + (size_t)TMAX * KS;                          // [4][TMAX][2][16]
+  // LDS: activations, their 32-wide sums, the scale/zero sections of the two row blocks,
+  // and the cross-wave reduction buffer
+  uint16_t *xs = (uint16_t *)smem;                                    // [TMAX][K]
+  float *xsum = (float *)(smem + (size_t)TMAX * K * 2);              // [TMAX][K/32]
+  uint16_t *s_sc = (uint16_t *)(xsum + (size_t)TMAX * KS);            // [2][G][16] fp16
+  unsigned char *s_zz = (unsigned char *)(s_sc + 2 * G * 16);         // [2][G][8]
+  float *red = (float *)(s_zz + 2 * G * 8);                           // [4][TMAX][2][16]
 
-  const int g0 = (w * G) >> 2, g1 = ((w + 1) * G) >> 2;
-  const int rbA = 2 * b, rbB = 2 * b + 1;
-  const uint4 *qA = (const uint4 *)(base + c.off_q) + (size_t)rbA * G * 64 + lane;
-  const uint4 *qB = (const uint4 *)(base + c.off_q) + (size_t)rbB * G * 64 + lane;
-  const uint16_t *sA = (const uint16_t *)(base + c.off_s) + (size_t)rbA * G * 16 + r;
-  const uint16_t *sB = (const uint16_t *)(base + c.off_s) + (size_t)rbB * G * 16 + r;
-  const unsigned char *zA = base + c.off_z + (size_t)rbA * G * 8 + (r >> 1);
-  const unsigned char *zB = base + c.off_z + (size_t)rbB * G * 8 + (r >> 1);
+  const int GPW = (G - w + 3) >> 2;  // groups of this wave: g = w + 4j, j < GPW
+  const int rbA = 2 * b;
+  // tiles of block A then block B are contiguous: 2*G KiB
+  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, 2u * G * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, 2u * G * 32u);
+  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, 2u * G * 8u);
+  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
   const int zsh = (r & 1) * 4;
-
-  constexpr int CH = 4;
-  uint4 wa[CH], wb[CH];
-  uint16_t sa[CH], sb[CH];
-  unsigned char za[CH], zb[CH];
-  auto load_chunk = [&](int gc) {
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const int g = gc + i;
-      if (g < g1) {
-        wa[i] = qA[(size_t)g * 64];
-        wb[i] = qB[(size_t)g * 64];
-        sa[i] = sA[g * 16];
-        sb[i] = sB[g * 16];
-        za[i] = zA[g * 8];
-        zb[i] = zB[g * 8];
-      }
-    }
-  };
+  const int vec_per_row = K >> 3;
+  const int n_sc = 2 * G * 8;   // dwords of scales
+  const int n_zz = 2 * G * 2;   // dwords of zeros
+  constexpr int XT = TMAX < 2 ? TMAX : 2;  // rows whose first 256 vectors are staged through registers
 
   for (int t0 = 0; t0 < m; t0 += TMAX) {
     const int mc = (m - t0) < TMAX ? (m - t0) : TMAX;
-    load_chunk(g0);  // weights in flight while the activations are staged
-    // stage activations
-    const int vec_per_row = K >> 3;
-    for (int i = tid; i < mc * vec_per_row; i += 256) {
-      const int t = i / vec_per_row, v = i - t * vec_per_row;
+    // ---- straight-line load section: small loads first, then the weight tiles --------------
+    uint4 xv[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+      const int row = row0 + t0 + (t < mc ? t : 0);
+      const int arow = c.gather ? c.gather[row] : row;  // uniform: a scalar load
+      // threads past the row's end re-read vector 0 (staged nowhere): never past the tensor
+      xv[t] = bload16(rx, (tid < vec_per_row ? tid : 0) * 16, arow * c.act_stride * 2);
+    }
+    const u32 msc0 = bload4(rs, tid * 4, 0), msc1 = bload4(rs, tid * 4, 1024);
+    const u32 mzz = bload4(rz, tid * 4, 0);
+    uint4 wa[CH], wb[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int g = j < GPW ? w + 4 * j : 0;  // clamped: tile 0 always exists
+      wa[j] = bload16(rq, lane * 16, g * 1024);
+      wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+    }
+    // ---- stage: x -> LDS (+ 32-wide sums via a quad reduction), scale/zero -> LDS ----------
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+      float ps = sum8_bf16(xv[t]);
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      if (tid < vec_per_row && t < mc) {
+        ((uint4 *)xs)[t * vec_per_row + tid] = xv[t];
+        if ((tid & 3) == 0) xsum[(t * vec_per_row + tid) >> 2] = ps;
+      }
+    }
+    if (tid < n_sc) ((u32 *)s_sc)[tid] = msc0;
+    if (tid + 256 < n_sc) ((u32 *)s_sc)[tid + 256] = msc1;
+    if (tid < n_zz) ((u32 *)s_zz)[tid] = mzz;
+    // leftovers (more rows, K > 2048): plain loops
+    for (int t = 0; t < mc; ++t) {
       const int row = row0 + t0 + t;
       const int arow = c.gather ? c.gather[row] : row;
-      ((uint4 *)xs)[(size_t)t * vec_per_row + v] =
-          ((const uint4 *)(c.act + (size_t)arow * c.act_stride))[v];
-    }
-    __syncthreads();
-    for (int i = tid; i < mc * KS; i += 256) {
-      const int t = i / KS, s = i - t * KS;
-      const uint4 *p = (const uint4 *)(xs + (size_t)t * K + s * 32);
-      float acc = 0.f;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint4 v = p[j];
-        acc += bf16lo(v.x); acc += bf16hi(v.x); acc += bf16lo(v.y); acc += bf16hi(v.y);
-        acc += bf16lo(v.z); acc += bf16hi(v.z); acc += bf16lo(v.w); acc += bf16hi(v.w);
+      for (int v = tid + (t < XT ? 256 : 0); v < vec_per_row; v += 256) {
+        const uint4 x4 = bload16(rx, v * 16, arow * c.act_stride * 2);
+        float ps = sum8_bf16(x4);
+        ps += __shfl_xor(ps, 1, 64);
+        ps += __shfl_xor(ps, 2, 64);
+        ((uint4 *)xs)[t * vec_per_row + v] = x4;
+        if ((tid & 3) == 0) xsum[(t * vec_per_row + v) >> 2] = ps;
       }
-      xsum[i] = acc;
     }
+    for (int i = tid + 512; i < n_sc; i += 256) ((u32 *)s_sc)[i] = bload4(rs, i * 4, 0);
+    for (int i = tid + 256; i < n_zz; i += 256) ((u32 *)s_zz)[i] = bload4(rz, i * 4, 0);
     __syncthreads();
 
     float accA[TMAX], accB[TMAX];
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) { accA[t] = 0.f; accB[t] = 0.f; }
 
-    for (int gc = g0; gc < g1; gc += CH) {
-      uint4 ca[CH], cb[CH];
-      float fsa[CH], fsb[CH], fza[CH], fzb[CH];
+    for (int jc = 0; jc < GPW; jc += CH) {
+      if (jc > 0) {
 #pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        ca[i] = wa[i]; cb[i] = wb[i];
-        fsa[i] = half_bits_to_f32(sa[i]); fsb[i] = half_bits_to_f32(sb[i]);
-        fza[i] = 128.f + (float)((za[i] >> zsh) & 15);
-        fzb[i] = 128.f + (float)((zb[i] >> zsh) & 15);
+        for (int j = 0; j < CH; ++j) {
+          const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
+          wa[j] = bload16(rq, lane * 16, g * 1024);
+          wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+        }
       }
-      if (gc + CH < g1) load_chunk(gc + CH);
 #pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const int g = gc + i;
-        if (g < g1) {
+      for (int j = 0; j < CH; ++j) {
+        const bool valid = jc + j < GPW;
+        const int g = valid ? w + 4 * (jc + j) : 0;
+        // a clamped (duplicate) tile contributes through a zero scale
+        const float fsa = valid ? half_bits_to_f32(s_sc[g * 16 + r]) : 0.f;
+        const float fsb = valid ? half_bits_to_f32(s_sc[(G + g) * 16 + r]) : 0.f;
+        const float fza = 128.f + (float)((s_zz[g * 8 + (r >> 1)] >> zsh) & 15);
+        const float fzb = 128.f + (float)((s_zz[(G + g) * 8 + (r >> 1)] >> zsh) & 15);
 #pragma unroll
-          for (int t = 0; t < TMAX; ++t) {
-            if (t < mc) {
-              const uint4 *xp = (const uint4 *)(xs + (size_t)t * K + g * 128 + qd * 32);
-              const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
-              const float xq = xsum[t * KS + g * 4 + qd];
-              float dA = dot8_q4(ca[i].x, x0, 0.f);
-              float dB = dot8_q4(cb[i].x, x0, 0.f);
-              dA = dot8_q4(ca[i].y, x1, dA); dB = dot8_q4(cb[i].y, x1, dB);
-              dA = dot8_q4(ca[i].z, x2, dA); dB = dot8_q4(cb[i].z, x2, dB);
-              dA = dot8_q4(ca[i].w, x3, dA); dB = dot8_q4(cb[i].w, x3, dB);
-              accA[t] = fmaf(fsa[i], dA - fza[i] * xq, accA[t]);
-              accB[t] = fmaf(fsb[i], dB - fzb[i] * xq, accB[t]);
-            }
+        for (int t = 0; t < TMAX; ++t) {
+          if (t < mc) {
+            const uint4 *xp = (const uint4 *)(xs + (size_t)t * K + g * 128 + qd * 32);
+            const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+            const float xq = xsum[t * KS + g * 4 + qd];
+            float dA = dot8_q4(wa[j].x, x0, 0.f);
+            float dB = dot8_q4(wb[j].x, x0, 0.f);
+            dA = dot8_q4(wa[j].y, x1, dA); dB = dot8_q4(wb[j].y, x1, dB);
+            dA = dot8_q4(wa[j].z, x2, dA); dB = dot8_q4(wb[j].z, x2, dB);
+            dA = dot8_q4(wa[j].w, x3, dA); dB = dot8_q4(wb[j].w, x3, dB);
+            accA[t] = fmaf(fsa, dA - fza * xq, accA[t]);
+            accB[t] = fmaf(fsb, dB - fzb * xq, accB[t]);
           }
         }
+        // keep the scheduler from hoisting the next tile's LDS reads (register pressure)
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     // reduce the four k-quarters of the wave, then the four waves
@@ -397,26 +458,26 @@ __global__ __launch_bounds__(256) void k_gemv_int4(const GemvArgs a) {
     __syncthreads();
     if (SWIGLU) {
       for (int i = tid; i < mc * 16; i += 256) {
-        const int t = i >> 4, rr = i & 15;
+        const int t = i >> 4, rr2 = i & 15;
         float ga = 0.f, up = 0.f;
 #pragma unroll
         for (int ww = 0; ww < 4; ++ww) {
-          ga += red[((ww * TMAX + t) * 2 + 0) * 16 + rr];
-          up += red[((ww * TMAX + t) * 2 + 1) * 16 + rr];
+          ga += red[((ww * TMAX + t) * 2 + 0) * 16 + rr2];
+          up += red[((ww * TMAX + t) * 2 + 1) * 16 + rr2];
         }
         const float hv = ga / (1.f + expf(-ga)) * up;
-        ((uint16_t *)c.out)[(size_t)(row0 + t0 + t) * c.out_stride + b * 16 + rr] = f32_to_bf16(hv);
+        ((uint16_t *)c.out)[(size_t)(row0 + t0 + t) * c.out_stride + b * 16 + rr2] = f32_to_bf16(hv);
       }
     } else {
       for (int i = tid; i < mc * 32; i += 256) {
-        const int t = i >> 5, ab = (i >> 4) & 1, rr = i & 15;
+        const int t = i >> 5, ab = (i >> 4) & 1, rr2 = i & 15;
         float v = 0.f;
 #pragma unroll
-        for (int ww = 0; ww < 4; ++ww) v += red[((ww * TMAX + t) * 2 + ab) * 16 + rr];
-        ((float *)c.out)[(size_t)(row0 + t0 + t) * c.out_stride + (2 * b + ab) * 16 + rr] = v;
+        for (int ww = 0; ww < 4; ++ww) v += red[((ww * TMAX + t) * 2 + ab) * 16 + rr2];
+        ((float *)c.out)[(size_t)(row0 + t0 + t) * c.out_stride + (2 * b + ab) * 16 + rr2] = v;
       }
     }
-    __syncthreads();
+    if (t0 + TMAX < m) __syncthreads();
   }
 }
 
@@ -523,11 +584,11 @@ extern "C" int moe_dispatch(const int *idx, int T, int k, int E, int *counts, in
   return moe_check_launch("k_dispatch");
 }
 
-template <int TMAX, bool SW>
+template <int TMAX, bool SW, int CH>
 static int launch_gemv(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW>,
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW, CH>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
@@ -536,17 +597,30 @@ static int launch_gemv(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  hipLaunchKernelGGL((k_gemv_int4<TMAX, SW>), dim3(grid), dim3(256), lds, s, a);
+  hipLaunchKernelGGL((k_gemv_int4<TMAX, SW, CH>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4");
 }
 
 static size_t gemv_lds(int tmax, int K) {
-  return (size_t)tmax * K * 2 + (size_t)tmax * (K / 32) * 4 + (size_t)4 * tmax * 2 * 16 * 4;
+  const size_t G = K / 128;
+  return (size_t)tmax * K * 2 + (size_t)tmax * (K / 32) * 4 + 2 * G * 32 + 2 * G * 8 +
+         (size_t)4 * tmax * 2 * 16 * 4;
+}
+
+template <bool SW, int CH>
+static int launch_gemv_c(const GemvArgs &a, int grid, int tmax, size_t lds, hipStream_t s) {
+  switch (tmax) {
+    case 1: return launch_gemv<1, SW, CH>(a, grid, lds, s);
+    case 2: return launch_gemv<2, SW, CH>(a, grid, lds, s);
+    case 4: return launch_gemv<4, SW, CH>(a, grid, lds, s);
+    case 8: return launch_gemv<8, SW, CH>(a, grid, lds, s);
+    default: return launch_gemv<16, SW, CH>(a, grid, lds, s);
+  }
 }
 
 template <bool SW>
-static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, hipStream_t s) {
+static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_routed, hipStream_t s) {
   // rows per pass: the smallest bucket >= T that fits the LDS budget
   int tmax = 1;
   while (tmax < T && tmax < 16) tmax <<= 1;
@@ -556,12 +630,16 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, hipStream
     moe_set_error("k_gemv_int4: K=%d does not fit LDS", Kmax);
     return MOE_EINVAL;
   }
-  switch (tmax) {
-    case 1: return launch_gemv<1, SW>(a, grid, lds, s);
-    case 2: return launch_gemv<2, SW>(a, grid, lds, s);
-    case 4: return launch_gemv<4, SW>(a, grid, lds, s);
-    case 8: return launch_gemv<8, SW>(a, grid, lds, s);
-    default: return launch_gemv<16, SW>(a, grid, lds, s);
+  // tiles in flight per wave and block: the routed class's groups per wave, at most 4
+  // (a partial last chunk re-reads a tile, so pick the chunk that divides best)
+  const int gpw = (G_routed + 3) / 4;
+  int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
+  if (ch < 1) ch = 1;
+  switch (ch) {
+    case 1: return launch_gemv_c<SW, 1>(a, grid, tmax, lds, s);
+    case 2: return launch_gemv_c<SW, 2>(a, grid, tmax, lds, s);
+    case 3: return launch_gemv_c<SW, 3>(a, grid, tmax, lds, s);
+    default: return launch_gemv_c<SW, 4>(a, grid, tmax, lds, s);
   }
 }
 
@@ -569,9 +647,10 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                                        const moe_unit *units, int max_units, const int *sorted_tok,
                                        const uint64_t *expert_ptr, const void *shared_ptr,
                                        void *h_r, void *h_s, float *part_r, float *part_s,
-                                       int *err, void *stream) {
+                                       int *err, const moe_unit *units_host,
+                                       const uint64_t *expert_ptr_host, void *stream) {
   if (!x || T <= 0 || H <= 0 || H % 128 || I < 0 || I % 128 || I_sh < 0 || I_sh % 128 || !err ||
-      (max_units > 0 && (!units || !sorted_tok || !expert_ptr || !h_r || !part_r || I == 0)) ||
+      (max_units > 0 && ((!units && !units_host) || !sorted_tok || (!expert_ptr && !expert_ptr_host) || !h_r || !part_r || I == 0)) ||
       (shared_ptr && (!h_s || !part_s || I_sh == 0))) {
     moe_set_error("moe_experts_decode_int4: bad argument (T=%d H=%d I=%d I_sh=%d)", T, H, I, I_sh);
     return MOE_EINVAL;
@@ -588,26 +667,35 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
   memset(&a, 0, sizeof a);
   a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
   a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err;
+  if (units_host && expert_ptr_host && max_units <= GEMV_MAX_KUNITS) {
+    a.units = nullptr;
+    for (int u = 0; u < max_units; ++u) {
+      const moe_unit &h = units_host[u];
+      a.ku[u].m = h.m; a.ku[u].row0 = h.row0;
+      a.ku[u].base = (h.m > 0 && h.expert >= 0) ? expert_ptr_host[h.expert] : 0;
+    }
+  }
   // pass 1: w13 + SwiGLU
+  // one token: every row reads activation row 0 (stride 0), no gather load on the critical path
   a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z,
-                       H, H / 128, H, I_sh, I_sh / 16};
-  a.cls[1] = GemvClass{(const uint16_t *)x, sorted_tok, h_r, lr.off13_q, lr.off13_s, lr.off13_z,
-                       H, H / 128, H, I, I / 16};
+                       H, H / 128, T == 1 ? 0 : H, I_sh, I_sh / 16, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)x, T == 1 ? nullptr : sorted_tok, h_r, lr.off13_q, lr.off13_s,
+                       lr.off13_z, H, H / 128, T == 1 ? 0 : H, I, I / 16, 0};
   a.n_sh_blocks = sh ? I_sh / 16 : 0;
   int grid = a.n_sh_blocks + max_units * (I / 16);
   if (grid > 0) {
-    int rc = launch_gemv_t<true>(a, grid, T, H, s);
+    int rc = launch_gemv_t<true>(a, grid, T, H, H / 128, s);
     if (rc) return rc;
   }
   // pass 2: w2
   a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z,
-                       I_sh, I_sh / 128, I_sh, H, H / 32};
+                       I_sh, I_sh / 128, I_sh, H, H / 32, 0};
   a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z,
-                       I, I / 128, I, H, H / 32};
+                       I, I / 128, I, H, H / 32, 0};
   a.n_sh_blocks = sh ? H / 32 : 0;
   grid = a.n_sh_blocks + max_units * (H / 32);
   if (grid > 0) {
-    int rc = launch_gemv_t<false>(a, grid, T, I_sh > I ? I_sh : I, s);
+    int rc = launch_gemv_t<false>(a, grid, T, I_sh > I ? I_sh : I, (max_units > 0 ? I : I_sh) / 128, s);
     if (rc) return rc;
   }
   return MOE_OK;

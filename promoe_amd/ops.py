@@ -68,7 +68,7 @@ def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispa
 
 
 def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
-                        H: int, I: int, I_sh: int):
+                        H: int, I: int, I_sh: int, host_units: bool = False):
     """Returns (part_r [P,H] fp32, part_s [T,H] fp32 or None, err int32[1])."""
     T, k = d.T, d.k
     P = T * k
@@ -80,10 +80,14 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
         h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
         part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
     err = torch.zeros(1, dtype=torch.int32, device=dev)
+    uh = th = None
+    if host_units:   # unit list and slot table resolved on the host, sent in the kernel arguments
+        uh = d.units.cpu().contiguous()
+        th = expert_ptr.cpu().contiguous()
     check(lib.moe_experts_decode_int4(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
                                       ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
                                       ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
-                                      ptr(err), cur_stream()), "moe_experts_decode_int4")
+                                      ptr(err), ptr(uh), ptr(th), cur_stream()), "moe_experts_decode_int4")
     return part_r, part_s, err, h_r, h_s
 
 

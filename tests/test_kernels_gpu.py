@@ -79,7 +79,7 @@ def test_dispatch_bit_exact(cuda, T, k, E):
     assert np.all(d.units.cpu().numpy()[n_act:d.max_units, 1] == 0)
 
 
-def run_layer_gpu(layer, x, k, mode, dev, resident=None):
+def run_layer_gpu(layer, x, k, mode, dev, resident=None, host_units=False):
     """gate -> topk -> dispatch -> int4 decode experts -> combine, all on the GPU."""
     from promoe_amd import ops
     H, I, E, I_sh = layer.H, layer.I, layer.E, layer.I_sh
@@ -97,7 +97,7 @@ def run_layer_gpu(layer, x, k, mode, dev, resident=None):
     table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
                           for e in range(E)], dtype=torch.int64, device=dev)
     shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
-    part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh)
+    part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh, host_units=host_units)
     sg = logits[:, E] if layer.shared_gate is not None else None
     y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
     torch.cuda.synchronize()
@@ -121,6 +121,9 @@ def check_layer(layer, T, k, mode, dev, seed=1):
     err = np.abs(got["y"] - ref["out"]).max() / np.abs(ref["out"]).max()
     print(f"  T={T} k={k} mode={mode} max-rel-err={err:.3e}", flush=True)
     assert err <= TOL
+    # units resolved on the host and passed in the kernel arguments: same kernels, same bits
+    got2 = run_layer_gpu(layer, x, k, mode, dev, host_units=True)
+    assert got2["err"] == 0 and np.array_equal(got2["y"], got["y"])
     return err
 
 
