@@ -144,20 +144,29 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   int rc;
   // hook order of the reference (utils/hooks.py:216-223)
   if (layer == 0 && (rc = moe_report_layer_logits(eng, 0, x, 1, T, d.H))) return rc;
-  if (!d.gate_bias) {
-    if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+  const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
+  const size_t route_lds = (size_t)T * d.H * 2 + (size_t)T * ldl * 4 + (size_t)T * k * 4 + (size_t)(18 * E + 64) * 4;
+  if (T <= 16 && E <= 256 && route_lds <= 140 * 1024) {
+    // decode batch: gate + top-k + dispatch in one launch
+    if ((rc = moe_route_decode(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, n_gate_rows, ldl, k, d.route_mode,
+                               s->idx, s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair,
+                               s->sorted_tok, s->units, s->n_active, s->active_ids, max_units, st)))
+      return rc;
   } else {
-    // the bias covers the routed experts only; the shared-gate row (row E) has none
-    if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
-    if (d.shared_gated &&
-        (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+    if (!d.gate_bias) {
+      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+    } else {
+      // the bias covers the routed experts only; the shared-gate row (row E) has none
+      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+      if (d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    }
+    if ((rc = moe_topk(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, st))) return rc;
+    if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
+                           s->units, s->n_active, s->active_ids, max_units, st)))
       return rc;
   }
-  if ((rc = moe_topk(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, st))) return rc;
-  const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
-  if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
-                         s->units, s->n_active, s->active_ids, max_units, st)))
-    return rc;
   // the active expert list comes back to the host
   HIPC(hipMemcpyAsync(s->units_host, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
   HIPC(hipMemcpyAsync(s->n_active_host, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));

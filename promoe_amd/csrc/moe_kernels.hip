@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "moe_kernels.h"
@@ -240,6 +241,200 @@ __global__ __launch_bounds__(DISP_THREADS) void k_dispatch(
 }
 
 // ---------------------------------------------------------------------------
+// k1+k2 fused for decode batches (T <= 16): one workgroup of 16 waves computes the gate
+// logits (same fixed summation order as k_gate_logits, so the same bits), the top-k
+// routing (wave t = token t) and the stable dispatch, with the logits and indices
+// staying in LDS between the phases.  Three launches become one.
+// ---------------------------------------------------------------------------
+#define ROUTE_MAXT 16
+struct RouteArgs {
+  const uint16_t *x, *wg;
+  const float *bias;
+  float *logits;  // [T, ldl]
+  int T, H, E, Erows, ldl, k, mode, nbits, max_units;
+  int *idx; float *w;
+  int *counts, *offsets, *sorted_pair, *pos_of_pair, *sorted_tok;
+  moe_unit *units; int *n_active; long long *active_ids;
+};
+
+__global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
+  extern __shared__ __align__(16) unsigned char rsm[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int T = a.T, H = a.H, E = a.E, k = a.k, P = T * k;
+  uint16_t *xs = (uint16_t *)rsm;                              // [T][H]
+  float *s_lg = (float *)(rsm + (size_t)T * H * 2);            // [T][ldl]
+  int *s_idx = (int *)(s_lg + (size_t)T * a.ldl);              // [P]
+  int *s_cnt = s_idx + ((P + 3) & ~3);                         // [E]
+  int *s_off = s_cnt + E;                                      // [E+1]
+  int *s_ws = s_off + E + 1;                                   // [16][E] per-wave counts
+  int *s_misc = s_ws + 16 * E;                                 // [34]
+
+  // ---- stage x -------------------------------------------------------------------------
+  const int nvec = T * (H >> 3);
+  for (int i = tid; i < nvec; i += 1024) ((uint4 *)xs)[i] = ((const uint4 *)a.x)[i];
+  for (int e = tid; e < E; e += 1024) s_cnt[e] = 0;
+  __syncthreads();
+  // ---- gate logits: wave w takes rows w, w+16, ... --------------------------------------
+  for (int e = w; e < a.Erows; e += 16) {
+    const uint16_t *wr = a.wg + (size_t)e * H;
+    float acc[ROUTE_MAXT];
+#pragma unroll
+    for (int t = 0; t < ROUTE_MAXT; ++t) acc[t] = 0.f;
+    for (int c = 0; c < H; c += 512) {
+      const int kk = c + 8 * lane;
+      if (kk < H) {
+        const uint4 wv = *(const uint4 *)(wr + kk);
+#pragma unroll
+        for (int t = 0; t < ROUTE_MAXT; ++t) {
+          if (t < T) {
+            const uint4 xv = *(const uint4 *)(xs + (size_t)t * H + kk);
+            float v = acc[t];
+            v = fmaf(bf16lo(xv.x), bf16lo(wv.x), v); v = fmaf(bf16hi(xv.x), bf16hi(wv.x), v);
+            v = fmaf(bf16lo(xv.y), bf16lo(wv.y), v); v = fmaf(bf16hi(xv.y), bf16hi(wv.y), v);
+            v = fmaf(bf16lo(xv.z), bf16lo(wv.z), v); v = fmaf(bf16hi(xv.z), bf16hi(wv.z), v);
+            v = fmaf(bf16lo(xv.w), bf16lo(wv.w), v); v = fmaf(bf16hi(xv.w), bf16hi(wv.w), v);
+            acc[t] = v;
+          }
+        }
+      }
+    }
+    const float be = (a.bias && e < E) ? a.bias[e] : 0.f;
+#pragma unroll
+    for (int t = 0; t < ROUTE_MAXT; ++t) {
+      if (t < T) {
+        float v = acc[t];
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
+        if (lane == 0) {
+          const float lg = (a.bias && e < E) ? v + be : v;
+          s_lg[t * a.ldl + e] = lg;
+          a.logits[(size_t)t * a.ldl + e] = lg;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  // ---- top-k: wave t = token t ----------------------------------------------------------
+  if (w < T) {
+    const int t = w;
+    const float NEG = -__builtin_inff();
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int e = lane + 64 * r;
+      v[r] = (e < E) ? s_lg[t * a.ldl + e] : NEG;
+    }
+    float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    float den = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (lane + 64 * r < E) den += expf(v[r] - mx);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
+    float sel_v = 0.f, sum_sel = 0.f;
+    for (int j = 0; j < k; ++j) {
+      float bv = v[0];
+      int bi = lane;
+#pragma unroll
+      for (int r = 1; r < 4; ++r)
+        if (v[r] > bv) { bv = v[r]; bi = lane + 64 * r; }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) {
+        const float ov = __shfl_xor(bv, m, 64);
+        const int oi = __shfl_xor(bi, m, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (bi == lane + 64 * r) v[r] = NEG;
+      if (lane == j) sel_v = bv;
+      if (lane == 0) { a.idx[(size_t)t * k + j] = bi; s_idx[t * k + j] = bi; }
+      sum_sel += expf(bv - mx);
+    }
+    const float ex = expf(sel_v - mx);
+    float wgt;
+    if (a.mode == MOE_ROUTE_TOPK_SOFTMAX) wgt = ex / sum_sel;
+    else {
+      wgt = ex / den;
+      if (a.mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
+    }
+    if (lane < k) a.w[(size_t)t * k + lane] = wgt;
+  }
+  __syncthreads();
+  // ---- dispatch: P <= 1024 pairs, one chunk ----------------------------------------------
+  const int p = tid;
+  const int e_p = p < P ? s_idx[p] : -1;
+  const bool valid = (unsigned)e_p < (unsigned)E;
+  if (valid) atomicAdd(&s_cnt[e_p], 1);
+  __syncthreads();
+  {
+    const int c = (tid < E) ? s_cnt[tid] : 0;
+    const int act = c > 0 ? 1 : 0;
+    int sc = c, sa = act;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int oc = __shfl_up(sc, d, 64), oa = __shfl_up(sa, d, 64);
+      if (lane >= d) { sc += oc; sa += oa; }
+    }
+    if (lane == 63) { s_misc[w] = sc; s_misc[16 + w] = sa; }
+    __syncthreads();
+    int bc = 0, ba = 0;
+    for (int i = 0; i < w; ++i) { bc += s_misc[i]; ba += s_misc[16 + i]; }
+    const int excl = bc + sc - c, uidx = ba + sa - act;
+    if (tid < E) {
+      s_off[tid] = excl;
+      a.counts[tid] = c;
+      a.offsets[tid] = excl;
+      if (act && uidx < a.max_units) {
+        moe_unit uu; uu.expert = tid; uu.m = c; uu.row0 = excl; uu.pad = 0;
+        a.units[uidx] = uu;
+        a.active_ids[uidx] = tid;
+      }
+    }
+    if (tid == 1023) {
+      const int tot_act = ba + sa;
+      a.offsets[E] = bc + sc;
+      *a.n_active = tot_act < a.max_units ? tot_act : a.max_units;
+      s_misc[32] = tot_act;
+    }
+    __syncthreads();
+    for (int uu = s_misc[32] + tid; uu < a.max_units; uu += 1024) {
+      moe_unit z; z.expert = -1; z.m = 0; z.row0 = 0; z.pad = 0;
+      a.units[uu] = z;
+      a.active_ids[uu] = -1;
+    }
+  }
+  for (int i = tid; i < 16 * E; i += 1024) s_ws[i] = 0;
+  __syncthreads();
+  unsigned long long peers = __ballot(valid);
+  for (int bb = 0; bb < a.nbits; ++bb) {
+    const bool bit = (e_p >> bb) & 1;
+    const unsigned long long bal = __ballot(valid && bit);
+    peers &= bit ? bal : ~bal;
+  }
+  const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+  if (valid && rank == 0) s_ws[w * E + e_p] = __popcll(peers);
+  __syncthreads();
+  for (int ee = tid; ee < E; ee += 1024) {
+    int run = 0;
+    for (int ww = 0; ww < 16; ++ww) {
+      const int c = s_ws[ww * E + ee];
+      s_ws[ww * E + ee] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  if (valid) {
+    const int pos = s_off[e_p] + s_ws[w * E + e_p] + rank;
+    a.sorted_pair[pos] = p;
+    a.pos_of_pair[p] = pos;
+    a.sorted_tok[pos] = p / k;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // k3 int4 grouped GEMV (decode).  One workgroup (4 waves) owns two adjacent
 // 16-row blocks of one unit's matrix; wave w takes the K groups w, w+4, w+8, ...
 //   SWIGLU: blocks are (gate rows, up rows) -> out = silu(g)*u, bf16, 16 values
@@ -296,36 +491,67 @@ static __device__ __forceinline__ u32 bload4(rsrc_t r, int voff, int soff) {
   return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
 }
 
-template <int TMAX, bool SWIGLU, int CH>
+// Work item of a GEMV workgroup, resolved from the kernel arguments without dependent
+// loads when the units travel by value: both classes and the first 8 units are fetched
+// in one batch of scalar loads and selected with scalar ops (a dependent second fetch
+// costs ~0.5 us of kernel time at these sizes).
+struct GemvWork {
+  GemvClass c;
+  const unsigned char *base;
+  int m, row0, b;
+};
+template <bool DEVUNITS>
+static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
+  GemvWork wk;
+  const GemvClass c0 = a.cls[0], c1 = a.cls[1];
+  const int n_sh = a.n_sh_blocks;
+  const bool sh = (int)blockIdx.x < n_sh;
+  GemvClass &c = wk.c;
+  c.act = sh ? c0.act : c1.act; c.gather = sh ? c0.gather : c1.gather; c.out = sh ? c0.out : c1.out;
+  c.off_q = sh ? c0.off_q : c1.off_q; c.off_s = sh ? c0.off_s : c1.off_s; c.off_z = sh ? c0.off_z : c1.off_z;
+  c.K = sh ? c0.K : c1.K; c.G = sh ? c0.G : c1.G; c.act_stride = sh ? c0.act_stride : c1.act_stride;
+  c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk; c.pad = 0;
+  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
+  const int u = sh ? 0 : rr / c.nblk;
+  wk.b = rr - u * c.nblk;
+  if (DEVUNITS) {
+    if (sh) {
+      wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
+    } else {
+      const moe_unit ud = a.units[u];
+      wk.m = ud.m; wk.row0 = ud.row0;
+      wk.base = ud.m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
+    }
+  } else {
+    // the first 8 units sit at fixed argument offsets: fetched with the rest, picked by scalar selects
+    unsigned long long ub = a.ku[0].base;
+    int um = a.ku[0].m, ur = a.ku[0].row0;
+#pragma unroll
+    for (int i = 1; i < 8; ++i) {
+      const bool hit = u == i;
+      ub = hit ? a.ku[i].base : ub; um = hit ? a.ku[i].m : um; ur = hit ? a.ku[i].row0 : ur;
+    }
+    if (u >= 8) { ub = a.ku[u].base; um = a.ku[u].m; ur = a.ku[u].row0; }
+    wk.m = sh ? a.T : um; wk.row0 = sh ? 0 : ur;
+    ub = sh ? (unsigned long long)a.shared_base : ub;
+    // uniform by construction; say so, or the buffer resources end up in vector registers
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)ub);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(ub >> 32));
+    wk.base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+  }
+  return wk;
+}
+
+template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS>
 __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  // all kernel arguments are fetched in one batch (both classes, then selected): the
-  // scalar loads do not depend on one another
-  const GemvClass c0 = a.cls[0], c1 = a.cls[1];
-  const int n_sh = a.n_sh_blocks;
-  const bool sh = (int)blockIdx.x < n_sh;
-  GemvClass c;
-  c.act = sh ? c0.act : c1.act; c.gather = sh ? c0.gather : c1.gather; c.out = sh ? c0.out : c1.out;
-  c.off_q = sh ? c0.off_q : c1.off_q; c.off_s = sh ? c0.off_s : c1.off_s; c.off_z = sh ? c0.off_z : c1.off_z;
-  c.K = sh ? c0.K : c1.K; c.G = sh ? c0.G : c1.G; c.act_stride = sh ? c0.act_stride : c1.act_stride;
-  c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk;
-  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
-  const int u = sh ? 0 : rr / c.nblk;
-  const int b = rr - u * c.nblk;
-  int m, row0;
-  const unsigned char *base;
-  if (a.units && !sh) {
-    const moe_unit ud = a.units[u];
-    m = ud.m; row0 = ud.row0;
-    base = m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
-  } else {
-    const KUnit ku = a.ku[u];
-    m = sh ? a.T : ku.m; row0 = sh ? 0 : ku.row0;
-    base = sh ? a.shared_base : (const unsigned char *)ku.base;
-  }
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  const GemvClass &c = wk.c;
+  const int m = wk.m, row0 = wk.row0, b = wk.b;
+  const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
     if (tid == 0) atomicOr(a.err, 1);
@@ -482,6 +708,210 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
 }
 
 // ---------------------------------------------------------------------------
+// k3, matrix-core form: same work split and load section as k_gemv_int4, but the
+// products run on v_mfma_f32_16x16x32_bf16 with the (up to 16) tokens of the unit as
+// the N dimension, so the weight tiles are dequantised once for all tokens.
+//   A (16 rows x 32 k): lane l = row l&15, k-chunk l>>4 -> exactly one dequantised dword
+//   B (32 k x 16 tok) : lane l = token l&15, k-chunk l>>4 -> 16 bytes of that token's row
+//   D (16 x 16)       : lane l holds rows 4(l>>4)+i, token l&15
+// Per tile (one quantisation group): D_g = sum (128+q) x ; acc += s_row (D_g - (128+z_row) X_tok,g).
+// ---------------------------------------------------------------------------
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+static __device__ __forceinline__ bf16x8_t deq8_bf16(u32 w) {
+  const u32 M = 0x000f000fu, C = 0x43004300u;
+  u32x4_t v;
+  v.x = (w & M) | C; v.y = ((w >> 4) & M) | C; v.z = ((w >> 8) & M) | C; v.w = ((w >> 12) & M) | C;
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+static __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &x) {
+  u32x4_t v; v.x = x.x; v.y = x.y; v.z = x.z; v.w = x.w;
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+
+template <bool SWIGLU, int CH, bool DEVUNITS>
+__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, qd = lane >> 4;
+
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  const GemvClass &c = wk.c;
+  const int m = wk.m, row0 = wk.row0;
+  const unsigned char *base = wk.base;
+  if (m <= 0) return;
+  if (base == nullptr) {
+    if (tid == 0) atomicOr(a.err, 1);
+    return;
+  }
+  const int K = c.K, G = c.G;
+  const int XS = K * 2 + 16;  // padded row stride (bytes): 16 token rows hit 16 distinct bank quads
+  unsigned char *xs = smem;                                           // [TB][XS]
+  float *xsum = (float *)(smem + (size_t)TB * XS);                    // [TB][G]
+  uint16_t *s_sc = (uint16_t *)(xsum + (((size_t)TB * G + 3) & ~(size_t)3));  // [2][G][16] fp16, 16-B aligned
+  unsigned char *s_zz = (unsigned char *)(s_sc + 2 * G * 16);         // [2][G][8]
+  float *red = (float *)(s_zz + 2 * G * 8);                           // [4][2][16 rows][16 tok]
+
+  const int GPW = (G - w + 3) >> 2;
+  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
+  const int vec_per_row = K >> 3;
+  const int n_sc = 2 * G * 8, n_zz = 2 * G * 2;
+
+  for (int t0 = 0; t0 < m; t0 += TB) {
+    const int mc = (m - t0) < TB ? (m - t0) : TB;
+   // RPW consecutive (gate,up) / (row,row) block pairs per workgroup: the activations are
+   // staged once and the fixed per-workgroup cost is spread over more weight tiles
+   for (int pp = 0; pp < RPW; ++pp) {
+    const int b = wk.b * RPW + pp;
+    const int rbA = 2 * b;
+    const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, 2u * G * 1024u);
+    const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, 2u * G * 32u);
+    const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, 2u * G * 8u);
+    // ---- straight-line load section ------------------------------------------------------
+    const int row_first = row0 + t0;
+    const int arow0 = c.gather ? c.gather[row_first] : row_first;
+    const uint4 xv0 = bload16(rx, (tid < vec_per_row ? tid : 0) * 16, arow0 * c.act_stride * 2);
+    const u32 msc0 = bload4(rs, tid * 4, 0), msc1 = bload4(rs, tid * 4, 1024);
+    const u32 mzz = bload4(rz, tid * 4, 0);
+    uint4 wa[CH], wb[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int g = j < GPW ? w + 4 * j : 0;
+      wa[j] = bload16(rq, lane * 16, g * 1024);
+      wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+    }
+    // ---- stage x rows (+ per-group sums over 128 values = 16 consecutive vectors) ----------
+    if (pp == 0) {
+      float ps = sum8_bf16(xv0);
+      ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
+      if (tid < vec_per_row) {
+        *(uint4 *)(xs + (size_t)tid * 16) = xv0;
+        if ((tid & 15) == 0) xsum[tid >> 4] = ps;
+      }
+    }
+    if (tid < n_sc) ((u32 *)s_sc)[tid] = msc0;
+    if (tid + 256 < n_sc) ((u32 *)s_sc)[tid + 256] = msc1;
+    if (tid < n_zz) ((u32 *)s_zz)[tid] = mzz;
+    // remaining (row, 256-vector chunk) pieces, four loads in flight at a time; piece 0 is
+    // the early load above
+    if (pp == 0) {
+      const int cpr = (vec_per_row + 255) >> 8;  // chunks per row
+      const int total = mc * cpr;
+      // row index of every token of this pass, one per lane (lanes >= mc repeat the last)
+      const int grow = row_first + (lane < mc ? lane : mc - 1);
+      const int arow_l = c.gather ? c.gather[grow] : grow;
+      for (int pb = 1; pb < total; pb += 4) {
+        uint4 xb[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int pi = pb + q < total ? pb + q : 0;
+          const int t = pi / cpr, ch = pi - t * cpr;
+          const int v = tid + 256 * ch;
+          const int arow = __builtin_amdgcn_readlane(arow_l, t);
+          xb[q] = bload16(rx, (v < vec_per_row ? v : 0) * 16, arow * c.act_stride * 2);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int pi = pb + q;
+          const int t = pi / cpr, ch = pi - t * cpr;
+          const int v = tid + 256 * ch;
+          float ps = sum8_bf16(xb[q]);
+          ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
+          ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
+          if (pi < total && v < vec_per_row) {
+            *(uint4 *)(xs + (size_t)t * XS + (size_t)v * 16) = xb[q];
+            if ((tid & 15) == 0) xsum[t * G + (v >> 4)] = ps;
+          }
+        }
+      }
+    }
+    for (int i = tid + 512; i < n_sc; i += 256) ((u32 *)s_sc)[i] = bload4(rs, i * 4, 0);
+    for (int i = tid + 256; i < n_zz; i += 256) ((u32 *)s_zz)[i] = bload4(rz, i * 4, 0);
+    __syncthreads();
+
+    f32x4_t accA = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+    const int tok = r < mc ? r : mc - 1;  // lanes past the last token repeat it (ignored later)
+    const unsigned char *xrow = xs + (size_t)tok * XS + qd * 64;
+
+    for (int jc = 0; jc < GPW; jc += CH) {
+      if (jc > 0) {
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+          const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
+          wa[j] = bload16(rq, lane * 16, g * 1024);
+          wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const bool valid = jc + j < GPW;
+        const int g = valid ? w + 4 * (jc + j) : 0;
+        const uint4 *xp = (const uint4 *)(xrow + g * 256);
+        const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+        const float xg = xsum[tok * G + g];
+        // scales / zeros of the 4 rows this lane owns in D: rows 4qd..4qd+3
+        const uint2 sA = *(const uint2 *)(s_sc + g * 16 + 4 * qd);
+        const uint2 sB = *(const uint2 *)(s_sc + (G + g) * 16 + 4 * qd);
+        const u32 zA = *(const uint16_t *)(s_zz + g * 8 + 2 * qd);
+        const u32 zB = *(const uint16_t *)(s_zz + (G + g) * 8 + 2 * qd);
+        f32x4_t dA = {0.f, 0.f, 0.f, 0.f}, dB = {0.f, 0.f, 0.f, 0.f};
+        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].x), as_bf16x8(x0), dA, 0, 0, 0);
+        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].x), as_bf16x8(x0), dB, 0, 0, 0);
+        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].y), as_bf16x8(x1), dA, 0, 0, 0);
+        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].y), as_bf16x8(x1), dB, 0, 0, 0);
+        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].z), as_bf16x8(x2), dA, 0, 0, 0);
+        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].z), as_bf16x8(x2), dB, 0, 0, 0);
+        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].w), as_bf16x8(x3), dA, 0, 0, 0);
+        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].w), as_bf16x8(x3), dB, 0, 0, 0);
+        const float vs = valid ? 1.f : 0.f;  // a clamped (duplicate) tile contributes nothing
+        const u32 sAw[2] = {sA.x, sA.y}, sBw[2] = {sB.x, sB.y};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float fsa = vs * half_bits_to_f32((uint16_t)(sAw[i >> 1] >> (16 * (i & 1))));
+          const float fsb = vs * half_bits_to_f32((uint16_t)(sBw[i >> 1] >> (16 * (i & 1))));
+          const float fza = 128.f + (float)((zA >> (4 * i)) & 15);
+          const float fzb = 128.f + (float)((zB >> (4 * i)) & 15);
+          accA[i] = fmaf(fsa, dA[i] - fza * xg, accA[i]);
+          accB[i] = fmaf(fsb, dB[i] - fzb * xg, accB[i]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // cross-wave reduction: red[w][ab][row][tok]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      red[((w * 2 + 0) * 16 + 4 * qd + i) * 16 + r] = accA[i];
+      red[((w * 2 + 1) * 16 + 4 * qd + i) * 16 + r] = accB[i];
+    }
+    __syncthreads();
+    {
+      const int row = tid >> 4, t = tid & 15;  // 256 threads = 16 rows x 16 tokens
+      float va = 0.f, vb = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        va += red[((ww * 2 + 0) * 16 + row) * 16 + t];
+        vb += red[((ww * 2 + 1) * 16 + row) * 16 + t];
+      }
+      if (t < mc) {
+        if (SWIGLU) {
+          const float hv = va / (1.f + expf(-va)) * vb;
+          ((uint16_t *)c.out)[(size_t)(row_first + t) * c.out_stride + b * 16 + row] = f32_to_bf16(hv);
+        } else {
+          float *o = (float *)c.out + (size_t)(row_first + t) * c.out_stride + 2 * b * 16 + row;
+          o[0] = va;
+          o[16] = vb;
+        }
+      }
+    }
+    if (pp + 1 < RPW) __syncthreads();
+   }
+    if (t0 + TB < m) __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
 // k5 combine
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_r,
@@ -588,8 +1018,11 @@ template <int TMAX, bool SW, int CH>
 static int launch_gemv(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW, CH>,
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW, CH, true>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW, CH, false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
       return MOE_EHIP;
@@ -597,7 +1030,8 @@ static int launch_gemv(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  hipLaunchKernelGGL((k_gemv_int4<TMAX, SW, CH>), dim3(grid), dim3(256), lds, s, a);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4<TMAX, SW, CH, true>), dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL((k_gemv_int4<TMAX, SW, CH, false>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4");
 }
@@ -619,8 +1053,73 @@ static int launch_gemv_c(const GemvArgs &a, int grid, int tmax, size_t lds, hipS
   }
 }
 
+static size_t gemv_mfma_lds(int tb, int K) {
+  const size_t G = K / 128;
+  return (size_t)tb * (K * 2 + 16) + (((size_t)tb * G + 3) & ~(size_t)3) * 4 + 2 * G * 32 + 2 * G * 8 +
+         (size_t)4 * 2 * 256 * 4;
+}
+
+template <bool SW, int CH>
+static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t lds, hipStream_t s) {
+  // block pairs per workgroup: enough workgroups to fill the chip twice, then fewer, larger ones
+  GemvArgs a = a_in;
+  int rpw = 1;
+  while (rpw < 4 && grid_in / (rpw * 2) >= 1024 && a.cls[1].nblk % (rpw * 2) == 0 &&
+         (a.n_sh_blocks == 0 || (a.cls[0].nblk % (rpw * 2) == 0)))
+    rpw *= 2;
+  a.cls[0].nblk /= rpw; a.cls[1].nblk /= rpw; a.n_sh_blocks /= rpw;
+  const int grid = grid_in / rpw;
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma<SW, CH, true>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma<SW, CH, false>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
+      return MOE_EHIP;
+    }
+    attr_set = true;
+  }
+  moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, true>), dim3(grid), dim3(256), lds, s, a, tb, rpw);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, false>), dim3(grid), dim3(256), lds, s, a, tb, rpw);
+  moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
+  return moe_check_launch("k_gemv_int4_mfma");
+}
+
+// 0: dot2 GEMV for T == 1, matrix-core form otherwise (default); 1: always dot2; 2: always MFMA
+static int gemv_mode() {
+  static int mode = -1;
+  if (mode < 0) {
+    const char *e = getenv("MOE_DECODE_GEMV");
+    mode = e ? atoi(e) : 0;
+  }
+  return mode;
+}
+
 template <bool SW>
 static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_routed, hipStream_t s) {
+  // tiles in flight per wave and block: the routed class's groups per wave, at most 4
+  // (a partial last chunk re-reads a tile, so pick the chunk that divides best)
+  const int gpw = (G_routed + 3) / 4;
+  int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
+  if (ch < 1) ch = 1;
+  const int mode = gemv_mode();
+  if (mode == 2 || (mode == 0 && T > 1)) {
+    int tb = 1;
+    while (tb < T && tb < 16) tb <<= 1;
+    while (tb > 1 && gemv_mfma_lds(tb, Kmax) > 150 * 1024) tb >>= 1;
+    const size_t lds = gemv_mfma_lds(tb, Kmax);
+    if (lds > 150 * 1024) { moe_set_error("k_gemv_int4_mfma: K=%d does not fit LDS", Kmax); return MOE_EINVAL; }
+    switch (ch) {
+      case 1: return launch_gemv_mfma<SW, 1>(a, grid, tb, lds, s);
+      case 2: return launch_gemv_mfma<SW, 2>(a, grid, tb, lds, s);
+      case 3: return launch_gemv_mfma<SW, 3>(a, grid, tb, lds, s);
+      default: return launch_gemv_mfma<SW, 4>(a, grid, tb, lds, s);
+    }
+  }
   // rows per pass: the smallest bucket >= T that fits the LDS budget
   int tmax = 1;
   while (tmax < T && tmax < 16) tmax <<= 1;
@@ -630,11 +1129,6 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
     moe_set_error("k_gemv_int4: K=%d does not fit LDS", Kmax);
     return MOE_EINVAL;
   }
-  // tiles in flight per wave and block: the routed class's groups per wave, at most 4
-  // (a partial last chunk re-reads a tile, so pick the chunk that divides best)
-  const int gpw = (G_routed + 3) / 4;
-  int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
-  if (ch < 1) ch = 1;
   switch (ch) {
     case 1: return launch_gemv_c<SW, 1>(a, grid, tmax, lds, s);
     case 2: return launch_gemv_c<SW, 2>(a, grid, tmax, lds, s);
@@ -699,6 +1193,47 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
     if (rc) return rc;
   }
   return MOE_OK;
+}
+
+extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias, float *logits,
+                                int T, int H, int E, int E_rows, int ldl, int k, int mode, int *idx,
+                                float *w, int *counts, int *offsets, int *sorted_pair,
+                                int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
+                                int64_t *active_ids, int max_units, void *stream) {
+  if (!x || !wg || !logits || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair ||
+      !sorted_tok || !units || !n_active || !active_ids || T <= 0 || T > ROUTE_MAXT || H <= 0 || H % 8 ||
+      E <= 0 || E > 256 || E_rows < E || E_rows > E + 1 || ldl < E_rows || k <= 0 || k > 32 || k > E ||
+      mode < 0 || mode > 2 || max_units < 0) {
+    moe_set_error("moe_route_decode: bad argument (T=%d H=%d E=%d k=%d)", T, H, E, k);
+    return MOE_EINVAL;
+  }
+  const int P = T * k;
+  const size_t lds = (size_t)T * H * 2 + (size_t)T * ldl * 4 + (size_t)((P + 3) & ~3) * 4 +
+                     (size_t)(E + E + 1 + 16 * E + 34) * 4;
+  if (lds > 150 * 1024) {
+    moe_set_error("moe_route_decode: T=%d H=%d does not fit LDS; use the separate kernels", T, H);
+    return MOE_EINVAL;
+  }
+  static bool attr_set = false;
+  if (lds > 48 * 1024 && !attr_set) {
+    if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_route_decode,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                               "hipFuncSetAttribute(k_route_decode)"))
+      return rc;
+    attr_set = true;
+  }
+  RouteArgs a;
+  a.x = (const uint16_t *)x; a.wg = (const uint16_t *)wg; a.bias = bias; a.logits = logits;
+  a.T = T; a.H = H; a.E = E; a.Erows = E_rows; a.ldl = ldl; a.k = k; a.mode = mode;
+  a.nbits = 0;
+  while ((1 << a.nbits) < E) ++a.nbits;
+  a.max_units = max_units; a.idx = idx; a.w = w; a.counts = counts; a.offsets = offsets;
+  a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
+  a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
+  moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
+  hipLaunchKernelGGL(k_route_decode, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
+  moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
+  return moe_check_launch("k_route_decode");
 }
 
 extern "C" int moe_combine(const float *part_r, const float *part_s, const float *topk_w,

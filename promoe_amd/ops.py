@@ -67,6 +67,21 @@ def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispa
     return d
 
 
+def route_decode(x, wg, bias, E: int, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
+    """Fused gate logits + top-k + dispatch for T <= 16.  wg may carry one extra row (shared gate)."""
+    T, H = x.shape
+    rows = wg.shape[0]
+    logits = torch.empty(T, rows, dtype=torch.float32, device=x.device)
+    idx = torch.empty(T, k, dtype=torch.int32, device=x.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=x.device)
+    d = Dispatch(T, k, E, min(E, T * k), x.device)
+    check(lib.moe_route_decode(ptr(_dev(x)), ptr(_dev(wg)), ptr(bias), ptr(logits), T, H, E, rows, rows, k, mode,
+                               ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets), ptr(d.sorted_pair),
+                               ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units), ptr(d.n_active),
+                               ptr(d.active_ids), d.max_units, cur_stream()), "moe_route_decode")
+    return logits, idx, w, d
+
+
 def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
                         H: int, I: int, I_sh: int, host_units: bool = False):
     """Returns (part_r [P,H] fp32, part_s [T,H] fp32 or None, err int32[1])."""

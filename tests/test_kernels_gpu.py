@@ -158,3 +158,26 @@ def test_non_resident_expert_is_reported(cuda):
     x = O.synth_acts(2, 256)
     got = run_layer_gpu(layer, x, 2, 0, cuda, resident=set())
     assert got["err"] == 1
+
+
+@pytest.mark.parametrize("T,H,E,k,mode,extra", [(1, 2048, 64, 6, 0, 0), (4, 2048, 64, 6, 0, 1), (16, 2048, 64, 6, 1, 0),
+                                               (3, 4096, 8, 2, 2, 0), (16, 3584, 64, 8, 0, 1), (7, 256, 60, 4, 0, 0)])
+def test_fused_route_equals_separate_kernels(cuda, T, H, E, k, mode, extra):
+    from promoe_amd import ops
+    print(f"case route_decode T={T} H={H} E={E} k={k} mode={mode} extra={extra}", flush=True)
+    x = bf16_dev(O.synth_acts(T, H, seed=5), cuda)
+    wg = bf16_dev(O.round_bf16(O.synth_weights((E + extra, H), seed=6)), cuda)
+    bias = torch.from_numpy(O.zipf_gate_bias(E, 1.2)).to(cuda)
+    lg, idx, w, d = ops.route_decode(x, wg, bias, E, k, mode)
+    lg_ref = ops.gate_logits(x, wg[:E].contiguous(), bias)
+    idx_ref, w_ref = ops.topk(lg_ref, k, mode)
+    d_ref = ops.dispatch(idx_ref, E)
+    assert torch.equal(lg[:, :E], lg_ref) and torch.equal(idx, idx_ref) and torch.equal(w, w_ref)
+    if extra:
+        assert torch.equal(lg[:, E:], ops.gate_logits(x, wg[E:].contiguous()))
+    P = T * k
+    for name in ("counts", "offsets", "n_active"):
+        assert torch.equal(getattr(d, name), getattr(d_ref, name)), name
+    for name in ("sorted_pair", "pos_of_pair", "sorted_tok"):
+        assert torch.equal(getattr(d, name)[:P], getattr(d_ref, name)[:P]), name
+    assert torch.equal(d.units, d_ref.units) and torch.equal(d.active_ids, d_ref.active_ids)
