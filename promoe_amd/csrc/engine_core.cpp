@@ -352,6 +352,7 @@ static int cache_miss(moe_engine *eng, Expert *in, bool precise, Expert **victim
     v->status = kIdle;  // a partially fetched expert
   }
   ENG_CHECK(eng, v->slot == slot, "slot bookkeeping mismatch");
+  if (v->num_ready == eng->cfg.num_per_expert_param) eng->layer_complete[v->layer]--;
   v->num_ready = 0;
   if (*victim_wait == nullptr) {
     set_table(eng, v, false);
@@ -494,6 +495,7 @@ static int fetch_done(moe_engine *eng) {
     ENG_CHECK(eng, e->status.load() == kFetching, "fetch done for an expert in state %d", e->status.load());
     e->status = eng->current.precise ? kLaunching : kReady;
     set_table(eng, e, true);
+    eng->layer_complete[e->layer]++;
   }
   eng->current.e = nullptr;
   return 0;
@@ -597,6 +599,7 @@ extern "C" int moe_engine_create(const moe_cfg *cfg, int backend, void *compute_
   eng->layer_q.resize(L);
   eng->table_dirty.assign(L, 0);
   eng->layer_event.assign(L, nullptr);
+  eng->layer_complete.assign(L, 0);
   eng->budget = cfg->max_prefetch_layer_distance;
   eng->layer_desc.resize(L);
   for (auto &d : eng->layer_desc) memset(&d, 0, sizeof d);
@@ -1093,8 +1096,22 @@ extern "C" int moe_streams(moe_engine *eng, void **compute, void **copy) {
   return MOE_OK;
 }
 
+int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n) {
+  std::lock_guard<std::mutex> lk(eng->mu);
+  for (int i = 0; i < n; ++i) {
+    if (units[i].expert < 0 || units[i].expert >= eng->cfg.num_expert) continue;
+    Expert *e = eng->ex(layer, units[i].expert);
+    if (!in_cache(eng, e)) continue;
+    if (int rc = cache_hit(eng, e, true)) return rc;
+    eng->ctr.ready++;
+    eng->ctr.activated++;
+  }
+  return MOE_OK;
+}
+
 extern "C" int moe_get_counters(moe_engine *eng, moe_counters *out) {
   if (!eng || !out) { moe_set_error("moe_get_counters: null"); return MOE_EINVAL; }
+  if (eng->fw) moe_forward_harvest(eng, true);
   std::lock_guard<std::mutex> lk(eng->mu);
   *out = eng->ctr;
   return MOE_OK;

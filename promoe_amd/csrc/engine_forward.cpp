@@ -6,6 +6,7 @@
 // resident go out as ONE grouped launch, missed experts follow one by one as their
 // copies land (the returned order of report_one_layer), then combine.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "engine_internal.h"
@@ -25,6 +26,11 @@ struct LayerState {
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
   int sub_cursor = 0;
+  // routing results of calls that ran without a host round trip, accounted later
+  struct Pending { int layer = -1, max_units = 0; hipEvent_t ev = nullptr; moe_unit *units = nullptr; int *n_active = nullptr; bool busy = false; };
+  static const int kPending = 8;
+  Pending pend[kPending];
+  int pend_head = 0;
 };
 
 void moe_forward_free(LayerState *s) {
@@ -32,6 +38,7 @@ void moe_forward_free(LayerState *s) {
   for (auto p : s->dev_allocs) (void)hipFree(p);
   for (auto p : s->host_allocs) (void)hipHostFree(p);
   if (s->ev) (void)hipEventDestroy(s->ev);
+  for (auto &p : s->pend) if (p.ev) (void)hipEventDestroy(p.ev);
   delete s;
 }
 
@@ -112,9 +119,29 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
   rc |= halloc(s, &s->n_active_host, 1);
   rc |= halloc(s, &s->err_host, 1);
+  for (auto &p : s->pend) {
+    rc |= halloc(s, &p.units, s->max_units);
+    rc |= halloc(s, &p.n_active, 1);
+    if (hipEventCreateWithFlags(&p.ev, hipEventDisableTiming) != hipSuccess) rc = 1;
+  }
   if (rc) return MOE_EHIP;
   HIPC(hipMemset(s->err, 0, sizeof(int)));
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
+  return MOE_OK;
+}
+
+int moe_forward_harvest(moe_engine *eng, bool wait) {
+  LayerState *s = eng->fw;
+  if (!s) return MOE_OK;
+  for (int i = 0; i < LayerState::kPending; ++i) {
+    LayerState::Pending &p = s->pend[(s->pend_head + i) % LayerState::kPending];  // oldest first
+    if (!p.busy) continue;
+    if (wait) { if (hipEventSynchronize(p.ev) != hipSuccess) return MOE_EHIP; }
+    else if (hipEventQuery(p.ev) != hipSuccess) { (void)hipGetLastError(); break; }
+    const int n = std::min(*p.n_active, p.max_units);
+    if (int rc = engine_account_hits(eng, p.layer, p.units, n)) return rc;
+    p.busy = false;
+  }
   return MOE_OK;
 }
 
@@ -146,7 +173,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   if (layer == 0 && (rc = moe_report_layer_logits(eng, 0, x, 1, T, d.H))) return rc;
   const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
   const size_t route_lds = (size_t)T * d.H * 2 + (size_t)T * ldl * 4 + (size_t)T * k * 4 + (size_t)(18 * E + 64) * 4;
-  if (T <= 16 && E <= 256 && route_lds <= 140 * 1024) {
+  static const bool fused_route = getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) != 0;
+  if (fused_route && T <= 16 && E <= 256 && route_lds <= 140 * 1024) {
     // decode batch: gate + top-k + dispatch in one launch
     if ((rc = moe_route_decode(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, n_gate_rows, ldl, k, d.route_mode,
                                s->idx, s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair,
@@ -166,6 +194,37 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
                            s->units, s->n_active, s->active_ids, max_units, st)))
       return rc;
+  }
+  if ((rc = moe_forward_harvest(eng, false))) return rc;
+  // Every expert of the layer resident, and the layer's slot group can hold them all: there
+  // is nothing for the host to decide, so no round trip.  The kernels take the device-built
+  // unit list; the routing comes back asynchronously and the hits are accounted when it lands.
+  bool all_resident = false;
+  {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
+                   eng->layer_complete[layer] == E;
+  }
+  if (all_resident) {
+    LayerState::Pending &p = s->pend[s->pend_head];
+    if (p.busy && (rc = moe_forward_harvest(eng, true))) return rc;
+    s->pend_head = (s->pend_head + 1) % LayerState::kPending;
+    HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
+    HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
+    HIPC(hipEventRecord(p.ev, st));
+    p.layer = layer; p.max_units = max_units; p.busy = true;
+    const uint64_t *table = nullptr;
+    if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    if ((rc = moe_experts_decode_int4(x, T, d.H, d.I, d.I_sh, k, s->units, max_units, s->sorted_tok, table,
+                                      d.I_sh > 0 ? d.shared : nullptr, s->h_r, s->h_s, s->part_r, s->part_s, s->err,
+                                      nullptr, nullptr, st)))
+      return rc;
+    const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
+    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
+      return rc;
+    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    return moe_layer_done(eng, layer);
   }
   // the active expert list comes back to the host
   HIPC(hipMemcpyAsync(s->units_host, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));

@@ -176,6 +176,7 @@ struct moe_engine {
   std::vector<char> table_dirty;  // per layer
   std::vector<void *> dummy_bufs;
   std::vector<void *> layer_event;  // one per layer, used by moe_release_layer
+  std::vector<int> layer_complete;  // fully fetched resident experts per layer
 
   // NN / MIN policy state (cache.hpp:262-266)
   std::vector<float> priority;  // [L*E]
@@ -211,3 +212,7 @@ struct moe_engine {
 
 int engine_fail(moe_engine *eng, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void moe_forward_free(LayerState *);
+// account demand hits of experts that were launched without a host round trip
+int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);
+// collect the routing results of earlier moe_forward calls (wait: block until all are in)
+int moe_forward_harvest(moe_engine *eng, bool wait);

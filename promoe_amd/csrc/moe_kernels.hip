@@ -257,6 +257,7 @@ struct RouteArgs {
   moe_unit *units; int *n_active; long long *active_ids;
 };
 
+template <int TR>
 __global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
   extern __shared__ __align__(16) unsigned char rsm[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -269,46 +270,75 @@ __global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
   int *s_ws = s_off + E + 1;                                   // [16][E] per-wave counts
   int *s_misc = s_ws + 16 * E;                                 // [34]
 
-  // ---- stage x -------------------------------------------------------------------------
+  // ---- gate logits: wave w takes rows w, w+16, ...; the (row, 512-wide chunk) pieces of the
+  // gate matrix are fetched 16 at a time, the first batch before x is staged -------------------
+  const int chunks = (H + 511) >> 9;
+  const int nrows_w = (a.Erows - w + 15) >> 4;
+  const int npieces = nrows_w * chunks;
+  constexpr int NB = 8;
+  uint4 wv[NB];
+  auto load_batch = [&](int pb) {
+#pragma unroll
+    for (int q = 0; q < NB; ++q) {
+      int pi = pb + q;
+      pi = pi < npieces ? pi : (npieces > 0 ? npieces - 1 : 0);
+      const int ri = pi / chunks, ch = pi - ri * chunks;
+      int e = w + 16 * ri;
+      e = e < a.Erows ? e : 0;
+      const int kk = ch * 512 + 8 * lane;
+      wv[q] = *(const uint4 *)(a.wg + (size_t)e * H + (kk < H ? kk : 0));
+    }
+  };
+  load_batch(0);
   const int nvec = T * (H >> 3);
   for (int i = tid; i < nvec; i += 1024) ((uint4 *)xs)[i] = ((const uint4 *)a.x)[i];
   for (int e = tid; e < E; e += 1024) s_cnt[e] = 0;
   __syncthreads();
-  // ---- gate logits: wave w takes rows w, w+16, ... --------------------------------------
-  for (int e = w; e < a.Erows; e += 16) {
-    const uint16_t *wr = a.wg + (size_t)e * H;
-    float acc[ROUTE_MAXT];
+  {
+    float acc[TR];
 #pragma unroll
-    for (int t = 0; t < ROUTE_MAXT; ++t) acc[t] = 0.f;
-    for (int c = 0; c < H; c += 512) {
-      const int kk = c + 8 * lane;
-      if (kk < H) {
-        const uint4 wv = *(const uint4 *)(wr + kk);
+    for (int t = 0; t < TR; ++t) acc[t] = 0.f;
+    for (int pb = 0; pb < npieces; pb += NB) {
+      if (pb > 0) load_batch(pb);
 #pragma unroll
-        for (int t = 0; t < ROUTE_MAXT; ++t) {
-          if (t < T) {
-            const uint4 xv = *(const uint4 *)(xs + (size_t)t * H + kk);
-            float v = acc[t];
-            v = fmaf(bf16lo(xv.x), bf16lo(wv.x), v); v = fmaf(bf16hi(xv.x), bf16hi(wv.x), v);
-            v = fmaf(bf16lo(xv.y), bf16lo(wv.y), v); v = fmaf(bf16hi(xv.y), bf16hi(wv.y), v);
-            v = fmaf(bf16lo(xv.z), bf16lo(wv.z), v); v = fmaf(bf16hi(xv.z), bf16hi(wv.z), v);
-            v = fmaf(bf16lo(xv.w), bf16lo(wv.w), v); v = fmaf(bf16hi(xv.w), bf16hi(wv.w), v);
-            acc[t] = v;
+      for (int q = 0; q < NB; ++q) {
+        const int pi = pb + q;
+        if (pi < npieces) {
+          const int ri = pi / chunks, ch = pi - ri * chunks;
+          const int e = w + 16 * ri;
+          const int kk = ch * 512 + 8 * lane;
+          if (kk < H) {
+#pragma unroll
+            for (int t = 0; t < TR; ++t) {
+              if (t < T) {
+                const uint4 xv = *(const uint4 *)(xs + (size_t)t * H + kk);
+                float v = acc[t];
+                v = fmaf(bf16lo(xv.x), bf16lo(wv[q].x), v); v = fmaf(bf16hi(xv.x), bf16hi(wv[q].x), v);
+                v = fmaf(bf16lo(xv.y), bf16lo(wv[q].y), v); v = fmaf(bf16hi(xv.y), bf16hi(wv[q].y), v);
+                v = fmaf(bf16lo(xv.z), bf16lo(wv[q].z), v); v = fmaf(bf16hi(xv.z), bf16hi(wv[q].z), v);
+                v = fmaf(bf16lo(xv.w), bf16lo(wv[q].w), v); v = fmaf(bf16hi(xv.w), bf16hi(wv[q].w), v);
+                acc[t] = v;
+              }
+            }
           }
-        }
-      }
-    }
-    const float be = (a.bias && e < E) ? a.bias[e] : 0.f;
+          if (ch == chunks - 1) {  // row complete: butterfly, bias, store, reset
+            const bool biased = a.bias && e < E;
+            const float be = biased ? a.bias[e] : 0.f;
 #pragma unroll
-    for (int t = 0; t < ROUTE_MAXT; ++t) {
-      if (t < T) {
-        float v = acc[t];
+            for (int t = 0; t < TR; ++t) {
+              if (t < T) {
+                float v = acc[t];
 #pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
-        if (lane == 0) {
-          const float lg = (a.bias && e < E) ? v + be : v;
-          s_lg[t * a.ldl + e] = lg;
-          a.logits[(size_t)t * a.ldl + e] = lg;
+                for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
+                if (lane == 0) {
+                  const float lg = biased ? v + be : v;
+                  s_lg[t * a.ldl + e] = lg;
+                  a.logits[(size_t)t * a.ldl + e] = lg;
+                }
+              }
+              acc[t] = 0.f;
+            }
+          }
         }
       }
     }
@@ -1216,9 +1246,10 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
   }
   static bool attr_set = false;
   if (lds > 48 * 1024 && !attr_set) {
-    if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_route_decode,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                               "hipFuncSetAttribute(k_route_decode)"))
+    hipError_t e1 = hipFuncSetAttribute((const void *)k_route_decode<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e2 = hipFuncSetAttribute((const void *)k_route_decode<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t e3 = hipFuncSetAttribute((const void *)k_route_decode<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (int rc = moe_check_hip(e1 != hipSuccess ? e1 : (e2 != hipSuccess ? e2 : e3), "hipFuncSetAttribute(k_route_decode)"))
       return rc;
     attr_set = true;
   }
@@ -1231,7 +1262,9 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
   a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
   a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
-  hipLaunchKernelGGL(k_route_decode, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
+  if (T == 1) hipLaunchKernelGGL(k_route_decode<1>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
+  else if (T <= 4) hipLaunchKernelGGL(k_route_decode<4>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(k_route_decode<16>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
   moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
   return moe_check_launch("k_route_decode");
 }

@@ -104,6 +104,21 @@ def test_forward_all_resident_has_no_misses_after_warmup(cuda):
             assert np.abs(y.float().cpu().numpy() - ref["out"]).max() <= TOL * np.abs(ref["out"]).max()
     c = pm.counters()
     assert c["miss"] <= 8 and c["evictions"] == 0
+    # with every expert in its slot the forward runs without a host round trip; results and
+    # the (lazily accounted) hit counters must not change character
+    pm.acquire_layer(0, np.arange(8, dtype=np.int64))
+    pm.release_layer(0)
+    c0 = pm.counters()
+    n_act = 0
+    for T in (1, 5, 16, 2):
+        x = O.synth_acts(T, 256, seed=50 + T)
+        y = pm.forward(0, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+        torch.cuda.synchronize()
+        ref = ref_forward(layer, x, 2, 2)
+        assert np.abs(y.float().cpu().numpy() - ref["out"]).max() <= TOL * np.abs(ref["out"]).max()
+        n_act += len(np.unique(ref["idx"]))
+    c1 = pm.counters()
+    assert c1["miss"] == c0["miss"] and c1["hit"] - c0["hit"] == n_act and c1["activated"] - c0["activated"] == n_act
     pm.close()
 
 
