@@ -111,13 +111,14 @@ int moe_route_decode(const void *x_bf16, const void *wg_bf16, const float *bias,
  * Covers tokens-per-expert of any size by chunks of <=16 rows; meant for T <= 16.
  * units_host / expert_ptr_host (HOST copies of the unit list and of the slot table row,
  * both optional): when given and max_units <= 64 the units travel in the kernel arguments
- * and the kernels read neither `units` nor `expert_ptr`. */
+ * and the kernels read neither `units` nor `expert_ptr`.
+ * phases: bit 0 = w13 + SwiGLU (x -> h), bit 1 = w2 (h -> partial rows); 3 = both. */
 int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, int k,
                             const moe_unit *units, int max_units, const int *sorted_tok,
                             const uint64_t *expert_ptr, const void *shared_ptr, void *h_r,
                             void *h_s, float *part_r, float *part_s, int *err,
                             const moe_unit *units_host, const uint64_t *expert_ptr_host,
-                            void *stream);
+                            int phases, void *stream);
 
 /* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
  * g_t = sigmoid(shared_gate_logit[t*sg_stride]) when shared_gate_logit != NULL, else 1;

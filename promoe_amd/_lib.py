@@ -48,7 +48,7 @@ _sig("moe_gate_logits", [vp, vp, vp, vp, i32, i32, i32, i32, vp])
 _sig("moe_topk", [vp, i32, i32, i32, i32, i32, vp, vp, vp])
 _sig("moe_dispatch", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_route_decode", [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
-_sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp])
+_sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_kernel_timing", [i32])
 _sig("moe_kernel_timing_read", [i32, C.POINTER(C.c_double), C.POINTER(i32)])
 _sig("moe_combine", [vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, vp])

@@ -152,7 +152,7 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
   const uint64_t *table_host = eng->h_table + (size_t)layer * eng->cfg.num_expert;
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
-                                 s->part_r, s->part_s, s->err, units_host, table_host, st);
+                                 s->part_r, s->part_s, s->err, units_host, table_host, 3, st);
 }
 
 extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
@@ -218,7 +218,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
     if ((rc = moe_experts_decode_int4(x, T, d.H, d.I, d.I_sh, k, s->units, max_units, s->sorted_tok, table,
                                       d.I_sh > 0 ? d.shared : nullptr, s->h_r, s->h_s, s->part_r, s->part_s, s->err,
-                                      nullptr, nullptr, st)))
+                                      nullptr, nullptr, 3, st)))
       return rc;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))

@@ -1172,7 +1172,7 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                                        const uint64_t *expert_ptr, const void *shared_ptr,
                                        void *h_r, void *h_s, float *part_r, float *part_s,
                                        int *err, const moe_unit *units_host,
-                                       const uint64_t *expert_ptr_host, void *stream) {
+                                       const uint64_t *expert_ptr_host, int phases, void *stream) {
   if (!x || T <= 0 || H <= 0 || H % 128 || I < 0 || I % 128 || I_sh < 0 || I_sh % 128 || !err ||
       (max_units > 0 && ((!units && !units_host) || !sorted_tok || (!expert_ptr && !expert_ptr_host) || !h_r || !part_r || I == 0)) ||
       (shared_ptr && (!h_s || !part_s || I_sh == 0))) {
@@ -1207,7 +1207,7 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                        lr.off13_z, H, H / 128, T == 1 ? 0 : H, I, I / 16, 0};
   a.n_sh_blocks = sh ? I_sh / 16 : 0;
   int grid = a.n_sh_blocks + max_units * (I / 16);
-  if (grid > 0) {
+  if (grid > 0 && (phases & 1)) {
     int rc = launch_gemv_t<true>(a, grid, T, H, H / 128, s);
     if (rc) return rc;
   }
@@ -1218,7 +1218,7 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                        I, I / 128, I, H, H / 32, 0};
   a.n_sh_blocks = sh ? H / 32 : 0;
   grid = a.n_sh_blocks + max_units * (H / 32);
-  if (grid > 0) {
+  if (grid > 0 && (phases & 2)) {
     int rc = launch_gemv_t<false>(a, grid, T, I_sh > I ? I_sh : I, (max_units > 0 ? I : I_sh) / 128, s);
     if (rc) return rc;
   }

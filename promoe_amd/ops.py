@@ -83,18 +83,21 @@ def route_decode(x, wg, bias, E: int, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
 
 
 def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
-                        H: int, I: int, I_sh: int, host_units: bool = False):
+                        H: int, I: int, I_sh: int, host_units: bool = False, phases: int = 3, ws=None):
     """Returns (part_r [P,H] fp32, part_s [T,H] fp32 or None, err int32[1])."""
     T, k = d.T, d.k
     P = T * k
     dev = x.device
-    h_r = torch.empty(max(P, 1), max(I, 1), dtype=torch.bfloat16, device=dev)
-    part_r = torch.empty(max(P, 1), H, dtype=torch.float32, device=dev)
-    h_s = part_s = None
-    if shared is not None:
-        h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
-        part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
-    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    if ws is not None:          # caller-provided workspace (part_r, part_s, err, h_r, h_s)
+        part_r, part_s, err, h_r, h_s = ws
+    else:
+        h_r = torch.empty(max(P, 1), max(I, 1), dtype=torch.bfloat16, device=dev)
+        part_r = torch.empty(max(P, 1), H, dtype=torch.float32, device=dev)
+        h_s = part_s = None
+        if shared is not None:
+            h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
+            part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+        err = torch.zeros(1, dtype=torch.int32, device=dev)
     uh = th = None
     if host_units:   # unit list and slot table resolved on the host, sent in the kernel arguments
         uh = d.units.cpu().contiguous()
@@ -102,7 +105,7 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
     check(lib.moe_experts_decode_int4(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
                                       ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
                                       ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
-                                      ptr(err), ptr(uh), ptr(th), cur_stream()), "moe_experts_decode_int4")
+                                      ptr(err), ptr(uh), ptr(th), phases, cur_stream()), "moe_experts_decode_int4")
     return part_r, part_s, err, h_r, h_s
 
 
