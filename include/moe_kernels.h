@@ -120,6 +120,23 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
                             const moe_unit *units_host, const uint64_t *expert_ptr_host,
                             int phases, void *stream);
 
+/* k4 (prefill): grouped SwiGLU expert product on the matrix cores for large token groups.
+ * Same arguments and buffer meanings as moe_experts_decode_int4 (rows of h_r / part_r in the
+ * sorted pair order; expert_ptr[e] == 0 for an active expert sets *err |= 1 and skips it).
+ *   fmt       : MOE_FMT_BF16 (expert image = w13 [2I,H] then w2 [H,I], row-major bf16)
+ *   tiles_ws  : device workspace of moe_prefill_workspace_bytes(T, k, max_units) bytes; the
+ *               list of 128-row blocks per expert is built there by a kernel, so the host
+ *               needs no copy of the dispatch counts.
+ * H % 256 == 0, I % 128 == 0, I_sh % 128 == 0.  The reference leaves this product to the
+ * framework's own expert modules (SimulateMoeLayer.forward, transformers-deepseek-moe.py:36-49). */
+int64_t moe_prefill_workspace_bytes(int T, int k, int max_units);
+int moe_prefill_tile_rows(void);
+int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int I_sh, int k, int fmt,
+                        const moe_unit *units, int max_units, const int *sorted_tok,
+                        const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
+                        float *part_r, float *part_s, void *tiles_ws, int *err, int phases,
+                        void *stream);
+
 /* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
  * g_t = sigmoid(shared_gate_logit[t*sg_stride]) when shared_gate_logit != NULL, else 1;
  * part_s may be NULL (no shared expert). */

@@ -40,3 +40,32 @@ class Int4Layer:
             ex.append((qw, s, qz))
             deq.append(O.dequant_int4(qw, s, qz, n, k))
         return tuple(deq), LY.pack_expert_int4(ex[0], ex[1], ex[2], H, I)
+
+
+class Bf16Layer:
+    """One bf16 MoE layer: bf16-representable fp32 weights (oracle side) and expert images
+    in the row-major bf16 slot layout (w13 = gate rows then up rows, then w2)."""
+
+    def __init__(self, H, I, E, I_sh=0, seed=0, shared_gate=False, zipf=None):
+        self.H, self.I, self.E, self.I_sh = H, I, E, I_sh
+        g = torch.Generator().manual_seed(seed)
+
+        def mat(n, k):
+            return O.round_bf16((torch.randn(n, k, generator=g, dtype=torch.float32) * 0.02).numpy())
+
+        self.wg = mat(E, H)
+        self.bias = O.zipf_gate_bias(E, zipf, seed=2) if zipf else None
+        self.experts_fp32, self.slots = [], []
+        for _ in range(E):
+            ws = (mat(I, H), mat(I, H), mat(H, I))
+            self.experts_fp32.append(ws)
+            self.slots.append(self.image(ws))
+        self.shared_fp32 = self.shared_img = None
+        if I_sh:
+            self.shared_fp32 = (mat(I_sh, H), mat(I_sh, H), mat(H, I_sh))
+            self.shared_img = self.image(self.shared_fp32)
+        self.shared_gate = mat(1, H)[0] if shared_gate else None
+
+    @staticmethod
+    def image(ws):
+        return np.concatenate([O.f32_to_bf16_bits(w).reshape(-1) for w in ws]).view(np.uint8)

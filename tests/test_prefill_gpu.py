@@ -1,0 +1,89 @@
+"""Parity of the MFMA prefill expert kernels (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.synth import Bf16Layer
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-2  # max |y - ref| / max |ref|
+
+
+def bf16_dev(a, dev):
+    return torch.from_numpy(np.asarray(a, np.float32)).to(torch.bfloat16).to(dev)
+
+
+def run_prefill_gpu(layer, x, k, mode, dev, resident=None):
+    from promoe_amd import ops, _lib as L
+    H, I, E, I_sh = layer.H, layer.I, layer.E, layer.I_sh
+    T = x.shape[0]
+    xd = bf16_dev(x, dev)
+    wg = layer.wg
+    if layer.shared_gate is not None:
+        wg = np.concatenate([wg, layer.shared_gate[None, :]], axis=0)
+    bias = None
+    if layer.bias is not None:
+        bias = torch.from_numpy(np.concatenate([layer.bias, np.zeros(wg.shape[0] - E, np.float32)])).to(dev)
+    logits = ops.gate_logits(xd, bf16_dev(wg, dev), bias)
+    idx, w = ops.topk(logits, k, mode, E=E)
+    d = ops.dispatch(idx, E)
+    slots = [torch.from_numpy(s).to(dev) for s in layer.slots]
+    table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
+                          for e in range(E)], dtype=torch.int64, device=dev)
+    shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
+    part_r, part_s, err, h_r, h_s, _ = ops.experts_prefill(xd, d, table, shared, H, I, I_sh, L.FMT_BF16)
+    sg = logits[:, E] if layer.shared_gate is not None else None
+    y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
+    torch.cuda.synchronize()
+    return dict(y=y.float().cpu().numpy(), idx=idx.cpu().numpy(), w=w.cpu().numpy(),
+                logits=logits.cpu().numpy(), err=int(err.cpu()[0]), d=d)
+
+
+def check_prefill(layer, T, k, mode, dev, seed=1):
+    x = O.synth_acts(T, layer.H, seed=seed)
+    got = run_prefill_gpu(layer, x, k, mode, dev)
+    lg = O.gate_logits_ordered(x, layer.wg)
+    if layer.bias is not None:
+        lg = (lg + layer.bias[None, :]).astype(np.float32)
+    ref = O.moe_forward(x, layer.wg, layer.experts_fp32, k, mode, shared=layer.shared_fp32,
+                        shared_gate=layer.shared_gate, logits=lg)
+    assert got["err"] == 0
+    assert np.array_equal(got["idx"], ref["idx"])
+    _, _, sp, _ = O.dispatch(ref["idx"], layer.E)
+    assert np.array_equal(got["d"].sorted_pair.cpu().numpy()[:T * k], sp)
+    err = np.abs(got["y"] - ref["out"]).max() / np.abs(ref["out"]).max()
+    print(f"  T={T} k={k} mode={mode} max-rel-err={err:.3e}", flush=True)
+    assert err <= TOL
+    return err
+
+
+@pytest.mark.parametrize("T", [1, 17, 128, 129, 300, 700])
+def test_prefill_layer_small(cuda, T):
+    print(f"case prefill_small T={T}", flush=True)
+    check_prefill(Bf16Layer(H=256, I=384, E=8, I_sh=256, seed=3), T, 2, 0, cuda)
+
+
+def test_prefill_layer_small_variants(cuda):
+    print("case prefill_small_variants", flush=True)
+    # no shared expert, Mixtral routing
+    check_prefill(Bf16Layer(H=512, I=128, E=8, I_sh=0, seed=4), 200, 2, 2, cuda)
+    # sigmoid-gated shared expert, renormalised routing, Zipf bias: some experts get no token
+    check_prefill(Bf16Layer(H=256, I=256, E=60, I_sh=512, seed=5, shared_gate=True, zipf=1.4), 150, 4, 1, cuda)
+    # more units than one scan pass is not needed (E <= 1024), K not a multiple of 128
+    check_prefill(Bf16Layer(H=768, I=640, E=4, I_sh=128, seed=6), 260, 2, 0, cuda)
+
+
+def test_prefill_non_resident_expert_is_reported(cuda):
+    print("case prefill_non_resident", flush=True)
+    layer = Bf16Layer(H=256, I=128, E=4, I_sh=0, seed=7)
+    got = run_prefill_gpu(layer, O.synth_acts(64, 256), 2, 0, cuda, resident={0, 1})
+    assert got["err"] == 1
+
+
+def test_prefill_layer_qwen_shape(cuda):
+    print("case prefill_qwen T=2048", flush=True)
+    # Qwen1.5-MoE-A2.7B layer: H 2048, 60 experts x I 1408, top-4, sigmoid-gated shared expert I 5632
+    layer = Bf16Layer(H=2048, I=1408, E=60, I_sh=5632, seed=0, shared_gate=True)
+    check_prefill(layer, 2048, 4, 0, cuda)
