@@ -37,7 +37,9 @@ extern "C" {
 
 /* weight formats of an expert (all weights [out,in]) */
 #define MOE_FMT_INT4_G128 0 /* tiled int4, group 128 along K, fp16 scales, uint4 zeros */
-#define MOE_FMT_BF16 1      /* row-major bf16: w13 [2I,H] (gate rows then up rows), w2 [H,I] */
+#define MOE_FMT_BF16 1      /* bf16: w13 [2I,H] (gate rows then up rows) then w2 [H,I], each matrix in
+                             * blocks of 32 rows x 64 k (4 KiB; block (nb,kb) at element (((nb/4)*K/64+kb)*4+nb%4)*2048,
+                             * inside a block element [j][q][n][e] is W[32nb+n][64kb+32q+8j+e]) */
 
 const char *moe_last_error(void);
 
@@ -123,9 +125,9 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
 /* k4 (prefill): grouped SwiGLU expert product on the matrix cores for large token groups.
  * Same arguments and buffer meanings as moe_experts_decode_int4 (rows of h_r / part_r in the
  * sorted pair order; expert_ptr[e] == 0 for an active expert sets *err |= 1 and skips it).
- *   fmt       : MOE_FMT_BF16 (expert image = w13 [2I,H] then w2 [H,I], row-major bf16)
+ *   fmt       : MOE_FMT_BF16 (expert image = blocked w13 [2I,H] then blocked w2 [H,I])
  *   tiles_ws  : device workspace of moe_prefill_workspace_bytes(T, k, max_units) bytes; the
- *               list of 128-row blocks per expert is built there by a kernel, so the host
+ *               list of row tiles per expert is built there by a kernel, so the host
  *               needs no copy of the dispatch counts.
  * H % 256 == 0, I % 128 == 0, I_sh % 128 == 0.  The reference leaves this product to the
  * framework's own expert modules (SimulateMoeLayer.forward, transformers-deepseek-moe.py:36-49). */

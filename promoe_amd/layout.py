@@ -90,3 +90,53 @@ def split_chunks_int4(H: int, I: int):
     names = ["off13_q", "off13_s", "off13_z", "off2_q", "off2_s", "off2_z"]
     ends = [lay[n] for n in names[1:]] + [lay["total_bytes"]]
     return [(n.replace("off", "w"), lay[n], e - lay[n]) for n, e in zip(names, ends)]
+
+
+# ---- bf16 experts -------------------------------------------------------------------
+# A matrix W[N,K] is stored as blocks of 32 rows x 64 k (2048 elements, 4 KiB).  Block
+# (nb, kb) lies at element offset (((nb//4)*(K/64) + kb)*4 + nb%4)*2048: the four blocks of a
+# 128-row group are adjacent for each k slab.  The slabs of group g are stored rotated: slab
+# kb sits at position (kb + g*s) % (K/64), s = slab_step(K/64), which keeps groups that are
+# read in step on different DRAM channels.  Inside a block the order is [j][q][n][e] with
+# k = 64kb + 32q + 8j + e: the 64 lanes (lane = 32q + n) of a wave read 16 bytes each of one
+# contiguous KiB per j, already in the operand order of v_mfma_f32_32x32x16_bf16.
+
+def slab_step(nk: int) -> int:
+    """Smallest odd s >= 3 coprime with nk."""
+    import math
+    s = 3
+    while math.gcd(s, nk) != 1:
+        s += 2
+    return s
+
+
+def tile_bf16(w_bits: np.ndarray) -> np.ndarray:
+    """w_bits uint16 [N,K] (bf16 bit patterns) -> flat uint16 array in the block layout."""
+    N, K = w_bits.shape
+    assert N % 128 == 0 and K % 64 == 0
+    nk = K // 64
+    t = w_bits.reshape(N // 128, 4, 32, nk, 2, 4, 8)      # g w n kb q j e
+    t = np.ascontiguousarray(t.transpose(0, 3, 1, 5, 4, 2, 6))  # g kb w j q n e
+    s = slab_step(nk)
+    for g in range(N // 128):
+        t[g] = np.roll(t[g], (g * s) % nk, axis=0)
+    return t.reshape(-1)
+
+
+def untile_bf16(flat: np.ndarray, N: int, K: int) -> np.ndarray:
+    nk = K // 64
+    t = flat.reshape(N // 128, nk, 4, 4, 2, 32, 8).copy()       # g kb w j q n e
+    s = slab_step(nk)
+    for g in range(N // 128):
+        t[g] = np.roll(t[g], -((g * s) % nk), axis=0)
+    return np.ascontiguousarray(t.transpose(0, 2, 5, 1, 4, 3, 6)).reshape(N, K)
+
+
+def pack_expert_bf16(gate_bits, up_bits, down_bits) -> np.ndarray:
+    """Slot image of one bf16 expert: tiled w13 (gate rows, then up rows) followed by tiled w2."""
+    w13 = np.concatenate([gate_bits, up_bits], axis=0)
+    return np.concatenate([tile_bf16(w13), tile_bf16(down_bits)]).view(np.uint8)
+
+
+def bf16_expert_bytes(H: int, I: int) -> int:
+    return 3 * I * H * 2

@@ -44,7 +44,7 @@ class Int4Layer:
 
 class Bf16Layer:
     """One bf16 MoE layer: bf16-representable fp32 weights (oracle side) and expert images
-    in the row-major bf16 slot layout (w13 = gate rows then up rows, then w2)."""
+    in the blocked bf16 slot layout (w13 = gate rows then up rows, then w2)."""
 
     def __init__(self, H, I, E, I_sh=0, seed=0, shared_gate=False, zipf=None):
         self.H, self.I, self.E, self.I_sh = H, I, E, I_sh
@@ -68,4 +68,4 @@ class Bf16Layer:
 
     @staticmethod
     def image(ws):
-        return np.concatenate([O.f32_to_bf16_bits(w).reshape(-1) for w in ws]).view(np.uint8)
+        return LY.pack_expert_bf16(*[O.f32_to_bf16_bits(w) for w in ws])
