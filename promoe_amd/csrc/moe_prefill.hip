@@ -44,6 +44,7 @@ struct PfClass {
   const int *n_tiles_real;  // device: tiles actually in use (<= n_mtiles, the launch's upper bound)
   long long w_off;      // byte offset of the matrix inside the expert image
   long long half_delta; // weight-row offset of the second column half relative to the first
+  long long off_s, off_z; // int4: byte offsets of the scale / zero sections (w_off = the nibble section)
   int act_stride, out_stride, K, n_ntiles, n_mtiles, n_cols_per_tile;
   int m_fastest;        // block order inside the class
   int slab_step;        // storage rotation per 128-row group: smallest odd s >= 3 coprime with K/64
@@ -220,11 +221,248 @@ __global__ __launch_bounds__(512, 1) void k_prefill_gemm(const PfArgs a) {
     }
 }
 
+// ---- int4-g128 experts ----------------------------------------------------------------
+// Same tiling as the bf16 kernel (8 waves, tile of up to 256 rows, wave w of group g owns 64
+// weight rows and the 32-row blocks g, g+2, ...), K advances one quantisation group (128) at
+// a time.  The int4 tiles of the slot layout are already in the operand order of
+// v_mfma_f32_16x16x32_f16 (lane = row l&15, k quarter l>>4, dword j = 8 consecutive k), so a
+// wave loads them straight into registers and dequantises there: the nibble pair under mask
+// 0x000f000f is OR-ed into 0x6400 (fp16 1024+q), then (h - (1024+z)) * s with two packed
+// fp16 operations per pair (the subtraction is exact).  gfx950 has packed fp16 arithmetic
+// but no packed bf16 arithmetic, hence fp16 operands: activations are converted bf16 -> fp16
+// while they are staged into LDS (exact for |x| < 65504 outside the fp16 subnormal range).
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const uint16_t g_u16;
+typedef __attribute__((address_space(1))) const unsigned char g_u8;
+
+#define PI_LDK 136  // LDS row stride in fp16 (128 + 8 pad = 272 bytes)
+#define PI_BM 192   // most rows of one tile: 6 blocks of 32 (96 accumulator registers per wave)
+
+static __device__ __forceinline__ u32 pf_bf16x2_to_f16x2(u32 d) {
+  // both halves are bf16; fp16 has more mantissa bits, so round-to-zero conversion is exact
+  auto h = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(d << 16), __uint_as_float(d & 0xffff0000u));
+  return __builtin_bit_cast(u32, h);
+}
+// s2 / nz2: the row's scale and -(1024 + zero) as fp16 bit patterns replicated in both halves
+static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2) {
+  const u32 M = 0x000f000fu, C = 0x64006400u;
+  u32x4_t v;
+  v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
+  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1024 + q, exact
+  const f16x8_t nz8 = __builtin_bit_cast(f16x8_t, u32x4_t{nz2, nz2, nz2, nz2});
+  const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
+  return (h + nz8) * s8;                                // exact difference, then one rounding
+}
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
+static __device__ __forceinline__ rsrc_t pf_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
+}
+static __device__ __forceinline__ const unsigned char *pf_uniform(const unsigned char *p) {
+  const unsigned long long v = (unsigned long long)p;
+  const u32 lo = __builtin_amdgcn_readfirstlane((u32)v), hi = __builtin_amdgcn_readfirstlane((u32)(v >> 32));
+  return (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+}
+
+struct PiMeta { u32 sc[4]; u32 zz[4]; };  // raw fp16 scale bits / zero nibble of the lane's row in the 4 tiles
+
+template <int NBW>
+static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_t *As, const rsrc_t rx, const u32 (&a_off)[6],
+                                                   const rsrc_t rq, const rsrc_t rs, const rsrc_t rz, int G, int nb, int tid) {
+  const int lane = tid & 63, g = tid >> 8;
+  const int r = lane & 15, qd = lane >> 4;
+  const int ch = tid & 15, r0 = tid >> 4;  // staging: row r0 + 32 i (block i), 16-byte chunk ch of the 128-k group
+  u32x4_t ra[3], wA[4], wB[4];
+  PiMeta mA, mB;
+  // activations of the next group travel in two halves (row blocks 0..2, then 3..5) through
+  // the same three staging registers
+  auto gloadA = [&](int gi, int half) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (3 * half + i < nb) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[3 * half + i], gi * 256, 0);
+  };
+  auto sstore = [&](int st, int half) {
+    uint16_t *A_ = As + st * PI_BM * PI_LDK;
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+      if (3 * half + i < nb) {
+        u32x4_t v;
+        v.x = pf_bf16x2_to_f16x2(ra[i].x); v.y = pf_bf16x2_to_f16x2(ra[i].y);
+        v.z = pf_bf16x2_to_f16x2(ra[i].z); v.w = pf_bf16x2_to_f16x2(ra[i].w);
+        *(u32x4_t *)(A_ + (r0 + 32 * (3 * half + i)) * PI_LDK + ch * 8) = v;
+      }
+  };
+  auto gloadW = [&](u32x4_t(&wq)[4], PiMeta &m, int gi) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      wq[t] = __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, (t * G + gi) * 1024, 0);
+      m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * r, (t * G + gi) * 32, 0);
+      m.zz[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, r >> 1, (t * G + gi) * 8, 0);
+    }
+  };
+  auto compute2 = [&](int st, const u32x4_t(&wq)[4], const PiMeta &m, int j0) {
+    const uint16_t *A_ = As + st * PI_BM * PI_LDK + (32 * g + r) * PI_LDK + 32 * qd;
+    u32 s2[4], z2[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const u32 sb = m.sc[t] & 0xffffu;
+      s2[t] = sb | (sb << 16);
+      const u32 zb = 0xe400u | ((m.zz[t] >> (4 * (r & 1))) & 15u);  // -(1024 + zero)
+      z2[t] = zb | (zb << 16);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int j = j0 + jj;
+      f16x8_t wd[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) wd[t] = pf_deq8_f16(wq[t][j], s2[t], z2[t]);
+#pragma unroll
+      for (int tb = 0; tb < 2 * NBW; ++tb) {
+        const f16x8_t xa = *(const f16x8_t *)(A_ + (64 * (tb >> 1) + 16 * (tb & 1)) * PI_LDK + 8 * j);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t][tb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, wd[t], acc[t][tb], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto step = [&](int gi, const u32x4_t(&cur)[4], const PiMeta &mc, u32x4_t(&nxt)[4], PiMeta &mn) {
+    const bool more = gi + 1 < G;
+    if (more) {
+      gloadA(gi + 1, 0);
+      if (NBW > 0) gloadW(nxt, mn, gi + 1);
+    }
+    if (NBW > 0) compute2(gi & 1, cur, mc, 0);
+    if (more) {
+      sstore((gi + 1) & 1, 0);
+      if (nb > 3) gloadA(gi + 1, 1);
+    }
+    if (NBW > 0) compute2(gi & 1, cur, mc, 2);
+    if (more) {
+      if (nb > 3) sstore((gi + 1) & 1, 1);
+      __syncthreads();
+    }
+  };
+  gloadA(0, 0);
+  if (NBW > 0) gloadW(wA, mA, 0);
+  sstore(0, 0);
+  if (nb > 3) {
+    gloadA(0, 1);
+    sstore(0, 1);
+  }
+  __syncthreads();
+  for (int gi = 0; gi < G; gi += 2) {
+    step(gi, wA, mA, wB, mB);
+    if (gi + 1 < G) step(gi + 1, wB, mB, wA, mA);
+  }
+}
+
+template <bool SWIGLU>
+__global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
+  extern __shared__ __align__(16) uint16_t As[];  // [2][PI_BM][PI_LDK] fp16
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane((tid >> 6) & 3), g = tid >> 8;
+  const int r = lane & 15, qd = lane >> 4;
+
+  // block order: as in k_prefill_gemm
+  const int pad0 = (a.c[0].n_blocks + 7) & ~7;
+  const int ci = (int)blockIdx.x >= pad0;
+  const int pb = ci ? blockIdx.x - pad0 : blockIdx.x;
+  const int n_mt = *a.c[ci].n_tiles_real;
+  const int n_real = n_mt * a.c[ci].n_ntiles;
+  const int per_xcd = (n_real + 7) >> 3;
+  if ((pb >> 3) >= per_xcd) return;
+  int bid = (pb & 7) * per_xcd + (pb >> 3);
+  if (bid >= n_real) return;
+  const PfClass &c = a.c[ci];
+  int mt, nt;
+  if (c.m_fastest) { nt = bid / n_mt; mt = bid - nt * n_mt; }
+  else { mt = bid / c.n_ntiles; nt = bid - mt * c.n_ntiles; }
+  const PfTile tile = c.tiles[mt];
+  if (tile.rows <= 0) return;
+  const int K = c.K, G = K >> 7;
+
+  const int ch = tid & 15, r0 = tid >> 4;
+  u32 a_off[6];  // byte offsets into the activation matrix (< 2^31: checked by the launcher)
+#pragma unroll
+  for (int i = 0; i < 6; ++i) {
+    int row = r0 + 32 * i;
+    row = row < tile.rows ? row : 0;  // rows past the group's end re-read row 0 (never stored)
+    const int grow = tile.row0 + row;
+    const int arow = c.gather ? c.gather[grow] : grow;
+    a_off[i] = ((u32)arow * (u32)c.act_stride + ch * 8) * 2;
+  }
+  // the wave's 4 consecutive 16-row blocks: (gate, up, gate, up) of two 16-column blocks of
+  // h in the w13 pass, 64 consecutive output columns in the w2 pass
+  const int rb0 = 16 * nt + 4 * w;
+  const unsigned char *base = pf_uniform((const unsigned char *)tile.w_base);
+  const rsrc_t rq = pf_rsrc(base + c.w_off + (size_t)rb0 * G * 1024, 4u * G * 1024u);
+  const rsrc_t rs = pf_rsrc(base + c.off_s + (size_t)rb0 * G * 32, 4u * G * 32u);
+  const rsrc_t rz = pf_rsrc(base + c.off_z + (size_t)rb0 * G * 8, 4u * G * 8u);
+  const rsrc_t rx = pf_rsrc(c.act, 0x7fffffffu);
+
+  f32x4_t acc[4][6];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int tb = 0; tb < 6; ++tb) acc[t][tb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int nb = (tile.rows + 31) >> 5;
+  const int nbw = (nb - g + 1) >> 1;
+  switch (nbw) {
+    case 0: pi_mainloop<0>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 1: pi_mainloop<1>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 2: pi_mainloop<2>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    default: pi_mainloop<3>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+  }
+  // epilogue.  acc[t][tb] element i of lane l: weight row r of tile t, token row
+  // 32*(2*(tb/2)+g) + 16*(tb%2) + 4*qd + i of the tile
+#pragma unroll
+  for (int tb = 0; tb < 6; ++tb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 32 * (2 * (tb >> 1) + g) + 16 * (tb & 1) + 4 * qd + i;
+      if (row < tile.rows) {
+        const size_t orow = (size_t)(tile.row0 + row) * c.out_stride;
+        if (SWIGLU) {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const float gt = acc[2 * b][tb][i], up = acc[2 * b + 1][tb][i];
+            ((uint16_t *)c.out)[orow + 16 * (rb0 / 2 + b) + r] = pf_f32_to_bf16(gt / (1.f + expf(-gt)) * up);
+          }
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) ((float *)c.out)[orow + 16 * (rb0 + t) + r] = acc[t][tb][i];
+        }
+      }
+    }
+}
+
+
 static int pf_gcd(int a, int b) { return b ? pf_gcd(b, a % b) : a; }
 static int pf_slab_step(int nk) {
   int s = 3;
   while (pf_gcd(s, nk) != 1) s += 2;
   return s;
+}
+
+static int pi_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
+  if (a.n_blocks_total <= 0) return MOE_OK;
+  const int grid = ((a.c[0].n_blocks + 7) & ~7) + ((a.c[1].n_blocks + 7) & ~7);
+  const size_t lds = (size_t)2 * PI_BM * PI_LDK * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute((const void *)k_prefill_int4<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e2 = hipFuncSetAttribute((const void *)k_prefill_int4<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (int rc = moe_check_hip(e1 != hipSuccess ? e1 : e2, "hipFuncSetAttribute(k_prefill_int4)")) return rc;
+    attr_set = true;
+  }
+  moe_ktimer_begin(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
+  if (swiglu) hipLaunchKernelGGL(k_prefill_int4<true>, dim3(grid), dim3(512), lds, s, a);
+  else hipLaunchKernelGGL(k_prefill_int4<false>, dim3(grid), dim3(512), lds, s, a);
+  moe_ktimer_end(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
+  return moe_check_launch("k_prefill_int4");
 }
 
 static int pf_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
@@ -255,8 +493,8 @@ __global__ __launch_bounds__(1024) void k_prefill_tiles(const moe_unit *__restri
                                                         PfTile *__restrict__ tiles, int n_tiles_max,
                                                         PfTile *__restrict__ sh_tiles, int n_sh_tiles,
                                                         PfTile *__restrict__ sh_tiles2, int n_sh_tiles2,
-                                                        unsigned long long shared_base, int T, int *__restrict__ n_real,
-                                                        int *__restrict__ err) {
+                                                        unsigned long long shared_base, int T, int cap, int cap_s, int cap_s2,
+                                                        int *__restrict__ n_real, int *__restrict__ err) {
   __shared__ int scan[1024];
   const int tid = threadIdx.x;
   int total_prev = 0;
@@ -272,7 +510,7 @@ __global__ __launch_bounds__(1024) void k_prefill_tiles(const moe_unit *__restri
         else atomicOr(err, 1);
       }
     }
-    const int nt = (m + PF_BM - 1) / PF_BM;
+    const int nt = (m + cap - 1) / cap;
     // rows of a group are split evenly over its tiles, in multiples of 32
     const int per = nt ? ((((m + nt - 1) / nt) + 31) & ~31) : 0;
     scan[tid] = nt;
@@ -299,11 +537,11 @@ __global__ __launch_bounds__(1024) void k_prefill_tiles(const moe_unit *__restri
     tiles[i] = t;
   }
   for (int i = tid; i < n_sh_tiles; i += 1024) {
-    PfTile t; t.w_base = shared_base; t.row0 = i * PF_BM_SHARED; t.rows = min(PF_BM_SHARED, T - i * PF_BM_SHARED);
+    PfTile t; t.w_base = shared_base; t.row0 = i * cap_s; t.rows = min(cap_s, T - i * cap_s);
     sh_tiles[i] = t;
   }
   for (int i = tid; i < n_sh_tiles2; i += 1024) {
-    PfTile t; t.w_base = shared_base; t.row0 = i * PF_BM_SHARED_W2; t.rows = min(PF_BM_SHARED_W2, T - i * PF_BM_SHARED_W2);
+    PfTile t; t.w_base = shared_base; t.row0 = i * cap_s2; t.rows = min(cap_s2, T - i * cap_s2);
     sh_tiles2[i] = t;
   }
 }
@@ -312,7 +550,7 @@ extern "C" int moe_prefill_tile_rows(void) { return PF_BM; }
 
 extern "C" int64_t moe_prefill_workspace_bytes(int T, int k, int max_units) {
   const int64_t P = (int64_t)T * k;
-  return (P / PF_BM + max_units + (T + PF_BM_SHARED - 1) / PF_BM_SHARED + (T + PF_BM_SHARED_W2 - 1) / PF_BM_SHARED_W2 + 3) * (int64_t)sizeof(PfTile);
+  return (P / 128 + max_units + 2 * ((T + 127) / 128) + 3) * (int64_t)sizeof(PfTile);  // covers every tile height in use (>= 128)
 }
 
 extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int I_sh, int k, int fmt,
@@ -327,23 +565,32 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
     moe_set_error("moe_experts_prefill: NULL or negative argument");
     return MOE_EINVAL;
   }
-  if (fmt != MOE_FMT_BF16) {
+  if (fmt != MOE_FMT_BF16 && fmt != MOE_FMT_INT4_G128) {
     moe_set_error("moe_experts_prefill: weight format %d not supported by the prefill kernels", fmt);
     return MOE_EINVAL;
+  }
+  const bool int4 = fmt == MOE_FMT_INT4_G128;
+  {
+    const long long widest = I > H ? I : H, rows = (long long)T * (k > 1 ? k : 1);
+    if (int4 && (rows * widest * 2 >= (1ll << 31) || (shared_ptr && (long long)T * (I_sh > H ? I_sh : H) * 2 >= (1ll << 31)))) {
+      moe_set_error("moe_experts_prefill: activation buffers of 2 GiB or more are not supported (T=%d k=%d)", T, k);
+      return MOE_EINVAL;
+    }
   }
   if (H % 256 || I % 128 || (shared_ptr && I_sh % 128)) {
     moe_set_error("moe_experts_prefill: H %% 256 == 0 and I %% 128 == 0 required (H=%d I=%d I_sh=%d)", H, I, I_sh);
     return MOE_EINVAL;
   }
   const long long P = (long long)T * k;
-  const int n_r = (int)(P / PF_BM) + max_units;
-  const int n_s = shared_ptr ? (T + PF_BM_SHARED - 1) / PF_BM_SHARED : 0;
-  const int n_s2 = shared_ptr ? (T + PF_BM_SHARED_W2 - 1) / PF_BM_SHARED_W2 : 0;
+  const int cap = int4 ? PI_BM : PF_BM, cap_s = int4 ? PI_BM : PF_BM_SHARED, cap_s2 = PF_BM_SHARED_W2;
+  const int n_r = (int)(P / cap) + max_units;
+  const int n_s = shared_ptr ? (T + cap_s - 1) / cap_s : 0;
+  const int n_s2 = shared_ptr ? (T + cap_s2 - 1) / cap_s2 : 0;
   int *n_real = (int *)tiles_ws;  // [0] routed tiles in use, [1] shared tiles (w13 pass), [2] shared tiles (w2 pass)
   PfTile *tiles = (PfTile *)tiles_ws + 1, *sh_tiles = tiles + n_r, *sh_tiles2 = sh_tiles + n_s;
   hipLaunchKernelGGL(k_prefill_tiles, dim3(1), dim3(1024), 0, s, units, max_units,
                      (const unsigned long long *)expert_ptr, tiles, n_r, sh_tiles, n_s, sh_tiles2, n_s2,
-                     (unsigned long long)(uintptr_t)shared_ptr, T, n_real, err);
+                     (unsigned long long)(uintptr_t)shared_ptr, T, cap, cap_s, cap_s2, n_real, err);
   if (int rc = moe_check_launch("k_prefill_tiles")) return rc;
   for (int w2 = 0; w2 < 2; ++w2) {
     if (!(phases & (w2 ? 2 : 1))) continue;
@@ -369,11 +616,18 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
         c.K = Ii; c.w_off = (long long)2 * Ii * H * 2; c.half_delta = PF_BNH; c.n_cols_per_tile = 2 * PF_BNH;
         c.n_ntiles = H / (2 * PF_BNH);
       }
+      if (int4) {
+        moe_int4_layout lay;
+        if (int rc = moe_int4_layout_make(H, Ii, &lay)) return rc;
+        c.w_off = w2 ? lay.off2_q : lay.off13_q;
+        c.off_s = w2 ? lay.off2_s : lay.off13_s;
+        c.off_z = w2 ? lay.off2_z : lay.off13_z;
+      }
       c.n_blocks = c.n_mtiles * c.n_ntiles;
       c.slab_step = pf_slab_step(c.K / PF_BK);
       a.n_blocks_total += c.n_blocks;
     }
-    if (int rc = pf_launch(!w2, a, s)) return rc;
+    if (int rc = int4 ? pi_launch(!w2, a, s) : pf_launch(!w2, a, s)) return rc;
   }
   return MOE_OK;
 }

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from tests.synth import Bf16Layer
+from tests.synth import Bf16Layer, Int4Layer
 
 pytestmark = pytest.mark.gpu
 
@@ -33,7 +33,8 @@ def run_prefill_gpu(layer, x, k, mode, dev, resident=None):
     table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
                           for e in range(E)], dtype=torch.int64, device=dev)
     shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
-    part_r, part_s, err, h_r, h_s, _ = ops.experts_prefill(xd, d, table, shared, H, I, I_sh, L.FMT_BF16)
+    fmt = L.FMT_BF16 if isinstance(layer, Bf16Layer) else L.FMT_INT4_G128
+    part_r, part_s, err, h_r, h_s, _ = ops.experts_prefill(xd, d, table, shared, H, I, I_sh, fmt)
     sg = logits[:, E] if layer.shared_gate is not None else None
     y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
     torch.cuda.synchronize()
@@ -87,3 +88,32 @@ def test_prefill_layer_qwen_shape(cuda):
     # Qwen1.5-MoE-A2.7B layer: H 2048, 60 experts x I 1408, top-4, sigmoid-gated shared expert I 5632
     layer = Bf16Layer(H=2048, I=1408, E=60, I_sh=5632, seed=0, shared_gate=True)
     check_prefill(layer, 2048, 4, 0, cuda)
+
+
+# ---- int4-g128 experts through the same entry point ----
+
+@pytest.mark.parametrize("T", [1, 17, 96, 97, 193, 400, 700])
+def test_prefill_int4_layer_small(cuda, T):
+    print(f"case prefill_int4_small T={T}", flush=True)
+    check_prefill(Int4Layer(H=256, I=384, E=8, I_sh=256, seed=3), T, 2, 0, cuda)
+
+
+def test_prefill_int4_layer_small_variants(cuda):
+    print("case prefill_int4_small_variants", flush=True)
+    check_prefill(Int4Layer(H=512, I=128, E=8, I_sh=0, seed=4), 200, 2, 2, cuda)
+    check_prefill(Int4Layer(H=256, I=256, E=60, I_sh=512, seed=5, shared_gate=True, zipf=1.4), 150, 4, 1, cuda)
+    check_prefill(Int4Layer(H=768, I=640, E=4, I_sh=128, seed=6), 260, 2, 0, cuda)
+
+
+def test_prefill_int4_non_resident_expert_is_reported(cuda):
+    print("case prefill_int4_non_resident", flush=True)
+    layer = Int4Layer(H=256, I=128, E=4, I_sh=0, seed=7)
+    got = run_prefill_gpu(layer, O.synth_acts(64, 256), 2, 0, cuda, resident={0, 1})
+    assert got["err"] == 1
+
+
+def test_prefill_int4_deepseek_shape(cuda):
+    print("case prefill_int4_deepseek T=512", flush=True)
+    # DeepSeek-MoE-16B layer shape; 16 experts instead of 64 keeps host-side quantisation short
+    layer = Int4Layer(H=2048, I=1408, E=16, I_sh=2816, seed=0, zipf=1.2)
+    check_prefill(layer, 512, 6, 0, cuda)
