@@ -19,7 +19,7 @@ struct LayerState {
       *sorted_tok = nullptr, *n_active = nullptr, *err = nullptr;
   moe_unit *units = nullptr, *units_sub = nullptr;
   int64_t *active_ids = nullptr;
-  void *h_r = nullptr, *h_s = nullptr;
+  void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
   // pinned host mirrors
   moe_unit *units_host = nullptr, *units_sub_host = nullptr;
   int *n_active_host = nullptr, *err_host = nullptr;
@@ -56,7 +56,11 @@ extern "C" int moe_set_layer(moe_engine *eng, int layer, const moe_layer_desc *d
     moe_set_error("moe_set_layer: bad descriptor (H=%d I=%d I_sh=%d k=%d)", d->H, d->I, d->I_sh, d->top_k);
     return MOE_EINVAL;
   }
-  if (d->fmt != MOE_FMT_INT4_G128) { moe_set_error("moe_set_layer: weight format %d not supported by this entry point", d->fmt); return MOE_EINVAL; }
+  if (d->fmt != MOE_FMT_INT4_G128 && d->fmt != MOE_FMT_BF16) { moe_set_error("moe_set_layer: weight format %d not supported by this entry point", d->fmt); return MOE_EINVAL; }
+  if (d->fmt == MOE_FMT_BF16 && (d->H % 256 || d->I % 128 || d->I_sh % 128)) {
+    moe_set_error("moe_set_layer: bf16 experts need H %% 256 == 0 and I %% 128 == 0 (H=%d I=%d I_sh=%d)", d->H, d->I, d->I_sh);
+    return MOE_EINVAL;
+  }
   eng->layer_desc[layer] = *d;
   return MOE_OK;
 }
@@ -115,6 +119,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, (uint16_t **)&s->h_s, (size_t)T * I_sh);
   rc |= dalloc(s, &s->part_r, P * H);
   rc |= dalloc(s, &s->part_s, (size_t)T * H);
+  rc |= dalloc(s, (unsigned char **)&s->tiles_ws, (size_t)moe_prefill_workspace_bytes(T, k, s->max_units));
   rc |= halloc(s, &s->units_host, s->max_units);
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
   rc |= halloc(s, &s->n_active_host, 1);
@@ -145,11 +150,22 @@ int moe_forward_harvest(moe_engine *eng, bool wait) {
   return MOE_OK;
 }
 
+// Expert product of one launch group.  Token groups of prefill size (and every bf16 layer)
+// go to the matrix-core kernels, decode batches to the bandwidth-bound GEMV kernels.
+static bool use_prefill(const moe_layer_desc &d, int T) {
+  if (d.fmt == MOE_FMT_BF16) return true;
+  return T > 16 && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
+}
+
 static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
                      const moe_unit *units_dev, const moe_unit *units_host, int n_units, bool with_shared,
                      int layer, const uint64_t *table, hipStream_t st) {
+  if (use_prefill(d, T))
+    return moe_experts_prefill(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
+                               s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
+                               s->part_s, s->tiles_ws, s->err, 3, st);
   // the host knows the units and the slot addresses: they travel in the kernel arguments
-  const uint64_t *table_host = eng->h_table + (size_t)layer * eng->cfg.num_expert;
+  const uint64_t *table_host = units_host ? eng->h_table + (size_t)layer * eng->cfg.num_expert : nullptr;
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
                                  s->part_r, s->part_s, s->err, units_host, table_host, 3, st);
@@ -216,10 +232,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
-    if ((rc = moe_experts_decode_int4(x, T, d.H, d.I, d.I_sh, k, s->units, max_units, s->sorted_tok, table,
-                                      d.I_sh > 0 ? d.shared : nullptr, s->h_r, s->h_s, s->part_r, s->part_s, s->err,
-                                      nullptr, nullptr, 3, st)))
-      return rc;
+    if ((rc = run_units(eng, d, s, x, T, s->units, nullptr, max_units, d.I_sh > 0, layer, table, st))) return rc;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
       return rc;

@@ -270,8 +270,8 @@ class PrefetchMngr:
 
     # -- fused forward --
     def set_layer(self, layer_id: int, H, I, I_sh, top_k, route_mode, gate_w, gate_bias=None, shared=None,
-                  shared_gated=False):
-        d = L.LayerDesc(H, I, I_sh, top_k, route_mode, 0, int(shared_gated), L.ptr(gate_w), L.ptr(gate_bias),
+                  shared_gated=False, fmt: int = L.FMT_INT4_G128):
+        d = L.LayerDesc(H, I, I_sh, top_k, route_mode, fmt, int(shared_gated), L.ptr(gate_w), L.ptr(gate_bias),
                         L.ptr(shared))
         self._keep.append((gate_w, gate_bias, shared))
         check(lib.moe_set_layer(self._h, layer_id, C.byref(d)), "set_layer")

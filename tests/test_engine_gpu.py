@@ -9,17 +9,19 @@ from oracle import cache_oracle as CO
 from promoe_amd import _lib as L
 from promoe_amd import engine as EG
 from promoe_amd import layout as LY
-from tests.synth import Int4Layer
+from tests.synth import Int4Layer, Bf16Layer
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
 
 
-def build_engine(layers, k, dev, mode=0, **cfg):
-    """Register every expert image (pinned host memory, six chunks each) and start the engine."""
+def build_engine(layers, k, dev, mode=0, max_tokens=64, **cfg):
+    """Register every expert image (pinned host memory, six chunks each for int4, one for
+    bf16) and start the engine."""
     Lyr, E = len(layers), layers[0].E
     H, I, I_sh = layers[0].H, layers[0].I, layers[0].I_sh
-    chunks = LY.split_chunks_int4(H, I)
+    bf16 = isinstance(layers[0], Bf16Layer)
+    chunks = [("w", 0, LY.bf16_expert_bytes(H, I))] if bf16 else LY.split_chunks_int4(H, I)
     m = EG.ModuleMeta(Lyr, E)
     m.init_param_list([c[0] for c in chunks])
     d = {"num_expert_per_token": str(k)}
@@ -27,7 +29,7 @@ def build_engine(layers, k, dev, mode=0, **cfg):
     m.init_from_map(d)
     m.handle_uninited_configs()
     pm = EG.PrefetchMngr(m, backend=L.BACKEND_HIP, compute_stream=torch.cuda.current_stream().cuda_stream)
-    total = LY.int4_layout(H, I)["total_bytes"]
+    total = LY.bf16_expert_bytes(H, I) if bf16 else LY.int4_layout(H, I)["total_bytes"]
     stage = EG.PinnedBuffer(total * Lyr * E)
     pm._keep.append(stage)
     for l, layer in enumerate(layers):
@@ -42,8 +44,12 @@ def build_engine(layers, k, dev, mode=0, **cfg):
         gw = torch.from_numpy(layer.wg).to(torch.bfloat16).to(dev)
         bias = None if layer.bias is None else torch.from_numpy(layer.bias).to(dev)
         sh = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
-        pm.set_layer(l, H, I, I_sh, k, mode, gw, bias, sh)
-    pm.forward_prepare(64)
+        gated = getattr(layer, "shared_gate", None) is not None
+        if gated:
+            gw = torch.cat([gw, torch.from_numpy(layer.shared_gate[None, :]).to(torch.bfloat16).to(dev)])
+        pm.set_layer(l, H, I, I_sh, k, mode, gw, bias, sh, shared_gated=gated,
+                     fmt=L.FMT_BF16 if bf16 else L.FMT_INT4_G128)
+    pm.forward_prepare(max_tokens)
     pm.launch_thread()
     return pm
 
@@ -52,7 +58,8 @@ def ref_forward(layer, x, k, mode):
     lg = O.gate_logits_ordered(x, layer.wg)
     if layer.bias is not None:
         lg = (lg + layer.bias[None, :]).astype(np.float32)
-    return O.moe_forward(x, layer.wg, layer.experts_fp32, k, mode, shared=layer.shared_fp32, logits=lg)
+    return O.moe_forward(x, layer.wg, layer.experts_fp32, k, mode, shared=layer.shared_fp32,
+                         shared_gate=getattr(layer, "shared_gate", None), logits=lg)
 
 
 @pytest.mark.parametrize("impl", ["vmm", "slab"])
@@ -146,4 +153,38 @@ def test_stepwise_hooks_on_gpu_expose_resident_parameters(cuda):
             pm.one_expert_done(0, int(e))
         pm.one_moe_layer_done(0)
     assert sum(pm.is_in_cache(0, e) for e in range(E)) == 3
+    pm.close()
+
+
+@pytest.mark.parametrize("kind", ["int4", "bf16"])
+def test_forward_prefill_sizes_through_cache(cuda, kind):
+    """Token groups of prefill size take the matrix-core kernels (bf16 layers always do);
+    experts are still fetched and evicted underneath, one launch per missed expert."""
+    print(f"case engine_forward_prefill kind={kind}", flush=True)
+    Lyr, E, k = 2, 16, 4
+    mk = Int4Layer if kind == "int4" else Bf16Layer
+    layers = [mk(H=256, I=384, E=E, I_sh=256, seed=30 + l, zipf=1.2, shared_gate=True) for l in range(Lyr)]
+    pm = build_engine(layers, k, cuda, max_tokens=512, cache_rate=0.5, cache_policy="lru")
+    sim = CO.CacheSim(Lyr, E, 6 if kind == "int4" else 1, k, cache_rate=0.5, policy="lru")
+    worst = 0.0
+    for step, T in enumerate([300, 1, 17, 512, 3, 129]):
+        for l in range(Lyr):
+            x = O.synth_acts(T, 256, seed=200 + step * Lyr + l)
+            y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            ref = ref_forward(layers[l], x, k, 0)
+            err = np.abs(y.float().cpu().numpy() - ref["out"]).max() / np.abs(ref["out"]).max()
+            worst = max(worst, err)
+            assert err <= TOL, (step, l, T, err)
+            ids = sim.report_one_layer(l, np.unique(ref["idx"]))
+            for e in ids:
+                sim.wait_expert(l, e); sim.expert_launched(l, e)
+            sim.drain()
+            pm.drain()
+            assert [e for e in range(E) if pm.is_in_cache(l, e)] == sim.resident(l), (step, l)
+    c = pm.counters()
+    print(f"  worst max-rel-err {worst:.3e}; counters {c}", flush=True)
+    for key in ("hit", "miss", "evictions"):
+        assert c[key] == sim.ctr[key], key
+    assert c["miss"] > 0
     pm.close()
