@@ -38,6 +38,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-cache-run", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (matrix-core) legs")
     return ap.parse_args()
 
 
@@ -82,6 +83,68 @@ def cpu_baseline(T, H, I, E, I_sh, k, threads):
         times.append(time.perf_counter() - t0)
     med = statistics.median(times[2:])
     return T / med, med
+
+
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 / fp16
+
+
+def prefill_leg(torch, name, T, H, E, I, k, I_sh, fmt, gated, mode, steps=20):
+    """One MoE layer forward at prefill size on the matrix-core kernels (all experts resident,
+    uniform gate): whole-layer time and the two expert GEMM launches on their own."""
+    from promoe_amd import ops, synth, layout as LY, _lib as L
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(E + (1 if gated else 0), H, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    if fmt == L.FMT_BF16:
+        img = (torch.randn(E, 3 * I * H, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+        sh = (torch.randn(3 * I_sh * H, device=dev, generator=g) * 0.02).to(torch.bfloat16) if I_sh else None
+        wbytes = E * 3 * I * H * 2 + 3 * I_sh * H * 2
+    else:
+        img = synth.random_int4_images(E, H, I, dev, g)
+        sh = synth.random_int4_images(1, H, I_sh, dev, g)[0] if I_sh else None
+        wbytes = E * LY.int4_layout(H, I)["total_bytes"] + (LY.int4_layout(H, I_sh)["total_bytes"] if I_sh else 0)
+    table = torch.tensor([img[e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev)
+    y = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    logits = torch.empty(T, wg.shape[0], dtype=torch.float32, device=dev)
+    d = ops.Dispatch(T, k, E, min(E, T * k), dev)
+    ws = None
+
+    def layer():
+        nonlocal ws
+        ops.gate_logits(x, wg, None, out=logits)
+        idx, w = ops.topk(logits, k, mode, E=E)
+        ops.dispatch(idx, E, out=d)
+        ws = ops.experts_prefill(x, d, table, sh, H, I, I_sh, fmt, ws=ws)
+        ops.combine(ws[0], ws[1], w, d.pos_of_pair, logits[:, E] if gated else None, T, H, k, out=y)
+
+    def timed(fn, n):
+        fn(); fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+
+    t_layer = timed(layer, steps)
+    assert int(ws[2].cpu()[0]) == 0
+    t_w13 = timed(lambda: ops.experts_prefill(x, d, table, sh, H, I, I_sh, fmt, phases=1, ws=ws), steps)
+    t_w2 = timed(lambda: ops.experts_prefill(x, d, table, sh, H, I, I_sh, fmt, phases=2, ws=ws), steps)
+    flops = 2.0 * T * k * 3 * I * H + 2.0 * T * 3 * I_sh * H
+    ach = flops * 2 / 3 / t_w13 / 1e12
+    return {"workload": name, "tokens": T, "tokens_per_s": T / t_layer, "ms_per_layer": t_layer * 1e3,
+            "expert_flops": flops, "weight_bytes": wbytes,
+            "layer_TFLOPs": (flops + 2.0 * T * wg.shape[0] * H) / t_layer / 1e12,
+            "roofline": {"bound": "mfma", "kernel": "k_prefill_%s<true> (w13 + SwiGLU, routed + shared in one launch)" %
+                         ("gemm" if fmt == L.FMT_BF16 else "int4"),
+                         "achieved": ach, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK_TFLOPS,
+                         "traffic": None, "avg_launch_us": t_w13 * 1e6,
+                         "algorithmic_flops_per_launch": flops * 2 / 3,
+                         "method": "%d back-to-back launches (tile-list kernel included) between one HIP event pair" % steps},
+            "w2_launch_us": t_w2 * 1e6, "w2_TFLOPs": flops / 3 / t_w2 / 1e12}
 
 
 def main():
@@ -221,6 +284,18 @@ def main():
                      "h2d_GBps": (c2["h2d_bytes"] - c0["h2d_bytes"]) / d3 / 1e9, "steps": n2}
         pm2.close()
 
+    prefill = None
+    if not a.no_prefill:
+        from promoe_amd import _lib as L
+        prefill = [
+            prefill_leg(torch, "Qwen1.5-MoE-A2.7B-shaped layer, bf16 experts, prefill T=2048, all resident",
+                        2048, 2048, 60, 1408, 4, 5632, L.FMT_BF16, True, 0),
+            prefill_leg(torch, "DeepSeek-MoE-16B-shaped layer, int4-g128 experts, prefill T=2048, all resident",
+                        2048, 2048, 64, 1408, 6, 2816, L.FMT_INT4_G128, False, 0),
+            prefill_leg(torch, "Mixtral-8x7B-shaped layer, int4-g128 experts, prefill T=4096, all resident",
+                        4096, 4096, 8, 14336, 2, 0, L.FMT_INT4_G128, False, 2, steps=5),
+        ]
+
     cpu = None
     if not a.no_cpu:
         threads = 8   # the reference's own torch.set_num_threads(8) (utils/__init__.py:343)
@@ -237,7 +312,7 @@ def main():
                       "hidden": H, "experts": E, "intermediate": I, "shared_intermediate": I_sh, "top_k": k,
                       "tokens_per_step": T, "layers": L_, "zipf": 1.2},
            "roofline": roofline, "cpu_baseline": cpu, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
-           "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run}
+           "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run, "prefill": prefill}
     print(json.dumps(out))
 
 
