@@ -188,3 +188,39 @@ def test_forward_prefill_sizes_through_cache(cuda, kind):
         assert c[key] == sim.ctr[key], key
     assert c["miss"] > 0
     pm.close()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_patched_module_mirror_matches_oracle(cuda, fused):
+    """The module-level mirror of the reference's patched MoE block: `report_experts` after
+    routing, ExpertHook around every expert launch (unfused) or one fused call."""
+    from promoe_amd.module import SparseMoeBlock
+    print(f"case module_mirror fused={fused}", flush=True)
+    Lyr, E, k = 2, 16, 4
+    layers = [Int4Layer(H=256, I=384, E=E, I_sh=256, seed=40 + l, zipf=1.2) for l in range(Lyr)]
+    pm = build_engine(layers, k, cuda, max_tokens=64, cache_rate=0.5, cache_policy="lru")
+    blocks = []
+    for l, layer in enumerate(layers):
+        gw = torch.from_numpy(layer.wg).to(torch.bfloat16).to(cuda)
+        bias = torch.from_numpy(layer.bias).to(cuda)
+        sh = torch.from_numpy(layer.shared_img).to(cuda)
+        blocks.append(SparseMoeBlock(pm, l, E, 256, 384, 256, k, 0, gw, bias, sh, fused=fused))
+    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.5, policy="lru")
+    for step, T in enumerate([1, 4, 40, 1, 16]):
+        for l in range(Lyr):
+            x = O.synth_acts(T, 256, seed=300 + step * Lyr + l)
+            y = blocks[l](torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            ref = ref_forward(layers[l], x, k, 0)
+            err = np.abs(y.float().cpu().numpy() - ref["out"]).max() / np.abs(ref["out"]).max()
+            assert err <= TOL, (step, l, T, err)
+            ids = sim.report_one_layer(l, np.unique(ref["idx"]))
+            for e in ids:
+                sim.wait_expert(l, e); sim.expert_launched(l, e)
+            sim.drain()
+            pm.drain()
+            assert [e for e in range(E) if pm.is_in_cache(l, e)] == sim.resident(l), (step, l)
+    c = pm.counters()
+    for key in ("hit", "miss", "evictions"):
+        assert c[key] == sim.ctr[key], key
+    pm.close()
