@@ -41,6 +41,11 @@ extern "C" {
                              * blocks of 32 rows x 64 k (4 KiB; block (nb,kb) at element (((nb/4)*K/64+kb)*4+nb%4)*2048,
                              * inside a block element [j][q][n][e] is W[32nb+n][64kb+32q+8j+e]) */
 
+#define MOE_FMT_Q4K 2       /* ggml q4_K information (fp16 d, dmin per 256 weights; 6-bit scale and min per
+                             * 32) repacked: nibbles in the int4 tile order, one (scale, min) byte pair per
+                             * tile lane, one (d, dmin) fp16 pair per row and super-block; see
+                             * moe_q4k_layout_make.  w = d*sc*q - dmin*m. */
+
 const char *moe_last_error(void);
 
 /*
@@ -67,6 +72,14 @@ typedef struct moe_int4_layout {
  * registered through ModelLoader::add_one_expert_param (model_loader.hpp:282-288),
  * laid end to end as ExpertMemHanlderTensorUnified does (model_loader.cpp:208-234). */
 int moe_int4_layout_make(int H, int I, moe_int4_layout *out);
+
+/* q4_K experts.  Same section order as the int4 layout (q, s, z per matrix; the struct is
+ * reused): q = nibble tiles exactly as above; s = [N/16][G][64] byte pairs (sc, m): lane l of
+ * tile (rb, g) owns row 16rb + (l&15), sub-block 4*(g&1) + (l>>4) of super-block g/2;
+ * z = [N/16][G/2][16] pairs (fp16 d, fp16 dmin).  148 bytes per 256 weights (ggml: 144).
+ * H, I multiples of 256.  Source of the format: ggml block_q4_K, which the reference reaches
+ * through its llama.cpp fork (README.md:29-34, 45-54); it holds no q4_K code of its own. */
+int moe_q4k_layout_make(int H, int I, moe_int4_layout *out);
 
 /* k1a: logits[t*ldl + e] = sum_k x[t,k]*wg[e,k] (+ bias[e]); bf16 inputs, fp32 result.
  * Summation order is fixed (64 lane partials over k = c*512 + 8*lane + i, then an
@@ -122,10 +135,18 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
                             const moe_unit *units_host, const uint64_t *expert_ptr_host,
                             int phases, void *stream);
 
+/* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only. */
+int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, int k,
+                           const moe_unit *units, int max_units, const int *sorted_tok,
+                           const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
+                           float *part_r, float *part_s, int *err, int phases, void *stream);
+
 /* k4 (prefill): grouped SwiGLU expert product on the matrix cores for large token groups.
  * Same arguments and buffer meanings as moe_experts_decode_int4 (rows of h_r / part_r in the
  * sorted pair order; expert_ptr[e] == 0 for an active expert sets *err |= 1 and skips it).
- *   fmt       : MOE_FMT_BF16 (expert image = blocked w13 [2I,H] then blocked w2 [H,I])
+ *   fmt       : MOE_FMT_BF16 (expert image = blocked w13 [2I,H] then blocked w2 [H,I]; bf16 MFMA),
+ *               MOE_FMT_INT4_G128 or MOE_FMT_Q4K (nibble tiles dequantised in registers to fp16
+ *               operands, activations converted bf16 -> fp16 on the way into LDS; tiles of 192 rows)
  *   tiles_ws  : device workspace of moe_prefill_workspace_bytes(T, k, max_units) bytes; the
  *               list of row tiles per expert is built there by a kernel, so the host
  *               needs no copy of the dispatch counts.

@@ -22,7 +22,7 @@ lib = C.CDLL(LIB_PATH)
 
 MOE_OK, MOE_EINVAL, MOE_EHIP, MOE_ESTATE, MOE_ENOMEM, MOE_ENOTRESIDENT = 0, -1, -2, -3, -4, -5
 ROUTE_SOFTMAX_TOPK, ROUTE_SOFTMAX_TOPK_RENORM, ROUTE_TOPK_SOFTMAX = 0, 1, 2
-FMT_INT4_G128, FMT_BF16 = 0, 1
+FMT_INT4_G128, FMT_BF16, FMT_Q4K = 0, 1, 2
 
 vp, i32, i64, u64 = C.c_void_p, C.c_int, C.c_int64, C.c_uint64
 
@@ -50,6 +50,8 @@ _sig("moe_topk", [vp, i32, i32, i32, i32, i32, vp, vp, vp])
 _sig("moe_dispatch", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_route_decode", [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
+_sig("moe_q4k_layout_make", [i32, i32, C.POINTER(Int4Layout)])
+_sig("moe_experts_decode_q4k", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_prefill_workspace_bytes", [i32, i32, i32], C.c_int64)
 _sig("moe_prefill_tile_rows", [])
 _sig("moe_experts_prefill", [vp, i32, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])

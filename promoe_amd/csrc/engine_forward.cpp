@@ -56,9 +56,13 @@ extern "C" int moe_set_layer(moe_engine *eng, int layer, const moe_layer_desc *d
     moe_set_error("moe_set_layer: bad descriptor (H=%d I=%d I_sh=%d k=%d)", d->H, d->I, d->I_sh, d->top_k);
     return MOE_EINVAL;
   }
-  if (d->fmt != MOE_FMT_INT4_G128 && d->fmt != MOE_FMT_BF16) { moe_set_error("moe_set_layer: weight format %d not supported by this entry point", d->fmt); return MOE_EINVAL; }
+  if (d->fmt != MOE_FMT_INT4_G128 && d->fmt != MOE_FMT_BF16 && d->fmt != MOE_FMT_Q4K) { moe_set_error("moe_set_layer: weight format %d not supported by this entry point", d->fmt); return MOE_EINVAL; }
   if (d->fmt == MOE_FMT_BF16 && (d->H % 256 || d->I % 128 || d->I_sh % 128)) {
     moe_set_error("moe_set_layer: bf16 experts need H %% 256 == 0 and I %% 128 == 0 (H=%d I=%d I_sh=%d)", d->H, d->I, d->I_sh);
+    return MOE_EINVAL;
+  }
+  if (d->fmt == MOE_FMT_Q4K && (d->H % 256 || d->I % 256 || d->I_sh % 256)) {
+    moe_set_error("moe_set_layer: q4_K experts need H and I multiples of 256 (H=%d I=%d I_sh=%d)", d->H, d->I, d->I_sh);
     return MOE_EINVAL;
   }
   eng->layer_desc[layer] = *d;
@@ -164,6 +168,10 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
     return moe_experts_prefill(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
                                s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
                                s->part_s, s->tiles_ws, s->err, 3, st);
+  if (d.fmt == MOE_FMT_Q4K)
+    return moe_experts_decode_q4k(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
+                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
+                                  s->part_r, s->part_s, s->err, 3, st);
   // the host knows the units and the slot addresses: they travel in the kernel arguments
   const uint64_t *table_host = units_host ? eng->h_table + (size_t)layer * eng->cfg.num_expert : nullptr;
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,

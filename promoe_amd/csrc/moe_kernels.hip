@@ -572,7 +572,10 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
   return wk;
 }
 
-template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS>
+// Q4K: same nibble tiles, but the scale data is per 32-wide sub-block (= one lane's k quarter):
+// section s holds (6-bit scale, 6-bit min) byte pairs [N/16][G][64 lanes], section z holds
+// (fp16 d, fp16 dmin) pairs [N/16][G/2][16 rows]; w = d*sc*q - dmin*m.
+template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false>
 __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -592,21 +595,22 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   // and the cross-wave reduction buffer
   uint16_t *xs = (uint16_t *)smem;                                    // [TMAX][K]
   float *xsum = (float *)(smem + (size_t)TMAX * K * 2);              // [TMAX][K/32]
-  uint16_t *s_sc = (uint16_t *)(xsum + (size_t)TMAX * KS);            // [2][G][16] fp16
-  unsigned char *s_zz = (unsigned char *)(s_sc + 2 * G * 16);         // [2][G][8]
-  float *red = (float *)(s_zz + 2 * G * 8);                           // [4][TMAX][2][16]
+  uint16_t *s_sc = (uint16_t *)(xsum + (size_t)TMAX * KS);            // [2][G][16] fp16 | Q4K: [2][G][64] (sc, m)
+  const int SCB = Q4K ? 128 : 32, ZZB = Q4K ? 32 : 8;                // bytes of section s / z per tile
+  unsigned char *s_zz = (unsigned char *)s_sc + 2 * G * SCB;          // [2][G][8] | Q4K: [2][G/2][16] (d, dmin)
+  float *red = (float *)(s_zz + 2 * G * ZZB);                         // [4][TMAX][2][16]
 
   const int GPW = (G - w + 3) >> 2;  // groups of this wave: g = w + 4j, j < GPW
   const int rbA = 2 * b;
   // tiles of block A then block B are contiguous: 2*G KiB
   const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, 2u * G * 1024u);
-  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, 2u * G * 32u);
-  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, 2u * G * 8u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * SCB, 2u * G * SCB);
+  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * ZZB, 2u * G * ZZB);
   const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
   const int zsh = (r & 1) * 4;
   const int vec_per_row = K >> 3;
-  const int n_sc = 2 * G * 8;   // dwords of scales
-  const int n_zz = 2 * G * 2;   // dwords of zeros
+  const int n_sc = 2 * G * SCB / 4;   // dwords of section s
+  const int n_zz = 2 * G * ZZB / 4;   // dwords of section z
   constexpr int XT = TMAX < 2 ? TMAX : 2;  // rows whose first 256 vectors are staged through registers
 
   for (int t0 = 0; t0 < m; t0 += TMAX) {
@@ -678,10 +682,21 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
         const bool valid = jc + j < GPW;
         const int g = valid ? w + 4 * (jc + j) : 0;
         // a clamped (duplicate) tile contributes through a zero scale
-        const float fsa = valid ? half_bits_to_f32(s_sc[g * 16 + r]) : 0.f;
-        const float fsb = valid ? half_bits_to_f32(s_sc[(G + g) * 16 + r]) : 0.f;
-        const float fza = 128.f + (float)((s_zz[g * 8 + (r >> 1)] >> zsh) & 15);
-        const float fzb = 128.f + (float)((s_zz[(G + g) * 8 + (r >> 1)] >> zsh) & 15);
+        float fsa, fsb, fza, fzb;  // contribution of a lane: fs * D - fz' * xq with fz' = fs * fz
+        if (Q4K) {
+          const u32 smA = s_sc[g * 64 + lane], smB = s_sc[(G + g) * 64 + lane];
+          const u32 ddA = ((const u32 *)s_zz)[(g >> 1) * 16 + r], ddB = ((const u32 *)s_zz)[((G + g) >> 1) * 16 + r];
+          fsa = valid ? half_bits_to_f32((uint16_t)ddA) * (float)(smA & 0xff) : 0.f;
+          fsb = valid ? half_bits_to_f32((uint16_t)ddB) * (float)(smB & 0xff) : 0.f;
+          // w = fs*q - dmin*m = fs*(128+q) - (128*fs + dmin*m)
+          fza = valid ? fmaf(128.f, fsa, half_bits_to_f32((uint16_t)(ddA >> 16)) * (float)(smA >> 8)) : 0.f;
+          fzb = valid ? fmaf(128.f, fsb, half_bits_to_f32((uint16_t)(ddB >> 16)) * (float)(smB >> 8)) : 0.f;
+        } else {
+          fsa = valid ? half_bits_to_f32(s_sc[g * 16 + r]) : 0.f;
+          fsb = valid ? half_bits_to_f32(s_sc[(G + g) * 16 + r]) : 0.f;
+          fza = 128.f + (float)((s_zz[g * 8 + (r >> 1)] >> zsh) & 15);
+          fzb = 128.f + (float)((s_zz[(G + g) * 8 + (r >> 1)] >> zsh) & 15);
+        }
 #pragma unroll
         for (int t = 0; t < TMAX; ++t) {
           if (t < mc) {
@@ -693,8 +708,13 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
             dA = dot8_q4(wa[j].y, x1, dA); dB = dot8_q4(wb[j].y, x1, dB);
             dA = dot8_q4(wa[j].z, x2, dA); dB = dot8_q4(wb[j].z, x2, dB);
             dA = dot8_q4(wa[j].w, x3, dA); dB = dot8_q4(wb[j].w, x3, dB);
-            accA[t] = fmaf(fsa, dA - fza * xq, accA[t]);
-            accB[t] = fmaf(fsb, dB - fzb * xq, accB[t]);
+            if (Q4K) {
+              accA[t] = fmaf(fsa, dA, fmaf(-fza, xq, accA[t]));
+              accB[t] = fmaf(fsb, dB, fmaf(-fzb, xq, accB[t]));
+            } else {
+              accA[t] = fmaf(fsa, dA - fza * xq, accA[t]);
+              accB[t] = fmaf(fsb, dB - fzb * xq, accB[t]);
+            }
           }
         }
         // keep the scheduler from hoisting the next tile's LDS reads (register pressure)
@@ -1083,6 +1103,41 @@ static int launch_gemv_c(const GemvArgs &a, int grid, int tmax, size_t lds, hipS
   }
 }
 
+static size_t gemv_q4k_lds(int tmax, int K) {
+  const size_t G = K / 128;
+  return (size_t)tmax * K * 2 + (size_t)tmax * (K / 32) * 4 + 2 * G * 128 + 2 * G * 32 +
+         (size_t)4 * tmax * 2 * 16 * 4;
+}
+
+template <bool SW, int TMAX>
+static int launch_gemv_q4k_t(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gemv_int4<TMAX, SW, 2, true, true>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                               "hipFuncSetAttribute(k_gemv_int4 q4k)"))
+      return rc;
+    attr_set = true;
+  }
+  moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
+  hipLaunchKernelGGL((k_gemv_int4<TMAX, SW, 2, true, true>), dim3(grid), dim3(256), lds, s, a);
+  moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
+  return moe_check_launch("k_gemv_int4<q4k>");
+}
+
+template <bool SW>
+static int launch_gemv_q4k(const GemvArgs &a, int grid, int T, int Kmax, hipStream_t s) {
+  int tmax = T <= 1 ? 1 : (T <= 4 ? 4 : 16);
+  while (tmax > 1 && gemv_q4k_lds(tmax, Kmax) > 150 * 1024) tmax >>= 2;
+  const size_t lds = gemv_q4k_lds(tmax, Kmax);
+  if (lds > 150 * 1024) { moe_set_error("k_gemv_int4<q4k>: K=%d does not fit LDS", Kmax); return MOE_EINVAL; }
+  switch (tmax) {
+    case 1: return launch_gemv_q4k_t<SW, 1>(a, grid, lds, s);
+    case 4: return launch_gemv_q4k_t<SW, 4>(a, grid, lds, s);
+    default: return launch_gemv_q4k_t<SW, 16>(a, grid, lds, s);
+  }
+}
+
 static size_t gemv_mfma_lds(int tb, int K) {
   const size_t G = K / 128;
   return (size_t)tb * (K * 2 + 16) + (((size_t)tb * G + 3) & ~(size_t)3) * 4 + 2 * G * 32 + 2 * G * 8 +
@@ -1222,6 +1277,63 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
     int rc = launch_gemv_t<false>(a, grid, T, I_sh > I ? I_sh : I, (max_units > 0 ? I : I_sh) / 128, s);
     if (rc) return rc;
   }
+  return MOE_OK;
+}
+
+extern "C" int moe_q4k_layout_make(int H, int I, moe_int4_layout *out) {
+  if (!out || H <= 0 || I <= 0 || H % 256 || I % 256) {
+    moe_set_error("moe_q4k_layout_make: H and I must be positive multiples of 256 (H=%d I=%d)", H, I);
+    return MOE_EINVAL;
+  }
+  const int64_t n13 = 2ll * I * H, n2 = (int64_t)H * I;
+  out->off13_q = 0;
+  out->off13_s = out->off13_q + n13 / 2;        // (sc, m) byte pairs: 2 bytes per 32 weights
+  out->off13_z = out->off13_s + n13 / 16;       // (d, dmin) fp16 pairs: 4 bytes per 256 weights
+  out->off2_q = out->off13_z + n13 / 64;
+  out->off2_s = out->off2_q + n2 / 2;
+  out->off2_z = out->off2_s + n2 / 16;
+  out->total_bytes = out->off2_z + n2 / 64;
+  return MOE_OK;
+}
+
+extern "C" int moe_experts_decode_q4k(const void *x, int T, int H, int I, int I_sh, int k,
+                                      const moe_unit *units, int max_units, const int *sorted_tok,
+                                      const uint64_t *expert_ptr, const void *shared_ptr,
+                                      void *h_r, void *h_s, float *part_r, float *part_s,
+                                      int *err, int phases, void *stream) {
+  if (!x || T <= 0 || H <= 0 || H % 256 || I < 0 || I % 256 || I_sh < 0 || I_sh % 256 || !err ||
+      (max_units > 0 && (!units || !sorted_tok || !expert_ptr || !h_r || !part_r || I == 0)) ||
+      (shared_ptr && (!h_s || !part_s || I_sh == 0))) {
+    moe_set_error("moe_experts_decode_q4k: bad argument (T=%d H=%d I=%d I_sh=%d)", T, H, I, I_sh);
+    return MOE_EINVAL;
+  }
+  (void)k;
+  moe_int4_layout lr, ls;
+  memset(&lr, 0, sizeof lr); memset(&ls, 0, sizeof ls);
+  if (max_units > 0 && moe_q4k_layout_make(H, I, &lr)) return MOE_EINVAL;
+  if (shared_ptr && moe_q4k_layout_make(H, I_sh, &ls)) return MOE_EINVAL;
+  const bool sh = shared_ptr != nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  GemvArgs a;
+  memset(&a, 0, sizeof a);
+  a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
+  a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err;
+  a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z,
+                       H, H / 128, T == 1 ? 0 : H, I_sh, I_sh / 16, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)x, T == 1 ? nullptr : sorted_tok, h_r, lr.off13_q, lr.off13_s,
+                       lr.off13_z, H, H / 128, T == 1 ? 0 : H, I, I / 16, 0};
+  a.n_sh_blocks = sh ? I_sh / 16 : 0;
+  int grid = a.n_sh_blocks + max_units * (I / 16);
+  if (grid > 0 && (phases & 1))
+    if (int rc = launch_gemv_q4k<true>(a, grid, T, H, s)) return rc;
+  a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z,
+                       I_sh, I_sh / 128, I_sh, H, H / 32, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z,
+                       I, I / 128, I, H, H / 32, 0};
+  a.n_sh_blocks = sh ? H / 32 : 0;
+  grid = a.n_sh_blocks + max_units * (H / 32);
+  if (grid > 0 && (phases & 2))
+    if (int rc = launch_gemv_q4k<false>(a, grid, T, I_sh > I ? I_sh : I, s)) return rc;
   return MOE_OK;
 }
 

@@ -256,6 +256,19 @@ static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2) {
   return (h + nz8) * s8;                                // exact difference, then one rounding
 }
 
+// q4_K flavour: w = s*q - m with the lane's own sub-block scale s = d*sc and min m = dmin*mn.
+// s2 / nm2: fp16 bit patterns of s and -m replicated in both halves.
+static __device__ __forceinline__ f16x8_t pf_deq8_q4k(u32 d, u32 s2, u32 nm2) {
+  const u32 M = 0x000f000fu, C = 0x64006400u;
+  u32x4_t v;
+  v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
+  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);
+  const f16x8_t n1024 = __builtin_bit_cast(f16x8_t, u32x4_t{0xe400e400u, 0xe400e400u, 0xe400e400u, 0xe400e400u});
+  const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
+  const f16x8_t nm8 = __builtin_bit_cast(f16x8_t, u32x4_t{nm2, nm2, nm2, nm2});
+  return (h + n1024) * s8 + nm8;  // q exact, then s*q - m
+}
+
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 // buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
 static __device__ __forceinline__ rsrc_t pf_rsrc(const void *p, unsigned bytes) {
@@ -267,9 +280,17 @@ static __device__ __forceinline__ const unsigned char *pf_uniform(const unsigned
   return (const unsigned char *)(((unsigned long long)hi << 32) | lo);
 }
 
+static __device__ __forceinline__ u32 pf_h2f(u32 hbits) {  // fp16 bits -> fp32 bits
+  const _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)hbits);
+  return __builtin_bit_cast(u32, (float)h);
+}
+static __device__ __forceinline__ u32 pf_f2h(float f) {  // fp32 -> fp16 bits (round to nearest)
+  return (u32)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
 struct PiMeta { u32 sc[4]; u32 zz[4]; };  // raw fp16 scale bits / zero nibble of the lane's row in the 4 tiles
 
-template <int NBW>
+template <int NBW, bool Q4K>
 static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_t *As, const rsrc_t rx, const u32 (&a_off)[6],
                                                    const rsrc_t rq, const rsrc_t rs, const rsrc_t rz, int G, int nb, int tid) {
   const int lane = tid & 63, g = tid >> 8;
@@ -299,8 +320,13 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       wq[t] = __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, (t * G + gi) * 1024, 0);
-      m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * r, (t * G + gi) * 32, 0);
-      m.zz[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, r >> 1, (t * G + gi) * 8, 0);
+      if (Q4K) {  // (sc, m) byte pair of the lane's sub-block; (d, dmin) of the row's super-block
+        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * lane, (t * G + gi) * 128, 0);
+        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b32(rz, 4 * r, (t * (G >> 1) + (gi >> 1)) * 64, 0);
+      } else {
+        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * r, (t * G + gi) * 32, 0);
+        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, r >> 1, (t * G + gi) * 8, 0);
+      }
     }
   };
   auto compute2 = [&](int st, const u32x4_t(&wq)[4], const PiMeta &m, int j0) {
@@ -308,17 +334,25 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
     u32 s2[4], z2[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const u32 sb = m.sc[t] & 0xffffu;
-      s2[t] = sb | (sb << 16);
-      const u32 zb = 0xe400u | ((m.zz[t] >> (4 * (r & 1))) & 15u);  // -(1024 + zero)
-      z2[t] = zb | (zb << 16);
+      if (Q4K) {
+        const float dsc = __builtin_bit_cast(float, pf_h2f(m.zz[t] & 0xffffu)) * (float)(m.sc[t] & 0xffu);
+        const float dmn = __builtin_bit_cast(float, pf_h2f(m.zz[t] >> 16)) * (float)((m.sc[t] >> 8) & 0xffu);
+        const u32 sb = pf_f2h(dsc), mb = pf_f2h(-dmn);
+        s2[t] = sb | (sb << 16);
+        z2[t] = mb | (mb << 16);
+      } else {
+        const u32 sb = m.sc[t] & 0xffffu;
+        s2[t] = sb | (sb << 16);
+        const u32 zb = 0xe400u | ((m.zz[t] >> (4 * (r & 1))) & 15u);  // -(1024 + zero)
+        z2[t] = zb | (zb << 16);
+      }
     }
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
       const int j = j0 + jj;
       f16x8_t wd[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wd[t] = pf_deq8_f16(wq[t][j], s2[t], z2[t]);
+      for (int t = 0; t < 4; ++t) wd[t] = Q4K ? pf_deq8_q4k(wq[t][j], s2[t], z2[t]) : pf_deq8_f16(wq[t][j], s2[t], z2[t]);
 #pragma unroll
       for (int tb = 0; tb < 2 * NBW; ++tb) {
         const f16x8_t xa = *(const f16x8_t *)(A_ + (64 * (tb >> 1) + 16 * (tb & 1)) * PI_LDK + 8 * j);
@@ -359,7 +393,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   }
 }
 
-template <bool SWIGLU>
+template <bool SWIGLU, bool Q4K>
 __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   extern __shared__ __align__(16) uint16_t As[];  // [2][PI_BM][PI_LDK] fp16
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane((tid >> 6) & 3), g = tid >> 8;
@@ -398,8 +432,8 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   const int rb0 = 16 * nt + 4 * w;
   const unsigned char *base = pf_uniform((const unsigned char *)tile.w_base);
   const rsrc_t rq = pf_rsrc(base + c.w_off + (size_t)rb0 * G * 1024, 4u * G * 1024u);
-  const rsrc_t rs = pf_rsrc(base + c.off_s + (size_t)rb0 * G * 32, 4u * G * 32u);
-  const rsrc_t rz = pf_rsrc(base + c.off_z + (size_t)rb0 * G * 8, 4u * G * 8u);
+  const rsrc_t rs = pf_rsrc(base + c.off_s + (size_t)rb0 * G * (Q4K ? 128 : 32), 4u * G * (Q4K ? 128u : 32u));
+  const rsrc_t rz = pf_rsrc(base + c.off_z + (size_t)rb0 * G * (Q4K ? 32 : 8), 4u * G * (Q4K ? 32u : 8u));
   const rsrc_t rx = pf_rsrc(c.act, 0x7fffffffu);
 
   f32x4_t acc[4][6];
@@ -411,10 +445,10 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   const int nb = (tile.rows + 31) >> 5;
   const int nbw = (nb - g + 1) >> 1;
   switch (nbw) {
-    case 0: pi_mainloop<0>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 1: pi_mainloop<1>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 2: pi_mainloop<2>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    default: pi_mainloop<3>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 0: pi_mainloop<0, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 1: pi_mainloop<1, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 2: pi_mainloop<2, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    default: pi_mainloop<3, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
   }
   // epilogue.  acc[t][tb] element i of lane l: weight row r of tile t, token row
   // 32*(2*(tb/2)+g) + 16*(tb%2) + 4*qd + i of the tile
@@ -447,20 +481,21 @@ static int pf_slab_step(int nk) {
   return s;
 }
 
+template <bool Q4K>
 static int pi_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
   if (a.n_blocks_total <= 0) return MOE_OK;
   const int grid = ((a.c[0].n_blocks + 7) & ~7) + ((a.c[1].n_blocks + 7) & ~7);
   const size_t lds = (size_t)2 * PI_BM * PI_LDK * 2;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)k_prefill_int4<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipError_t e2 = hipFuncSetAttribute((const void *)k_prefill_int4<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e1 = hipFuncSetAttribute((const void *)k_prefill_int4<true, Q4K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e2 = hipFuncSetAttribute((const void *)k_prefill_int4<false, Q4K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (int rc = moe_check_hip(e1 != hipSuccess ? e1 : e2, "hipFuncSetAttribute(k_prefill_int4)")) return rc;
     attr_set = true;
   }
   moe_ktimer_begin(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
-  if (swiglu) hipLaunchKernelGGL(k_prefill_int4<true>, dim3(grid), dim3(512), lds, s, a);
-  else hipLaunchKernelGGL(k_prefill_int4<false>, dim3(grid), dim3(512), lds, s, a);
+  if (swiglu) hipLaunchKernelGGL((k_prefill_int4<true, Q4K>), dim3(grid), dim3(512), lds, s, a);
+  else hipLaunchKernelGGL((k_prefill_int4<false, Q4K>), dim3(grid), dim3(512), lds, s, a);
   moe_ktimer_end(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
   return moe_check_launch("k_prefill_int4");
 }
@@ -565,11 +600,16 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
     moe_set_error("moe_experts_prefill: NULL or negative argument");
     return MOE_EINVAL;
   }
-  if (fmt != MOE_FMT_BF16 && fmt != MOE_FMT_INT4_G128) {
+  if (fmt != MOE_FMT_BF16 && fmt != MOE_FMT_INT4_G128 && fmt != MOE_FMT_Q4K) {
     moe_set_error("moe_experts_prefill: weight format %d not supported by the prefill kernels", fmt);
     return MOE_EINVAL;
   }
-  const bool int4 = fmt == MOE_FMT_INT4_G128;
+  const bool q4k = fmt == MOE_FMT_Q4K;
+  const bool int4 = fmt == MOE_FMT_INT4_G128 || q4k;  // nibble tiles + fp16 operands
+  if (q4k && (H % 256 || I % 256 || (shared_ptr && I_sh % 256))) {
+    moe_set_error("moe_experts_prefill: q4_K experts need H, I multiples of 256 (H=%d I=%d I_sh=%d)", H, I, I_sh);
+    return MOE_EINVAL;
+  }
   {
     const long long widest = I > H ? I : H, rows = (long long)T * (k > 1 ? k : 1);
     if (int4 && (rows * widest * 2 >= (1ll << 31) || (shared_ptr && (long long)T * (I_sh > H ? I_sh : H) * 2 >= (1ll << 31)))) {
@@ -618,7 +658,7 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
       }
       if (int4) {
         moe_int4_layout lay;
-        if (int rc = moe_int4_layout_make(H, Ii, &lay)) return rc;
+        if (int rc = q4k ? moe_q4k_layout_make(H, Ii, &lay) : moe_int4_layout_make(H, Ii, &lay)) return rc;
         c.w_off = w2 ? lay.off2_q : lay.off13_q;
         c.off_s = w2 ? lay.off2_s : lay.off13_s;
         c.off_z = w2 ? lay.off2_z : lay.off13_z;
@@ -627,7 +667,7 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
       c.slab_step = pf_slab_step(c.K / PF_BK);
       a.n_blocks_total += c.n_blocks;
     }
-    if (int rc = int4 ? pi_launch(!w2, a, s) : pf_launch(!w2, a, s)) return rc;
+    if (int rc = q4k ? pi_launch<true>(!w2, a, s) : (int4 ? pi_launch<false>(!w2, a, s) : pf_launch(!w2, a, s))) return rc;
   }
   return MOE_OK;
 }

@@ -140,3 +140,74 @@ def pack_expert_bf16(gate_bits, up_bits, down_bits) -> np.ndarray:
 
 def bf16_expert_bytes(H: int, I: int) -> int:
     return 3 * I * H * 2
+
+
+# ---- q4_K experts -------------------------------------------------------------------
+# The information of ggml's block_q4_K (fp16 d and dmin per 256 weights, a 6-bit scale and
+# min per 32-wide sub-block, 4-bit quants) in the tile order of the int4 kernels: nibble
+# tiles as in tile_int4; section s = [N/16][G][64] byte pairs (sc, m), lane l = 16*qd + r of
+# tile (rb, g) holding row 16rb + r, sub-block 4*(g&1) + qd of super-block g//2; section z =
+# [N/16][G/2][16] pairs (fp16 d, fp16 dmin).
+
+def q4k_layout(H: int, I: int) -> dict:
+    from ._lib import lib, Int4Layout, check
+    import ctypes as C
+    out = Int4Layout()
+    check(lib.moe_q4k_layout_make(H, I, C.byref(out)), "moe_q4k_layout_make")
+    return {n: int(getattr(out, n)) for n, _ in Int4Layout._fields_}
+
+
+def _q4k_fields(blocks: np.ndarray, N: int, K: int):
+    """ggml blocks uint8 [N, K/256, 144] -> q [N,K] (0..15), sc, mn [N, K/32] (0..63), d, dmin fp16 [N, K/256]."""
+    b = np.asarray(blocks, np.uint8).reshape(N, K // 256, 144)
+    d = b[:, :, 0:2].copy().view(np.float16)[:, :, 0]
+    dmin = b[:, :, 2:4].copy().view(np.float16)[:, :, 0]
+    s = b[:, :, 4:16].astype(np.int32)
+    sc = np.zeros(s.shape[:2] + (8,), np.int32)
+    mn = np.zeros_like(sc)
+    for j in range(8):
+        if j < 4:
+            sc[:, :, j] = s[:, :, j] & 63
+            mn[:, :, j] = s[:, :, j + 4] & 63
+        else:
+            sc[:, :, j] = (s[:, :, j + 4] & 0xF) | ((s[:, :, j - 4] >> 6) << 4)
+            mn[:, :, j] = (s[:, :, j + 4] >> 4) | ((s[:, :, j] >> 6) << 4)
+    qs = b[:, :, 16:144].reshape(N, K // 256, 4, 32)
+    q = np.stack([qs & 0xF, qs >> 4], axis=3).reshape(N, K)   # chunk c: low nibbles then high nibbles
+    return q.astype(np.uint32), sc.reshape(N, K // 32), mn.reshape(N, K // 32), d, dmin
+
+
+def tile_q4k(blocks: np.ndarray, N: int, K: int):
+    """One matrix of ggml q4_K blocks -> (q tiles, s section, z section) as uint8 arrays."""
+    assert N % 16 == 0 and K % 256 == 0
+    G = K // GROUP
+    q, sc, mn, d, dmin = _q4k_fields(blocks, N, K)
+    q6 = q.reshape(N // 16, 16, G, 4, 4, 8)
+    dw = np.zeros(q6.shape[:-1], np.uint32)
+    for i in range(8):
+        dw |= q6[..., i] << _NIB_SHIFT[i]
+    qt = np.ascontiguousarray(dw.transpose(0, 2, 3, 1, 4)).view(np.uint8).reshape(-1)   # [rb, g, qd, r, j]
+    pair = (sc.astype(np.uint16) | (mn.astype(np.uint16) << 8)).reshape(N // 16, 16, G, 4)  # [rb, r, g, qd]
+    st = np.ascontiguousarray(pair.transpose(0, 2, 3, 1)).view(np.uint8).reshape(-1)         # [rb, g, qd, r]
+    dd = (d.view(np.uint16).astype(np.uint32) | (dmin.view(np.uint16).astype(np.uint32) << 16))
+    zt = np.ascontiguousarray(dd.reshape(N // 16, 16, G // 2).transpose(0, 2, 1)).view(np.uint8).reshape(-1)
+    return qt, st, zt
+
+
+def pack_expert_q4k(gate_blocks, up_blocks, down_blocks, H: int, I: int) -> np.ndarray:
+    """Slot image of one q4_K expert from its three matrices in ggml block form
+    ([I, H/256, 144], [I, H/256, 144], [H, I/256, 144])."""
+    lay = q4k_layout(H, I)
+    g = np.asarray(gate_blocks, np.uint8).reshape(I, H // 256, 144)
+    u = np.asarray(up_blocks, np.uint8).reshape(I, H // 256, 144)
+    # gate / up rows interleaved in 16-row blocks, as in the int4 layout
+    w13 = np.stack([g.reshape(I // 16, 16, H // 256, 144), u.reshape(I // 16, 16, H // 256, 144)], axis=1)
+    w13 = w13.reshape(2 * I, H // 256, 144)
+    buf = np.zeros(lay["total_bytes"], np.uint8)
+    q13, s13, z13 = tile_q4k(w13, 2 * I, H)
+    q2, s2, z2 = tile_q4k(down_blocks, H, I)
+    for off, arr in ((lay["off13_q"], q13), (lay["off13_s"], s13), (lay["off13_z"], z13),
+                     (lay["off2_q"], q2), (lay["off2_s"], s2), (lay["off2_z"], z2)):
+        buf[off: off + arr.size] = arr
+    assert lay["off2_z"] + z2.size == lay["total_bytes"]
+    return buf

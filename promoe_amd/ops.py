@@ -109,6 +109,29 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
     return part_r, part_s, err, h_r, h_s
 
 
+def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
+                       H: int, I: int, I_sh: int, phases: int = 3, ws=None):
+    """q4_K flavour of experts_decode_int4 (device-side unit list)."""
+    T, k = d.T, d.k
+    P = T * k
+    dev = x.device
+    if ws is not None:
+        part_r, part_s, err, h_r, h_s = ws
+    else:
+        h_r = torch.empty(max(P, 1), max(I, 1), dtype=torch.bfloat16, device=dev)
+        part_r = torch.empty(max(P, 1), H, dtype=torch.float32, device=dev)
+        h_s = part_s = None
+        if shared is not None:
+            h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
+            part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+        err = torch.zeros(1, dtype=torch.int32, device=dev)
+    check(lib.moe_experts_decode_q4k(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
+                                     ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
+                                     ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
+                                     ptr(err), phases, cur_stream()), "moe_experts_decode_q4k")
+    return part_r, part_s, err, h_r, h_s
+
+
 def experts_prefill(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
                     H: int, I: int, I_sh: int, fmt: int = L.FMT_BF16, phases: int = 3, ws=None):
     """MFMA grouped expert product.  Returns (part_r, part_s, err, h_r, h_s, tiles)."""

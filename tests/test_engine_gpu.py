@@ -9,7 +9,7 @@ from oracle import cache_oracle as CO
 from promoe_amd import _lib as L
 from promoe_amd import engine as EG
 from promoe_amd import layout as LY
-from tests.synth import Int4Layer, Bf16Layer
+from tests.synth import Int4Layer, Bf16Layer, Q4KLayer
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
@@ -20,8 +20,10 @@ def build_engine(layers, k, dev, mode=0, max_tokens=64, **cfg):
     bf16) and start the engine."""
     Lyr, E = len(layers), layers[0].E
     H, I, I_sh = layers[0].H, layers[0].I, layers[0].I_sh
-    bf16 = isinstance(layers[0], Bf16Layer)
-    chunks = [("w", 0, LY.bf16_expert_bytes(H, I))] if bf16 else LY.split_chunks_int4(H, I)
+    bf16, q4k = isinstance(layers[0], Bf16Layer), isinstance(layers[0], Q4KLayer)
+    total = (LY.bf16_expert_bytes(H, I) if bf16 else LY.q4k_layout(H, I)["total_bytes"] if q4k
+             else LY.int4_layout(H, I)["total_bytes"])
+    chunks = [("w", 0, total)] if (bf16 or q4k) else LY.split_chunks_int4(H, I)
     m = EG.ModuleMeta(Lyr, E)
     m.init_param_list([c[0] for c in chunks])
     d = {"num_expert_per_token": str(k)}
@@ -29,7 +31,6 @@ def build_engine(layers, k, dev, mode=0, max_tokens=64, **cfg):
     m.init_from_map(d)
     m.handle_uninited_configs()
     pm = EG.PrefetchMngr(m, backend=L.BACKEND_HIP, compute_stream=torch.cuda.current_stream().cuda_stream)
-    total = LY.bf16_expert_bytes(H, I) if bf16 else LY.int4_layout(H, I)["total_bytes"]
     stage = EG.PinnedBuffer(total * Lyr * E)
     pm._keep.append(stage)
     for l, layer in enumerate(layers):
@@ -48,7 +49,7 @@ def build_engine(layers, k, dev, mode=0, max_tokens=64, **cfg):
         if gated:
             gw = torch.cat([gw, torch.from_numpy(layer.shared_gate[None, :]).to(torch.bfloat16).to(dev)])
         pm.set_layer(l, H, I, I_sh, k, mode, gw, bias, sh, shared_gated=gated,
-                     fmt=L.FMT_BF16 if bf16 else L.FMT_INT4_G128)
+                     fmt=L.FMT_BF16 if bf16 else (L.FMT_Q4K if q4k else L.FMT_INT4_G128))
     pm.forward_prepare(max_tokens)
     pm.launch_thread()
     return pm
@@ -156,14 +157,15 @@ def test_stepwise_hooks_on_gpu_expose_resident_parameters(cuda):
     pm.close()
 
 
-@pytest.mark.parametrize("kind", ["int4", "bf16"])
+@pytest.mark.parametrize("kind", ["int4", "bf16", "q4k"])
 def test_forward_prefill_sizes_through_cache(cuda, kind):
     """Token groups of prefill size take the matrix-core kernels (bf16 layers always do);
     experts are still fetched and evicted underneath, one launch per missed expert."""
     print(f"case engine_forward_prefill kind={kind}", flush=True)
     Lyr, E, k = 2, 16, 4
-    mk = Int4Layer if kind == "int4" else Bf16Layer
-    layers = [mk(H=256, I=384, E=E, I_sh=256, seed=30 + l, zipf=1.2, shared_gate=True) for l in range(Lyr)]
+    mk = {"int4": Int4Layer, "bf16": Bf16Layer, "q4k": Q4KLayer}[kind]
+    layers = [mk(H=256, I=512 if kind == "q4k" else 384, E=E, I_sh=256, seed=30 + l, zipf=1.2, shared_gate=True)
+              for l in range(Lyr)]
     pm = build_engine(layers, k, cuda, max_tokens=512, cache_rate=0.5, cache_policy="lru")
     sim = CO.CacheSim(Lyr, E, 6 if kind == "int4" else 1, k, cache_rate=0.5, policy="lru")
     worst = 0.0

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from tests.synth import Int4Layer
+from tests.synth import Int4Layer, Q4KLayer
 
 pytestmark = pytest.mark.gpu
 
@@ -97,7 +97,10 @@ def run_layer_gpu(layer, x, k, mode, dev, resident=None, host_units=False):
     table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
                           for e in range(E)], dtype=torch.int64, device=dev)
     shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
-    part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh, host_units=host_units)
+    if isinstance(layer, Q4KLayer):
+        part_r, part_s, err, h_r, h_s = ops.experts_decode_q4k(xd, d, table, shared, H, I, I_sh)
+    else:
+        part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh, host_units=host_units)
     sg = logits[:, E] if layer.shared_gate is not None else None
     y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
     torch.cuda.synchronize()
@@ -181,3 +184,18 @@ def test_fused_route_equals_separate_kernels(cuda, T, H, E, k, mode, extra):
     for name in ("sorted_pair", "pos_of_pair", "sorted_tok"):
         assert torch.equal(getattr(d, name)[:P], getattr(d_ref, name)[:P]), name
     assert torch.equal(d.units, d_ref.units) and torch.equal(d.active_ids, d_ref.active_ids)
+
+
+@pytest.mark.parametrize("T", [1, 3, 4, 16, 21])
+def test_decode_q4k_layer_small(cuda, T):
+    print(f"case decode_q4k_small T={T}", flush=True)
+    check_layer(Q4KLayer(H=256, I=512, E=8, I_sh=256, seed=3), T, 2, 0, cuda)
+
+
+def test_decode_q4k_qwen2_shape(cuda):
+    print("case decode_q4k_qwen2", flush=True)
+    # Qwen2-57B-A14B layer shape (H 3584, I 2560, sigmoid-gated shared expert), fewer experts and a
+    # smaller shared expert than the model to keep host-side quantisation short
+    layer = Q4KLayer(H=3584, I=2560, E=8, I_sh=5120, seed=1, shared_gate=True, zipf=1.1)
+    for T in (1, 3):
+        check_layer(layer, T, 4, 0, cuda)

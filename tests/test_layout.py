@@ -68,3 +68,34 @@ def test_product_quantizer_matches_oracle_quantizer():
     pw, ps, pz = quantize_int4(torch.from_numpy(w))
     assert np.array_equal(ps.view(np.uint16), s.view(np.uint16))
     assert np.array_equal(pw, qw) and np.array_equal(pz, qz)
+
+
+def test_q4k_repack_keeps_every_field():
+    """The q4_K slot image holds the same numbers as the ggml blocks: dequantising from the
+    repacked sections reproduces the oracle's dequantisation bit for bit."""
+    import numpy as np
+    from oracle import moe_oracle as O
+    from promoe_amd import layout as LY
+    rng = np.random.default_rng(0)
+    N, K = 32, 512
+    blocks = O.quantize_q4k(rng.normal(0, 0.02, (N, K)).astype(np.float32))
+    ref = O.dequant_q4k(blocks, N, K)
+    qt, st, zt = LY.tile_q4k(blocks, N, K)
+    G = K // 128
+    dw = qt.view(np.uint32).reshape(N // 16, G, 4, 16, 4)          # [rb, g, qd, r, j]
+    sm = st.view(np.uint16).reshape(N // 16, G, 4, 16)             # [rb, g, qd, r]
+    dd = zt.view(np.uint32).reshape(N // 16, G // 2, 16)           # [rb, sb, r]
+    out = np.zeros((N, K), np.float32)
+    shift = [0, 16, 4, 20, 8, 24, 12, 28]
+    for rb in range(N // 16):
+        for g in range(G):
+            for qd in range(4):
+                for r in range(16):
+                    d = np.array([dd[rb, g // 2, r] & 0xffff], np.uint16).view(np.float16)[0].astype(np.float32)
+                    dmin = np.array([dd[rb, g // 2, r] >> 16], np.uint16).view(np.float16)[0].astype(np.float32)
+                    sc, mn = np.float32(sm[rb, g, qd, r] & 0xff), np.float32(sm[rb, g, qd, r] >> 8)
+                    for j in range(4):
+                        for i in range(8):
+                            q = np.float32((dw[rb, g, qd, r, j] >> np.uint32(shift[i])) & np.uint32(15))
+                            out[16 * rb + r, 128 * g + 32 * qd + 8 * j + i] = d * sc * q - dmin * mn
+    assert np.array_equal(out, ref)

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from tests.synth import Bf16Layer, Int4Layer
+from tests.synth import Bf16Layer, Int4Layer, Q4KLayer
 
 pytestmark = pytest.mark.gpu
 
@@ -33,7 +33,7 @@ def run_prefill_gpu(layer, x, k, mode, dev, resident=None):
     table = torch.tensor([0 if (resident is not None and e not in resident) else slots[e].data_ptr()
                           for e in range(E)], dtype=torch.int64, device=dev)
     shared = torch.from_numpy(layer.shared_img).to(dev) if I_sh else None
-    fmt = L.FMT_BF16 if isinstance(layer, Bf16Layer) else L.FMT_INT4_G128
+    fmt = L.FMT_BF16 if isinstance(layer, Bf16Layer) else (L.FMT_Q4K if isinstance(layer, Q4KLayer) else L.FMT_INT4_G128)
     part_r, part_s, err, h_r, h_s, _ = ops.experts_prefill(xd, d, table, shared, H, I, I_sh, fmt)
     sg = logits[:, E] if layer.shared_gate is not None else None
     y = ops.combine(part_r, part_s, w, d.pos_of_pair, sg, T, H, k)
@@ -117,3 +117,17 @@ def test_prefill_int4_deepseek_shape(cuda):
     # DeepSeek-MoE-16B layer shape; 16 experts instead of 64 keeps host-side quantisation short
     layer = Int4Layer(H=2048, I=1408, E=16, I_sh=2816, seed=0, zipf=1.2)
     check_prefill(layer, 512, 6, 0, cuda)
+
+
+# ---- q4_K experts ----
+
+@pytest.mark.parametrize("T", [1, 17, 97, 193, 400])
+def test_prefill_q4k_layer_small(cuda, T):
+    print(f"case prefill_q4k_small T={T}", flush=True)
+    check_prefill(Q4KLayer(H=256, I=512, E=8, I_sh=256, seed=3), T, 2, 0, cuda)
+
+
+def test_prefill_q4k_variants(cuda):
+    print("case prefill_q4k_variants", flush=True)
+    check_prefill(Q4KLayer(H=512, I=256, E=8, I_sh=0, seed=4), 200, 2, 2, cuda)
+    check_prefill(Q4KLayer(H=256, I=256, E=60, I_sh=512, seed=5, shared_gate=True, zipf=1.1), 515, 8, 0, cuda)
