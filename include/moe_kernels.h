@@ -109,14 +109,16 @@ int moe_dispatch(const int *idx, int T, int k, int E, int *counts, int *offsets,
                  int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
                  int64_t *active_ids, int max_units, void *stream);
 
-/* k1a+k1b+k2 in one launch for decode batches (T <= 16, E <= 256): same results, bit for
- * bit, as moe_gate_logits + moe_topk + moe_dispatch.  E_rows = E, or E+1 when row E of
- * wg is the shared expert's gate vector (its logit lands in logits[t*ldl + E], no bias). */
+/* k1a+k1b+k2 in one launch for decode batches (T <= 16, E <= 256, T*k <= 512): same results,
+ * bit for bit, as moe_gate_logits + moe_topk + moe_dispatch.  E_rows = E, or E+1 when row E of
+ * wg is the shared expert's gate vector (its logit lands in logits[t*ldl + E], no bias).
+ * counter: one device word, zero before the first call; the workgroup that finishes its
+ * logits last runs the routing and leaves the word zero again. */
 int moe_route_decode(const void *x_bf16, const void *wg_bf16, const float *bias, float *logits,
                      int T, int H, int E, int E_rows, int ldl, int k, int mode, int *idx, float *w,
                      int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                      moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
-                     void *stream);
+                     unsigned *counter, void *stream);
 
 /* k3 (decode): int4 grouped SwiGLU expert product through the slot table.
  *   expert_ptr[e] : device address of expert e's slot (0 = not resident -> *err |= 1)

@@ -241,118 +241,79 @@ __global__ __launch_bounds__(DISP_THREADS) void k_dispatch(
 }
 
 // ---------------------------------------------------------------------------
-// k1+k2 fused for decode batches (T <= 16): one workgroup of 16 waves computes the gate
-// logits (same fixed summation order as k_gate_logits, so the same bits), the top-k
-// routing (wave t = token t) and the stable dispatch, with the logits and indices
-// staying in LDS between the phases.  Three launches become one.
+// k1+k2 fused for decode batches (T <= 16, E <= 256, T*k <= 512): the grid of k_gate_logits
+// computes the logits (same arithmetic, same bits); the workgroup that finishes last (a
+// device-scope counter tells it) then runs the top-k routing (one wave per token) and the
+// stable dispatch on its own.  Three launches become one, and the logits are still spread
+// over as many workgroups as before.  The counter must be zero at launch and is left zero.
 // ---------------------------------------------------------------------------
 #define ROUTE_MAXT 16
+#define ROUTE_MAXP 512
 struct RouteArgs {
   const uint16_t *x, *wg;
   const float *bias;
-  float *logits;  // [T, ldl]
+  float *logits;
   int T, H, E, Erows, ldl, k, mode, nbits, max_units;
   int *idx; float *w;
   int *counts, *offsets, *sorted_pair, *pos_of_pair, *sorted_tok;
   moe_unit *units; int *n_active; long long *active_ids;
+  unsigned *counter;
 };
 
-template <int TR>
-__global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
-  extern __shared__ __align__(16) unsigned char rsm[];
+__global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
+  __shared__ int s_last;
+  __shared__ int s_idx[ROUTE_MAXP];
+  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[4 * 256];
+  __shared__ int s_wsum[4], s_wact[4], s_tot;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int T = a.T, H = a.H, E = a.E, k = a.k, P = T * k;
-  uint16_t *xs = (uint16_t *)rsm;                              // [T][H]
-  float *s_lg = (float *)(rsm + (size_t)T * H * 2);            // [T][ldl]
-  int *s_idx = (int *)(s_lg + (size_t)T * a.ldl);              // [P]
-  int *s_cnt = s_idx + ((P + 3) & ~3);                         // [E]
-  int *s_off = s_cnt + E;                                      // [E+1]
-  int *s_ws = s_off + E + 1;                                   // [16][E] per-wave counts
-  int *s_misc = s_ws + 16 * E;                                 // [34]
-
-  // ---- gate logits: wave w takes rows w, w+16, ...; the (row, 512-wide chunk) pieces of the
-  // gate matrix are fetched 16 at a time, the first batch before x is staged -------------------
-  const int chunks = (H + 511) >> 9;
-  const int nrows_w = (a.Erows - w + 15) >> 4;
-  const int npieces = nrows_w * chunks;
-  constexpr int NB = 8;
-  uint4 wv[NB];
-  auto load_batch = [&](int pb) {
-#pragma unroll
-    for (int q = 0; q < NB; ++q) {
-      int pi = pb + q;
-      pi = pi < npieces ? pi : (npieces > 0 ? npieces - 1 : 0);
-      const int ri = pi / chunks, ch = pi - ri * chunks;
-      int e = w + 16 * ri;
-      e = e < a.Erows ? e : 0;
-      const int kk = ch * 512 + 8 * lane;
-      wv[q] = *(const uint4 *)(a.wg + (size_t)e * H + (kk < H ? kk : 0));
-    }
-  };
-  load_batch(0);
-  const int nvec = T * (H >> 3);
-  for (int i = tid; i < nvec; i += 1024) ((uint4 *)xs)[i] = ((const uint4 *)a.x)[i];
-  for (int e = tid; e < E; e += 1024) s_cnt[e] = 0;
-  __syncthreads();
+  const int H = a.H, E = a.E, T = a.T, k = a.k, P = T * k;
+  // ---- phase 1: one wave per (token, gate row) ------------------------------------------
   {
-    float acc[TR];
-#pragma unroll
-    for (int t = 0; t < TR; ++t) acc[t] = 0.f;
-    for (int pb = 0; pb < npieces; pb += NB) {
-      if (pb > 0) load_batch(pb);
-#pragma unroll
-      for (int q = 0; q < NB; ++q) {
-        const int pi = pb + q;
-        if (pi < npieces) {
-          const int ri = pi / chunks, ch = pi - ri * chunks;
-          const int e = w + 16 * ri;
-          const int kk = ch * 512 + 8 * lane;
-          if (kk < H) {
-#pragma unroll
-            for (int t = 0; t < TR; ++t) {
-              if (t < T) {
-                const uint4 xv = *(const uint4 *)(xs + (size_t)t * H + kk);
-                float v = acc[t];
-                v = fmaf(bf16lo(xv.x), bf16lo(wv[q].x), v); v = fmaf(bf16hi(xv.x), bf16hi(wv[q].x), v);
-                v = fmaf(bf16lo(xv.y), bf16lo(wv[q].y), v); v = fmaf(bf16hi(xv.y), bf16hi(wv[q].y), v);
-                v = fmaf(bf16lo(xv.z), bf16lo(wv[q].z), v); v = fmaf(bf16hi(xv.z), bf16hi(wv[q].z), v);
-                v = fmaf(bf16lo(xv.w), bf16lo(wv[q].w), v); v = fmaf(bf16hi(xv.w), bf16hi(wv[q].w), v);
-                acc[t] = v;
-              }
-            }
-          }
-          if (ch == chunks - 1) {  // row complete: butterfly, bias, store, reset
-            const bool biased = a.bias && e < E;
-            const float be = biased ? a.bias[e] : 0.f;
-#pragma unroll
-            for (int t = 0; t < TR; ++t) {
-              if (t < T) {
-                float v = acc[t];
-#pragma unroll
-                for (int m = 32; m >= 1; m >>= 1) v = v + __shfl_xor(v, m, 64);
-                if (lane == 0) {
-                  const float lg = biased ? v + be : v;
-                  s_lg[t * a.ldl + e] = lg;
-                  a.logits[(size_t)t * a.ldl + e] = lg;
-                }
-              }
-              acc[t] = 0.f;
-            }
-          }
+    const int e = blockIdx.x * 4 + w, t = blockIdx.y;
+    if (e < a.Erows) {
+      const uint16_t *xr = a.x + (size_t)t * H;
+      const uint16_t *wr = a.wg + (size_t)e * H;
+      float acc = 0.f;
+      for (int c = 0; c < H; c += 512) {
+        const int kk = c + 8 * lane;
+        if (kk < H) {
+          const uint4 xv = *(const uint4 *)(xr + kk);
+          const uint4 wv = *(const uint4 *)(wr + kk);
+          acc = fmaf(bf16lo(xv.x), bf16lo(wv.x), acc);
+          acc = fmaf(bf16hi(xv.x), bf16hi(wv.x), acc);
+          acc = fmaf(bf16lo(xv.y), bf16lo(wv.y), acc);
+          acc = fmaf(bf16hi(xv.y), bf16hi(wv.y), acc);
+          acc = fmaf(bf16lo(xv.z), bf16lo(wv.z), acc);
+          acc = fmaf(bf16hi(xv.z), bf16hi(wv.z), acc);
+          acc = fmaf(bf16lo(xv.w), bf16lo(wv.w), acc);
+          acc = fmaf(bf16hi(xv.w), bf16hi(wv.w), acc);
         }
       }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
+      if (lane == 0) a.logits[(size_t)t * a.ldl + e] = (a.bias && e < E) ? acc + a.bias[e] : acc;
     }
   }
+  // ---- who is last? ------------------------------------------------------------------------
+  __threadfence();
   __syncthreads();
-  // ---- top-k: wave t = token t ----------------------------------------------------------
-  if (w < T) {
-    const int t = w;
-    const float NEG = -__builtin_inff();
+  if (tid == 0) {
+    const unsigned prev = atomicAdd(a.counter, 1u);
+    s_last = prev == gridDim.x * gridDim.y - 1u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  if (tid == 0) atomicExch(a.counter, 0u);
+  __threadfence();
+  // ---- phase 2: top-k, wave w takes tokens w, w+4, ... (body of k_topk) ----------------------
+  const float NEG = -__builtin_inff();
+  for (int t = w; t < T; t += 4) {
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int e = lane + 64 * r;
-      v[r] = (e < E) ? s_lg[t * a.ldl + e] : NEG;
+      // written by other workgroups of this launch: read at device scope, past the L1
+      v[r] = (e < E) ? __hip_atomic_load(a.logits + (size_t)t * a.ldl + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : NEG;
     }
     float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
 #pragma unroll
@@ -368,8 +329,9 @@ __global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
       float bv = v[0];
       int bi = lane;
 #pragma unroll
-      for (int r = 1; r < 4; ++r)
+      for (int r = 1; r < 4; ++r) {
         if (v[r] > bv) { bv = v[r]; bi = lane + 64 * r; }
+      }
 #pragma unroll
       for (int m = 32; m >= 1; m >>= 1) {
         const float ov = __shfl_xor(bv, m, 64);
@@ -385,19 +347,18 @@ __global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
     }
     const float ex = expf(sel_v - mx);
     float wgt;
-    if (a.mode == MOE_ROUTE_TOPK_SOFTMAX) wgt = ex / sum_sel;
-    else {
+    if (a.mode == MOE_ROUTE_TOPK_SOFTMAX) {
+      wgt = ex / sum_sel;
+    } else {
       wgt = ex / den;
       if (a.mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
     }
     if (lane < k) a.w[(size_t)t * k + lane] = wgt;
   }
+  // ---- phase 3: dispatch (k_dispatch with 256 threads; thread e owns expert e) -------------
+  if (tid < E) { s_cnt[tid] = 0; s_run[tid] = 0; }
   __syncthreads();
-  // ---- dispatch: P <= 1024 pairs, one chunk ----------------------------------------------
-  const int p = tid;
-  const int e_p = p < P ? s_idx[p] : -1;
-  const bool valid = (unsigned)e_p < (unsigned)E;
-  if (valid) atomicAdd(&s_cnt[e_p], 1);
+  for (int p = tid; p < P; p += 256) atomicAdd(&s_cnt[s_idx[p]], 1);
   __syncthreads();
   {
     const int c = (tid < E) ? s_cnt[tid] : 0;
@@ -408,59 +369,67 @@ __global__ __launch_bounds__(1024) void k_route_decode(const RouteArgs a) {
       const int oc = __shfl_up(sc, d, 64), oa = __shfl_up(sa, d, 64);
       if (lane >= d) { sc += oc; sa += oa; }
     }
-    if (lane == 63) { s_misc[w] = sc; s_misc[16 + w] = sa; }
+    if (lane == 63) { s_wsum[w] = sc; s_wact[w] = sa; }
     __syncthreads();
     int bc = 0, ba = 0;
-    for (int i = 0; i < w; ++i) { bc += s_misc[i]; ba += s_misc[16 + i]; }
+    for (int i = 0; i < w; ++i) { bc += s_wsum[i]; ba += s_wact[i]; }
     const int excl = bc + sc - c, uidx = ba + sa - act;
     if (tid < E) {
       s_off[tid] = excl;
       a.counts[tid] = c;
       a.offsets[tid] = excl;
       if (act && uidx < a.max_units) {
-        moe_unit uu; uu.expert = tid; uu.m = c; uu.row0 = excl; uu.pad = 0;
-        a.units[uidx] = uu;
+        moe_unit u; u.expert = tid; u.m = c; u.row0 = excl; u.pad = 0;
+        a.units[uidx] = u;
         a.active_ids[uidx] = tid;
       }
     }
-    if (tid == 1023) {
+    if (tid == 255) {
       const int tot_act = ba + sa;
       a.offsets[E] = bc + sc;
       *a.n_active = tot_act < a.max_units ? tot_act : a.max_units;
-      s_misc[32] = tot_act;
+      s_tot = tot_act;
     }
     __syncthreads();
-    for (int uu = s_misc[32] + tid; uu < a.max_units; uu += 1024) {
+    for (int u = s_tot + tid; u < a.max_units; u += 256) {
       moe_unit z; z.expert = -1; z.m = 0; z.row0 = 0; z.pad = 0;
-      a.units[uu] = z;
-      a.active_ids[uu] = -1;
-    }
-  }
-  for (int i = tid; i < 16 * E; i += 1024) s_ws[i] = 0;
-  __syncthreads();
-  unsigned long long peers = __ballot(valid);
-  for (int bb = 0; bb < a.nbits; ++bb) {
-    const bool bit = (e_p >> bb) & 1;
-    const unsigned long long bal = __ballot(valid && bit);
-    peers &= bit ? bal : ~bal;
-  }
-  const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-  if (valid && rank == 0) s_ws[w * E + e_p] = __popcll(peers);
-  __syncthreads();
-  for (int ee = tid; ee < E; ee += 1024) {
-    int run = 0;
-    for (int ww = 0; ww < 16; ++ww) {
-      const int c = s_ws[ww * E + ee];
-      s_ws[ww * E + ee] = run;
-      run += c;
+      a.units[u] = z;
+      a.active_ids[u] = -1;
     }
   }
   __syncthreads();
-  if (valid) {
-    const int pos = s_off[e_p] + s_ws[w * E + e_p] + rank;
-    a.sorted_pair[pos] = p;
-    a.pos_of_pair[p] = pos;
-    a.sorted_tok[pos] = p / k;
+  for (int base = 0; base < P; base += 256) {
+    for (int i = tid; i < 4 * E; i += 256) s_w[i] = 0;
+    __syncthreads();
+    const int p = base + tid;
+    const int e = (p < P) ? s_idx[p] : -1;
+    const bool valid = e >= 0;
+    unsigned long long peers = __ballot(valid);
+    for (int b = 0; b < a.nbits; ++b) {
+      const bool bit = (e >> b) & 1;
+      const unsigned long long bal = __ballot(valid && bit);
+      peers &= bit ? bal : ~bal;
+    }
+    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+    if (valid && rank == 0) s_w[w * E + e] = __popcll(peers);
+    __syncthreads();
+    if (tid < E) {
+      int run = s_run[tid];
+      for (int ww = 0; ww < 4; ++ww) {
+        const int c = s_w[ww * E + tid];
+        s_w[ww * E + tid] = run;
+        run += c;
+      }
+      s_run[tid] = run;
+    }
+    __syncthreads();
+    if (valid) {
+      const int pos = s_off[e] + s_w[w * E + e] + rank;
+      a.sorted_pair[pos] = p;
+      a.pos_of_pair[p] = pos;
+      a.sorted_tok[pos] = p / k;
+    }
+    __syncthreads();
   }
 }
 
@@ -1341,29 +1310,13 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
                                 int T, int H, int E, int E_rows, int ldl, int k, int mode, int *idx,
                                 float *w, int *counts, int *offsets, int *sorted_pair,
                                 int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
-                                int64_t *active_ids, int max_units, void *stream) {
+                                int64_t *active_ids, int max_units, unsigned *counter, void *stream) {
   if (!x || !wg || !logits || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair ||
-      !sorted_tok || !units || !n_active || !active_ids || T <= 0 || T > ROUTE_MAXT || H <= 0 || H % 8 ||
+      !sorted_tok || !units || !n_active || !active_ids || !counter || T <= 0 || T > ROUTE_MAXT || H <= 0 || H % 8 ||
       E <= 0 || E > 256 || E_rows < E || E_rows > E + 1 || ldl < E_rows || k <= 0 || k > 32 || k > E ||
-      mode < 0 || mode > 2 || max_units < 0) {
+      T * k > ROUTE_MAXP || mode < 0 || mode > 2 || max_units < 0) {
     moe_set_error("moe_route_decode: bad argument (T=%d H=%d E=%d k=%d)", T, H, E, k);
     return MOE_EINVAL;
-  }
-  const int P = T * k;
-  const size_t lds = (size_t)T * H * 2 + (size_t)T * ldl * 4 + (size_t)((P + 3) & ~3) * 4 +
-                     (size_t)(E + E + 1 + 16 * E + 34) * 4;
-  if (lds > 150 * 1024) {
-    moe_set_error("moe_route_decode: T=%d H=%d does not fit LDS; use the separate kernels", T, H);
-    return MOE_EINVAL;
-  }
-  static bool attr_set = false;
-  if (lds > 48 * 1024 && !attr_set) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)k_route_decode<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipError_t e2 = hipFuncSetAttribute((const void *)k_route_decode<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipError_t e3 = hipFuncSetAttribute((const void *)k_route_decode<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (int rc = moe_check_hip(e1 != hipSuccess ? e1 : (e2 != hipSuccess ? e2 : e3), "hipFuncSetAttribute(k_route_decode)"))
-      return rc;
-    attr_set = true;
   }
   RouteArgs a;
   a.x = (const uint16_t *)x; a.wg = (const uint16_t *)wg; a.bias = bias; a.logits = logits;
@@ -1373,10 +1326,9 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
   a.max_units = max_units; a.idx = idx; a.w = w; a.counts = counts; a.offsets = offsets;
   a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
   a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
+  a.counter = counter;
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
-  if (T == 1) hipLaunchKernelGGL(k_route_decode<1>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
-  else if (T <= 4) hipLaunchKernelGGL(k_route_decode<4>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL(k_route_decode<16>, dim3(1), dim3(1024), lds, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(k_route_decode, dim3((E_rows + 3) / 4, T), dim3(256), 0, (hipStream_t)stream, a);
   moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
   return moe_check_launch("k_route_decode");
 }

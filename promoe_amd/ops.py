@@ -67,8 +67,13 @@ def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispa
     return d
 
 
+_route_counter = {}
+
+
 def route_decode(x, wg, bias, E: int, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
     """Fused gate logits + top-k + dispatch for T <= 16.  wg may carry one extra row (shared gate)."""
+    if x.device not in _route_counter:   # the launch counter of the fused kernel: zero between calls
+        _route_counter[x.device] = torch.zeros(1, dtype=torch.int32, device=x.device)
     T, H = x.shape
     rows = wg.shape[0]
     logits = torch.empty(T, rows, dtype=torch.float32, device=x.device)
@@ -78,7 +83,8 @@ def route_decode(x, wg, bias, E: int, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
     check(lib.moe_route_decode(ptr(_dev(x)), ptr(_dev(wg)), ptr(bias), ptr(logits), T, H, E, rows, rows, k, mode,
                                ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets), ptr(d.sorted_pair),
                                ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units), ptr(d.n_active),
-                               ptr(d.active_ids), d.max_units, cur_stream()), "moe_route_decode")
+                               ptr(d.active_ids), d.max_units, ptr(_route_counter[x.device]), cur_stream()),
+          "moe_route_decode")
     return logits, idx, w, d
 
 
