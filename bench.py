@@ -39,6 +39,11 @@ def parse():
     ap.add_argument("--no-cache-run", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (matrix-core) legs")
+    ap.add_argument("--only", default="", help="profiling aid: run only these prefill legs (comma list of "
+                    "qwen, deepseek, mixtral) and print their results, without the decode benchmark")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="profiling aid: also run a plain 256 MiB read + 256 MiB write elementwise kernel three "
+                         "times, the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
     return ap.parse_args()
 
 
@@ -156,6 +161,24 @@ def main():
     import torch
     from promoe_amd import synth, layout as LY
     from promoe_amd._lib import lib
+    if a.copy_calibration:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+    if a.only:
+        from promoe_amd import _lib as L
+        legs = {"qwen": ("Qwen1.5-MoE-A2.7B-shaped layer, bf16 experts, prefill T=2048, all resident",
+                         2048, 2048, 60, 1408, 4, 5632, L.FMT_BF16, True, 0, 20),
+                "deepseek": ("DeepSeek-MoE-16B-shaped layer, int4-g128 experts, prefill T=2048, all resident",
+                             2048, 2048, 64, 1408, 6, 2816, L.FMT_INT4_G128, False, 0, 20),
+                "mixtral": ("Mixtral-8x7B-shaped layer, int4-g128 experts, prefill T=4096, all resident",
+                            4096, 4096, 8, 14336, 2, 0, L.FMT_INT4_G128, False, 2, 5)}
+        res = [prefill_leg(torch, *legs[n][:-1], steps=legs[n][-1]) for n in a.only.split(",")]
+        print(json.dumps({"prefill": res}))
+        return
 
     global xs_out
     dev = torch.device("cuda:0")
