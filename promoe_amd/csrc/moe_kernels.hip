@@ -75,6 +75,78 @@ __global__ __launch_bounds__(256) void k_gate_logits(const uint16_t *__restrict_
   if (lane == 0) logits[(size_t)t * ldl + e] = bias ? acc + bias[e] : acc;
 }
 
+// Large T: a workgroup stages 16 token rows in LDS and every wave walks its gate rows over all
+// 16 tokens, so a gate row is fetched once per 16 tokens instead of once per token.  Each
+// (token, row) sum is formed in exactly the order of k_gate_logits (lane partials over
+// k = c*512 + 8*lane + i with one fma chain, then the xor butterfly 32..1): same bits.
+#define GATE_TT 16
+__global__ __launch_bounds__(256) void k_gate_logits_tile(const uint16_t *__restrict__ x,
+                                                           const uint16_t *__restrict__ wg,
+                                                           const float *__restrict__ bias,
+                                                           float *__restrict__ logits, int T, int H,
+                                                           int E, int ldl, int rows_per_block) {
+  extern __shared__ uint4 gxs[];  // [GATE_TT][H/8]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int t0 = blockIdx.x * GATE_TT;
+  const int nt = (T - t0) < GATE_TT ? (T - t0) : GATE_TT;
+  const int vpr = H >> 3;
+  const uint4 *xsrc = (const uint4 *)(x + (size_t)t0 * H);
+  for (int i = tid; i < nt * vpr; i += 256) gxs[i] = xsrc[i];
+  for (int i = nt * vpr + tid; i < GATE_TT * vpr; i += 256) gxs[i] = make_uint4(0, 0, 0, 0);
+  __syncthreads();
+  const int e_end = min(E, (int)(blockIdx.y + 1) * rows_per_block);
+  const int nch = (H + 511) >> 9;  // <= 8 (checked by the launcher)
+  const int kl = 8 * lane;
+  uint4 wv[8], wn[8];
+  auto load_row = [&](uint4(&dst)[8], int e) {
+    const uint16_t *wr = wg + (size_t)(e < e_end ? e : blockIdx.y * rows_per_block) * H;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+      if (c < nch) {
+        const int k = c * 512 + kl;
+        dst[c] = *(const uint4 *)(wr + (k < H ? k : 0));
+      }
+  };
+  int e = blockIdx.y * rows_per_block + w;
+  if (e < e_end) load_row(wv, e);
+  for (; e < e_end; e += 4) {
+    load_row(wn, e + 4);  // next row of this wave in flight while this one is used
+    float acc[GATE_TT];
+#pragma unroll
+    for (int t = 0; t < GATE_TT; ++t) acc[t] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int k = c * 512 + kl;
+      if (c < nch && k < H) {
+#pragma unroll
+        for (int t = 0; t < GATE_TT; ++t) {
+          const uint4 xv = gxs[t * vpr + (k >> 3)];
+          float a = acc[t];
+          a = fmaf(bf16lo(xv.x), bf16lo(wv[c].x), a);
+          a = fmaf(bf16hi(xv.x), bf16hi(wv[c].x), a);
+          a = fmaf(bf16lo(xv.y), bf16lo(wv[c].y), a);
+          a = fmaf(bf16hi(xv.y), bf16hi(wv[c].y), a);
+          a = fmaf(bf16lo(xv.z), bf16lo(wv[c].z), a);
+          a = fmaf(bf16hi(xv.z), bf16hi(wv[c].z), a);
+          a = fmaf(bf16lo(xv.w), bf16lo(wv[c].w), a);
+          a = fmaf(bf16hi(xv.w), bf16hi(wv[c].w), a);
+          acc[t] = a;
+        }
+      }
+    }
+    const float be = bias ? bias[e] : 0.f;
+#pragma unroll
+    for (int t = 0; t < GATE_TT; ++t) {
+      float a = acc[t];
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) a = a + __shfl_xor(a, m, 64);
+      if (lane == 0 && t < nt) logits[(size_t)(t0 + t) * ldl + e] = bias ? a + be : a;
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) wv[c] = wn[c];
+  }
+}
+
 // ---------------------------------------------------------------------------
 // k1b top-k: one wave per token, E <= 256
 // ---------------------------------------------------------------------------
@@ -990,6 +1062,28 @@ extern "C" int moe_gate_logits(const void *x, const void *wg, const float *bias,
     return MOE_EINVAL;
   }
   if (T == 0) return MOE_OK;
+  const size_t tile_lds = (size_t)GATE_TT * H * 2;
+  if (T > 16 && H <= 4096 && tile_lds <= 150 * 1024) {
+    static bool attr_set = false;
+    if (tile_lds > 64 * 1024 && !attr_set) {
+      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gate_logits_tile,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                 "hipFuncSetAttribute(k_gate_logits_tile)"))
+        return rc;
+      attr_set = true;
+    }
+    // enough workgroups to fill the chip: split the gate rows when there are few token tiles
+    const int tiles = (T + GATE_TT - 1) / GATE_TT;
+    int split = 1;
+    while (tiles * split < 1024 && split * 4 < E) split *= 2;
+    const int rows_per_block = (((E + split - 1) / split) + 3) & ~3;
+    dim3 grid(tiles, (E + rows_per_block - 1) / rows_per_block);
+    moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
+    hipLaunchKernelGGL(k_gate_logits_tile, grid, dim3(256), tile_lds, (hipStream_t)stream, (const uint16_t *)x,
+                       (const uint16_t *)wg, bias, logits, T, H, E, ldl, rows_per_block);
+    moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
+    return moe_check_launch("k_gate_logits_tile");
+  }
   dim3 grid((E + 3) / 4, T);
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_gate_logits, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,

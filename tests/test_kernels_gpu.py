@@ -16,7 +16,8 @@ def bf16_dev(a, dev):
 
 
 @pytest.mark.parametrize("T,H,E", [(1, 2048, 64), (4, 2048, 64), (16, 2048, 64), (5, 4096, 8),
-                                   (3, 3584, 65), (7, 256, 60), (2, 2048, 61)])
+                                   (3, 3584, 65), (7, 256, 60), (2, 2048, 61),
+                                   (17, 2048, 64), (515, 3584, 65), (300, 4096, 8), (2048, 2048, 61), (33, 256, 3)])
 def test_gate_logits_bit_exact(cuda, T, H, E):
     from promoe_amd import ops
     print(f"case gate_logits T={T} H={H} E={E}", flush=True)
