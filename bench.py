@@ -307,7 +307,8 @@ def main():
         hit, miss = c2["hit"] - c0["hit"], c2["miss"] - c0["miss"]
         cache_run = {"cache_rate": 0.375, "policy": "lru", "tokens_per_s": T * n2 / d3, "ms_per_step": d3 / n2 * 1e3,
                      "hit_rate": hit / max(hit + miss, 1), "h2d_GB": (c2["h2d_bytes"] - c0["h2d_bytes"]) / 1e9,
-                     "h2d_GBps": (c2["h2d_bytes"] - c0["h2d_bytes"]) / d3 / 1e9, "steps": n2}
+                     "h2d_GBps": (c2["h2d_bytes"] - c0["h2d_bytes"]) / d3 / 1e9, "steps": n2,
+                     "misses": miss, "wait_us_per_miss": (c2["wait_us"] - c0["wait_us"]) / max(miss, 1)}
         pm2.close()
 
     prefill = None

@@ -543,10 +543,20 @@ static void fetch_thread_main(moe_engine *eng) {
     lk.unlock();
     int rc = 0;
     size_t bytes = 0;
-    for (int c = start; c < stop && rc == 0; ++c) {
+    // chunks that are neighbours both in host memory and in the slot go out as one copy
+    for (int c = start; c < stop && rc == 0;) {
       const HostChunk &hc = e->chunks[c];
-      if (hc.nbytes) rc = eng->be->copy_h2d(dst + eng->chunk_off[c], hc.ptr, hc.nbytes);
-      bytes += hc.nbytes;
+      size_t n = hc.nbytes;
+      int c2 = c + 1;
+      while (c2 < stop && e->chunks[c2].nbytes && n &&
+             (const char *)e->chunks[c2].ptr == (const char *)hc.ptr + n &&
+             eng->chunk_off[c2] == eng->chunk_off[c] + n) {
+        n += e->chunks[c2].nbytes;
+        ++c2;
+      }
+      if (n) rc = eng->be->copy_h2d(dst + eng->chunk_off[c], hc.ptr, n);
+      bytes += n;
+      c = c2;
     }
     if (rc == 0) rc = eng->be->copy_sync();
     lk.lock();
