@@ -105,6 +105,10 @@ def prefill_leg(torch, name, T, H, E, I, k, I_sh, fmt, gated, mode, steps=20):
         img = (torch.randn(E, 3 * I * H, device=dev, generator=g) * 0.02).to(torch.bfloat16)
         sh = (torch.randn(3 * I_sh * H, device=dev, generator=g) * 0.02).to(torch.bfloat16) if I_sh else None
         wbytes = E * 3 * I * H * 2 + 3 * I_sh * H * 2
+    elif fmt == L.FMT_Q4K:
+        img = synth.random_q4k_images(E, H, I, dev, g)
+        sh = synth.random_q4k_images(1, H, I_sh, dev, g)[0] if I_sh else None
+        wbytes = E * LY.q4k_layout(H, I)["total_bytes"] + (LY.q4k_layout(H, I_sh)["total_bytes"] if I_sh else 0)
     else:
         img = synth.random_int4_images(E, H, I, dev, g)
         sh = synth.random_int4_images(1, H, I_sh, dev, g)[0] if I_sh else None
@@ -144,12 +148,106 @@ def prefill_leg(torch, name, T, H, E, I, k, I_sh, fmt, gated, mode, steps=20):
             "expert_flops": flops, "weight_bytes": wbytes,
             "layer_TFLOPs": (flops + 2.0 * T * wg.shape[0] * H) / t_layer / 1e12,
             "roofline": {"bound": "mfma", "kernel": "k_prefill_%s<true> (w13 + SwiGLU, routed + shared in one launch)" %
-                         ("gemm" if fmt == L.FMT_BF16 else "int4"),
+                         ("gemm" if fmt == L.FMT_BF16 else ("int4<q4_K>" if fmt == L.FMT_Q4K else "int4")),
                          "achieved": ach, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK_TFLOPS,
                          "traffic": None, "avg_launch_us": t_w13 * 1e6,
                          "algorithmic_flops_per_launch": flops * 2 / 3,
                          "method": "%d back-to-back launches (tile-list kernel included) between one HIP event pair" % steps},
             "w2_launch_us": t_w2 * 1e6, "w2_TFLOPs": flops / 3 / t_w2 / 1e12}
+
+
+def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf, steps=200):
+    """Decode-size MoE layer forward at kernel level, every expert resident in HBM (images of `layers`
+    layers in rotation, far more than the caches hold): route -> experts -> combine on one stream."""
+    import numpy as np
+    from promoe_amd import ops, synth, layout as LY, _lib as L
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(9)
+    q4k = fmt == L.FMT_Q4K
+    mk = synth.random_q4k_images if q4k else synth.random_int4_images
+    lay = LY.q4k_layout if q4k else LY.int4_layout
+    if T > 16:   # the rule of moe_forward: token groups above 16 rows take the matrix-core kernels
+        def run_experts(x, d_, table, sh, H_, I_, I_sh_, phases=3, ws=None):
+            return ops.experts_prefill(x, d_, table, sh, H_, I_, I_sh_, fmt, phases=phases, ws=ws)
+    else:
+        run_experts = ops.experts_decode_q4k if q4k else ops.experts_decode_int4
+    imgs, shs, gws, biases, tables = [], [], [], [], []
+    for l in range(layers):
+        imgs.append(mk(E, H, I, dev, g))
+        shs.append(mk(1, H, I_sh, dev, g)[0] if I_sh else None)
+        gws.append((torch.randn(E + (1 if gated else 0), H, device=dev, generator=g) * 0.02).to(torch.bfloat16))
+        b = None
+        if zipf:
+            b = torch.from_numpy(np.concatenate([synth.zipf_bias(E, zipf, 100 + l), np.zeros(1 if gated else 0, np.float32)])).to(dev)
+        biases.append(b)
+        tables.append(torch.tensor([imgs[l][e].data_ptr() for e in range(E)], dtype=torch.int64, device=dev))
+    xs = [torch.randn(T, H, device=dev, generator=g).to(torch.bfloat16) for _ in range(8)]
+    y = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+    rows = E + (1 if gated else 0)
+    logits = torch.empty(T, rows, dtype=torch.float32, device=dev)
+    d = ops.Dispatch(T, k, E, min(E, T * k), dev)
+    ws = None
+    nact = []
+
+    def step(i, phases=3, route=True):
+        nonlocal ws
+        l, x = i % layers, xs[i % len(xs)]
+        if route:
+            ops.gate_logits(x, gws[l], biases[l], out=logits)
+            idx, w = ops.topk(logits, k, mode, E=E)
+            ops.dispatch(idx, E, out=d)
+            step.w = w
+        ws = run_experts(x, d, tables[l], shs[l], H, I, I_sh, phases=phases, ws=ws)
+        if phases == 3:
+            ops.combine(ws[0], ws[1], step.w, d.pos_of_pair, logits[:, E] if gated else None, T, H, k, out=y)
+
+    def timed(fn, n):
+        for i in range(min(n, 2 * layers)):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+
+    for i in range(4 * layers):
+        step(i)
+        nact.append(int(d.n_active.cpu()[0]))
+    assert int(ws[2].cpu()[0]) == 0
+    t_layer = timed(step, steps)
+    # the w13 + SwiGLU GEMV alone, back to back, with the routing of the last full step kept
+    t_w13 = timed(lambda i: step(i, phases=1, route=False), steps)
+    D = float(np.mean(nact))
+    D_last = nact[-1]
+    lr = lay(H, I)
+    ls = lay(H, I_sh) if I_sh else {"total_bytes": 0, "off2_q": 0}
+    step_bytes = D * lr["total_bytes"] + ls["total_bytes"] + rows * H * 2 + 2 * T * H * 2
+    w13_bytes = D_last * lr["off2_q"] + ls["off2_q"] + 2 * T * H
+    ach = w13_bytes / t_w13 / 1e9
+    return {"workload": name, "tokens": T, "layers_in_rotation": layers, "tokens_per_s": T / t_layer,
+            "us_per_layer": t_layer * 1e6, "distinct_routed_experts_per_step": D,
+            "algorithmic_bytes_per_step": step_bytes, "layer_GBps": step_bytes / t_layer / 1e9,
+            "roofline": {"bound": "hbm", "kernel": ("k_prefill_int4 (w13 + SwiGLU)" if T > 16 else
+                                                    "k_gemv_int4%s (w13 + SwiGLU)" % ("<q4_K>" if q4k else ("_mfma" if T > 1 else ""))),
+                         "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+                         "algorithmic_bytes_per_launch": w13_bytes, "avg_launch_us": t_w13 * 1e6,
+                         "method": "%d back-to-back launches between one HIP event pair" % steps}}
+
+
+def other_configs(torch):
+    """Decode legs of the Mixtral-shaped int4 and Qwen2-57B-shaped q4_K configurations."""
+    from promoe_amd import _lib as L
+    out = []
+    for T in (1, 64):
+        out.append(decode_leg(torch, "Mixtral-8x7B-shaped layer, int4-g128 experts, decode T=%d, all resident, "
+                              "uniform routing" % T, L.FMT_INT4_G128, T, 4096, 8, 14336, 2, 0, False, 2, 4, None,
+                              steps=60 if T == 1 else 20))
+    out.append(decode_leg(torch, "Qwen2-57B-A14B-shaped layer, q4_K experts, decode T=3 (three sequences), all "
+                          "resident, Zipf(1.1)", L.FMT_Q4K, 3, 3584, 64, 2560, 8, 20480, True, 0, 3, 1.1, steps=60))
+    return out
 
 
 def main():
@@ -323,6 +421,13 @@ def main():
                         4096, 4096, 8, 14336, 2, 0, L.FMT_INT4_G128, False, 2, steps=5),
         ]
 
+    others = None
+    if not a.no_prefill:
+        others = other_configs(torch)
+        from promoe_amd import _lib as L
+        prefill.append(prefill_leg(torch, "Qwen2-57B-A14B-shaped layer, q4_K experts, prefill T=512, all resident",
+                                   512, 3584, 64, 2560, 8, 20480, L.FMT_Q4K, True, 0, steps=10))
+
     cpu = None
     if not a.no_cpu:
         threads = 8   # the reference's own torch.set_num_threads(8) (utils/__init__.py:343)
@@ -339,7 +444,7 @@ def main():
                       "hidden": H, "experts": E, "intermediate": I, "shared_intermediate": I_sh, "top_k": k,
                       "tokens_per_step": T, "layers": L_, "zipf": 1.2},
            "roofline": roofline, "cpu_baseline": cpu, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
-           "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run, "prefill": prefill}
+           "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run, "prefill": prefill, "other_decode_configs": others}
     print(json.dumps(out))
 
 

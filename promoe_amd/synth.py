@@ -27,6 +27,19 @@ def random_int4_images(n: int, H: int, I: int, device, gen: torch.Generator) -> 
     return buf
 
 
+def random_q4k_images(n: int, H: int, I: int, device, gen: torch.Generator) -> torch.Tensor:
+    """n q4_K expert images [n, total_bytes] uint8: uniform nibbles, 6-bit scales and mins, fp16 d and
+    dmin around 1e-4 (weights of a few 1e-2 in magnitude)."""
+    lay = LY.q4k_layout(H, I)
+    buf = torch.randint(0, 256, (n, lay["total_bytes"]), dtype=torch.uint8, device=device, generator=gen)
+    for s0, z0, end in ((lay["off13_s"], lay["off13_z"], lay["off2_q"]), (lay["off2_s"], lay["off2_z"], lay["total_bytes"])):
+        buf[:, s0:z0] &= 63
+        nd = (end - z0) // 2
+        d = (torch.rand(n, nd, device=device, generator=gen) * 1e-4 + 5e-5).to(torch.float16)
+        buf[:, z0:end] = d.view(torch.uint8)
+    return buf
+
+
 def zipf_bias(E: int, s: float, seed: int) -> np.ndarray:
     rng = np.random.default_rng(seed)
     rank = rng.permutation(E) + 1
