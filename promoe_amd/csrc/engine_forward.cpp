@@ -199,6 +199,48 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // hook order of the reference (utils/hooks.py:216-223)
   if (layer == 0 && (rc = moe_report_layer_logits(eng, 0, x, 1, T, d.H))) return rc;
   const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
+  if ((rc = moe_forward_harvest(eng, false))) return rc;
+  // Every expert of the layer resident, and the layer's slot group can hold them all: there
+  // is nothing for the host to decide, so no round trip.  The kernels take the device-built
+  // unit list; the routing comes back asynchronously and the hits are accounted when it lands.
+  bool all_resident = false;
+  {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
+                   eng->layer_complete[layer] == E;
+  }
+  static const bool token_route = !(getenv("MOE_TOKEN_ROUTE") && atoi(getenv("MOE_TOKEN_ROUTE")) == 0);
+  if (all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
+    // one token: gate logits, then the w13 kernel routes by itself (no top-k / dispatch launches)
+    if (!d.gate_bias) {
+      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+    } else {
+      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+      if (d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    }
+    const uint64_t *table = nullptr;
+    if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, st)))
+      return rc;
+    LayerState::Pending &p = s->pend[s->pend_head];
+    if (p.busy && (rc = moe_forward_harvest(eng, true))) return rc;
+    s->pend_head = (s->pend_head + 1) % LayerState::kPending;
+    HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
+    HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
+    HIPC(hipEventRecord(p.ev, st));
+    p.layer = layer; p.max_units = max_units; p.busy = true;
+    const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
+    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
+      return rc;
+    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    return moe_layer_done(eng, layer);
+  }
   static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
   if (fused_route && T <= 2 && E <= 256 && T * k <= 512) {
     // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
@@ -222,16 +264,6 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
                            s->units, s->n_active, s->active_ids, max_units, st)))
       return rc;
-  }
-  if ((rc = moe_forward_harvest(eng, false))) return rc;
-  // Every expert of the layer resident, and the layer's slot group can hold them all: there
-  // is nothing for the host to decide, so no round trip.  The kernels take the device-built
-  // unit list; the routing comes back asynchronously and the hits are accounted when it lands.
-  bool all_resident = false;
-  {
-    std::lock_guard<std::mutex> lk(eng->mu);
-    all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
-                   eng->layer_complete[layer] == E;
   }
   if (all_resident) {
     LayerState::Pending &p = s->pend[s->pend_head];

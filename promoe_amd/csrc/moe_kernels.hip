@@ -532,6 +532,12 @@ struct GemvArgs {
   int *err;
   KUnit ku[GEMV_MAX_KUNITS];             // units resolved on the host, passed by value: the
                                          // weight loads then depend on no global load
+  // one-token launches that route inside the kernel (ROUTE): inputs and the routing outputs
+  const float *r_logits;
+  int r_E, r_k, r_mode, r_pad;
+  int *r_idx; float *r_w;
+  int *r_counts, *r_offsets, *r_sorted_pair, *r_pos_of_pair, *r_sorted_tok;
+  moe_unit *r_units; int *r_n_active; long long *r_active_ids;
 };
 
 // global-address-space loads (pointers that come out of the slot table are generic
@@ -616,13 +622,157 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
 // Q4K: same nibble tiles, but the scale data is per 32-wide sub-block (= one lane's k quarter):
 // section s holds (6-bit scale, 6-bit min) byte pairs [N/16][G][64 lanes], section z holds
 // (fp16 d, fp16 dmin) pairs [N/16][G/2][16 rows]; w = d*sc*q - dmin*m.
-template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false>
+// One token: every workgroup derives the routing itself from the gate logits instead of
+// reading a unit list made by two earlier launches.  With one token the dispatch is trivial
+// (unit u = the u-th smallest selected expert id, one row each), and the top-k of <= 256
+// logits costs a wave well under a microsecond when done by ranking: lane l holds logits
+// l, l+64, ...; rank(e) = #{e' : v[e'] > v[e] or (v[e'] == v[e] and e' < e)} from one pass of
+// broadcasts; e is selected iff rank(e) < k, and is the rank(e)-th choice - the order and the
+// tie rule of k_topk.  The first routed workgroup also publishes the routing (indices,
+// weights, dispatch arrays, unit list) for the later kernels and the host.
+static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w) {
+  GemvWork wk;
+  const int n_sh = a.n_sh_blocks;
+  const bool sh = (int)blockIdx.x < n_sh;
+  wk.c = sh ? a.cls[0] : a.cls[1];
+  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
+  const int E = a.r_E, k = a.r_k;
+  // one extra workgroup at the end of the grid only publishes the routing (its first wave);
+  // it finishes long before the workgroups that stream weights
+  const bool publisher = !sh && rr == k * wk.c.nblk;
+  const int u = (sh || publisher) ? 0 : rr / wk.c.nblk;
+  wk.b = rr - u * wk.c.nblk;
+  if (sh) {
+    wk.m = 1; wk.row0 = 0; wk.base = a.shared_base;
+    return wk;
+  }
+  if (publisher && w != 0) { wk.m = 0; wk.row0 = 0; wk.base = nullptr; return wk; }
+  const float NEG = -__builtin_inff();
+  float v[4];
+  int rank[4];
+  unsigned long long ptrs[4];  // slot addresses of the lane's candidates, fetched alongside the logits
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int e = lane + 64 * r;
+    v[r] = (e < E) ? a.r_logits[e] : NEG;
+    ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
+    rank[r] = 0;
+  }
+#pragma unroll
+  for (int r2 = 0; r2 < 4; ++r2) {
+    if (64 * r2 < E) {
+#pragma unroll 16
+      for (int i = 0; i < 64; ++i) {
+        const float o = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[r2]), i));
+        const int oe = i + 64 * r2;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (64 * r < E) {  // uniform: only the logit columns that exist are ranked
+            const int e = lane + 64 * r;
+            rank[r] += (o > v[r] || (o == v[r] && oe < e)) ? 1 : 0;
+          }
+        }
+      }
+    }
+  }
+  unsigned long long msel[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) msel[r] = __ballot(lane + 64 * r < E && rank[r] < k);
+  // unit u = the u-th smallest selected id
+  int cum = 0;
+  bool found = false;
+  unsigned lo = 0, hi = 0;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int cnt = __popcll(msel[r]);
+    if (!found && u < cum + cnt) {
+      unsigned long long mm = msel[r];
+      for (int i = 0; i < u - cum; ++i) mm &= mm - 1;
+      const int src = (int)__builtin_ctzll(mm);  // expert 64 r + src
+      lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)ptrs[r], src);
+      hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(ptrs[r] >> 32), src);
+      found = true;
+    }
+    cum += cnt;
+  }
+  wk.m = 1; wk.row0 = u;
+  wk.base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+
+  if (publisher) {  // publish the routing: body of k_topk (weights) and k_dispatch (T = 1)
+    wk.m = 0;       // no weight tiles for this workgroup
+    // selected logits in choice order (lane j keeps choice j); the row maximum is choice 0
+    float mx = 0.f, sum_sel = 0.f, my_v = 0.f;
+    int my_e = 0;
+#pragma unroll 1
+    for (int j = 0; j < k; ++j) {
+      float val = 0.f; int ee = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const unsigned long long mj = __ballot(lane + 64 * r < E && rank[r] == j);
+        if (mj) {
+          const int src = (int)__builtin_ctzll(mj);
+          val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[r]), src));
+          ee = src + 64 * r;
+        }
+      }
+      if (j == 0) mx = val;
+      sum_sel += expf(val - mx);
+      if (lane == j) { my_v = val; my_e = ee; }
+    }
+    float den = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (lane + 64 * r < E) den += expf(v[r] - mx);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
+    const float ex = expf(my_v - mx);
+    float wgt;
+    if (a.r_mode == MOE_ROUTE_TOPK_SOFTMAX) {
+      wgt = ex / sum_sel;
+    } else {
+      wgt = ex / den;
+      if (a.r_mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
+    }
+    // dispatch of the k pairs of the one token: position = rank of the expert id among the selected
+    int below[4], cb = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { below[r] = cb; cb += __popcll(msel[r]); }
+    if (lane < k) {
+      const int r_ = my_e >> 6, l_ = my_e & 63;
+      int pos = 0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (r == r_) pos = below[r] + __popcll(msel[r] & ((1ull << l_) - 1ull));
+      a.r_idx[lane] = my_e;
+      a.r_w[lane] = wgt;
+      a.r_sorted_pair[pos] = lane;
+      a.r_pos_of_pair[lane] = pos;
+      a.r_sorted_tok[pos] = 0;
+      moe_unit un; un.expert = my_e; un.m = 1; un.row0 = pos; un.pad = 0;
+      a.r_units[pos] = un;
+      a.r_active_ids[pos] = my_e;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int e = lane + 64 * r;
+      if (e < E) {
+        const bool selb = (msel[r] >> lane) & 1ull;
+        a.r_counts[e] = selb ? 1 : 0;
+        a.r_offsets[e] = below[r] + __popcll(msel[r] & ((1ull << lane) - 1ull));
+      }
+    }
+    if (lane == 0) { a.r_offsets[E] = k; *a.r_n_active = k; }
+  }
+  return wk;
+}
+
+template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false, bool ROUTE = false>
 __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  const GemvWork wk = ROUTE ? gemv_resolve_route(a, lane, w) : gemv_resolve<DEVUNITS>(a);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0, b = wk.b;
   const unsigned char *base = wk.base;
@@ -1341,6 +1491,67 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
     if (rc) return rc;
   }
   return MOE_OK;
+}
+
+template <int CH>
+static int launch_gemv_route(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
+  moe_ktimer_begin(MOE_K_W13, s);
+  hipLaunchKernelGGL((k_gemv_int4<1, true, CH, true, false, true>), dim3(grid), dim3(256), lds, s, a);
+  moe_ktimer_end(MOE_K_W13, s);
+  return moe_check_launch("k_gemv_int4<route>");
+}
+
+extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, int k, int mode, int H, int I,
+                                     int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                     float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
+                                     int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
+                                     void *h_r, void *h_s, float *part_r, float *part_s, int *err, void *stream) {
+  if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
+      !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
+      mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
+      (shared_ptr && (!h_s || !part_s || I_sh == 0))) {
+    moe_set_error("moe_decode_token_int4: bad argument (E=%d k=%d H=%d I=%d I_sh=%d)", E, k, H, I, I_sh);
+    return MOE_EINVAL;
+  }
+  moe_int4_layout lr, ls;
+  memset(&lr, 0, sizeof lr); memset(&ls, 0, sizeof ls);
+  if (moe_int4_layout_make(H, I, &lr)) return MOE_EINVAL;
+  if (shared_ptr && moe_int4_layout_make(H, I_sh, &ls)) return MOE_EINVAL;
+  const bool sh = shared_ptr != nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  GemvArgs a;
+  memset(&a, 0, sizeof a);
+  a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
+  a.shared_base = (const unsigned char *)shared_ptr; a.T = 1; a.err = err;
+  a.r_logits = logits; a.r_E = E; a.r_k = k; a.r_mode = mode; a.r_idx = idx; a.r_w = w; a.r_counts = counts;
+  a.r_offsets = offsets; a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok;
+  a.r_units = units; a.r_n_active = n_active; a.r_active_ids = (long long *)active_ids;
+  // pass 1: w13 + SwiGLU, routing derived in the kernel
+  a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, 0, I_sh, I_sh / 16, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
+  a.n_sh_blocks = sh ? I_sh / 16 : 0;
+  int grid = a.n_sh_blocks + k * (I / 16) + 1;  // + the publishing workgroup
+  {
+    const int gpw = (H / 128 + 3) / 4;
+    int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
+    if (ch < 1) ch = 1;
+    const size_t lds = gemv_lds(1, H);
+    if (lds > 64 * 1024) { moe_set_error("moe_decode_token_int4: H=%d does not fit LDS", H); return MOE_EINVAL; }
+    int rc;
+    switch (ch) {
+      case 1: rc = launch_gemv_route<1>(a, grid, lds, s); break;
+      case 2: rc = launch_gemv_route<2>(a, grid, lds, s); break;
+      case 3: rc = launch_gemv_route<3>(a, grid, lds, s); break;
+      default: rc = launch_gemv_route<4>(a, grid, lds, s); break;
+    }
+    if (rc) return rc;
+  }
+  // pass 2: w2 over the unit list the first pass published
+  a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z, I_sh, I_sh / 128, I_sh, H, H / 32, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z, I, I / 128, I, H, H / 32, 0};
+  a.n_sh_blocks = sh ? H / 32 : 0;
+  grid = a.n_sh_blocks + k * (H / 32);
+  return launch_gemv_t<false>(a, grid, 1, I_sh > I ? I_sh : I, I / 128, s);
 }
 
 extern "C" int moe_q4k_layout_make(int H, int I, moe_int4_layout *out) {

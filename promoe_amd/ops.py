@@ -115,6 +115,30 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
     return part_r, part_s, err, h_r, h_s
 
 
+def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int, ws=None):
+    """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
+    dev = x.device
+    if ws is None:
+        idx = torch.empty(1, k, dtype=torch.int32, device=dev)
+        w = torch.empty(1, k, dtype=torch.float32, device=dev)
+        d = Dispatch(1, k, E, min(E, k), dev)
+        h_r = torch.empty(k, I, dtype=torch.bfloat16, device=dev)
+        part_r = torch.empty(k, H, dtype=torch.float32, device=dev)
+        h_s = part_s = None
+        if shared is not None:
+            h_s = torch.empty(1, I_sh, dtype=torch.bfloat16, device=dev)
+            part_s = torch.empty(1, H, dtype=torch.float32, device=dev)
+        err = torch.zeros(1, dtype=torch.int32, device=dev)
+    else:
+        idx, w, d, part_r, part_s, err, h_r, h_s = ws
+    check(lib.moe_decode_token_int4(ptr(_dev(x)), ptr(logits), E, k, mode, H, I, I_sh if shared is not None else 0,
+                                    ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
+                                    ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                    ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
+                                    ptr(err), cur_stream()), "moe_decode_token_int4")
+    return idx, w, d, part_r, part_s, err, h_r, h_s
+
+
 def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
                        H: int, I: int, I_sh: int, phases: int = 3, ws=None):
     """q4_K flavour of experts_decode_int4 (device-side unit list)."""

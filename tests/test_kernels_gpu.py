@@ -200,3 +200,40 @@ def test_decode_q4k_qwen2_shape(cuda):
     layer = Q4KLayer(H=3584, I=2560, E=8, I_sh=5120, seed=1, shared_gate=True, zipf=1.1)
     for T in (1, 3):
         check_layer(layer, T, 4, 0, cuda)
+
+
+@pytest.mark.parametrize("H,I,E,k,mode,I_sh,zipf", [(2048, 1408, 16, 6, 0, 2816, 1.2), (256, 384, 8, 2, 2, 256, None),
+                                                    (256, 256, 60, 4, 1, 512, 1.1), (512, 128, 200, 8, 0, 0, None)])
+def test_token_decode_routes_in_kernel_like_separate_kernels(cuda, H, I, E, k, mode, I_sh, zipf):
+    """One token: the w13 kernel derives the routing itself.  Indices, weights, dispatch arrays and
+    the layer output must equal those of gate -> top-k -> dispatch -> experts -> combine, bit for bit."""
+    from promoe_amd import ops
+    print(f"case token_route H={H} I={I} E={E} k={k} mode={mode}", flush=True)
+    layer = Int4Layer(H=H, I=I, E=E, I_sh=I_sh, seed=11, zipf=zipf)
+    slots = [torch.from_numpy(s).to(cuda) for s in layer.slots]
+    table = torch.tensor([s.data_ptr() for s in slots], dtype=torch.int64, device=cuda)
+    shared = torch.from_numpy(layer.shared_img).to(cuda) if I_sh else None
+    wg = bf16_dev(layer.wg, cuda)
+    bias = None if layer.bias is None else torch.from_numpy(layer.bias).to(cuda)
+    for seed in range(3):
+        x = O.synth_acts(1, H, seed=seed)
+        if seed == 2:   # constructed ties in the logits: equal gate rows give equal logits
+            wg = wg.clone(); wg[3] = wg[1]; wg[E - 1] = wg[1]
+            if bias is not None:
+                bias = bias.clone(); bias[3] = bias[1]; bias[E - 1] = bias[1]
+        xd = bf16_dev(x, cuda)
+        logits = ops.gate_logits(xd, wg, bias)
+        idx, w = ops.topk(logits, k, mode)
+        d = ops.dispatch(idx, E)
+        part_r, part_s, err, _, _ = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh)
+        y_ref = ops.combine(part_r, part_s, w, d.pos_of_pair, None, 1, H, k)
+        idx2, w2, d2, pr2, ps2, err2, _, _ = ops.decode_token_int4(xd, logits, E, k, mode, table, shared, H, I, I_sh)
+        y = ops.combine(pr2, ps2, w2, d2.pos_of_pair, None, 1, H, k)
+        torch.cuda.synchronize()
+        assert int(err.cpu()[0]) == 0 and int(err2.cpu()[0]) == 0
+        assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+        for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active"):
+            assert torch.equal(getattr(d, name), getattr(d2, name)), name
+        na = int(d.n_active.cpu()[0])
+        assert torch.equal(d.units[:na], d2.units[:na]) and torch.equal(d.active_ids[:na], d2.active_ids[:na])
+        assert torch.equal(y_ref, y)
