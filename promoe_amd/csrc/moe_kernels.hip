@@ -625,11 +625,28 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
 // One token: every workgroup derives the routing itself from the gate logits instead of
 // reading a unit list made by two earlier launches.  With one token the dispatch is trivial
 // (unit u = the u-th smallest selected expert id, one row each), and the top-k of <= 256
-// logits costs a wave well under a microsecond when done by ranking: lane l holds logits
-// l, l+64, ...; rank(e) = #{e' : v[e'] > v[e] or (v[e'] == v[e] and e' < e)} from one pass of
-// broadcasts; e is selected iff rank(e) < k, and is the rank(e)-th choice - the order and the
-// tie rule of k_topk.  The first routed workgroup also publishes the routing (indices,
-// weights, dispatch arrays, unit list) for the later kernels and the host.
+// logits is k rounds of a wave-wide maximum built from DPP row shifts and broadcasts (no LDS,
+// no scalar round trips): lane l holds logits l, l+64, ...; the winner of a round is the
+// lowest expert id that holds the maximum - the order and the tie rule of k_topk.  One spare
+// workgroup publishes the routing (indices, weights, dispatch arrays, unit list) for the
+// later kernels and the host.
+static __device__ __forceinline__ float wave_max_f32(float x) {
+  // inclusive max-scan inside each row of 16 lanes, then rows 0->1, 2->3, then 1->3: lane 63 holds the result
+#define WMAX_STEP(ctrl, rmask)                                                                          \
+  {                                                                                                     \
+    const int xi = __builtin_bit_cast(int, x);                                                          \
+    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, ctrl, rmask, 0xf, false))); \
+  }
+  WMAX_STEP(0x111, 0xf)  // row_shr:1
+  WMAX_STEP(0x112, 0xf)  // row_shr:2
+  WMAX_STEP(0x114, 0xf)  // row_shr:4
+  WMAX_STEP(0x118, 0xf)  // row_shr:8
+  WMAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+  WMAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef WMAX_STEP
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
 static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w) {
   GemvWork wk;
   const int n_sh = a.n_sh_blocks;
@@ -648,36 +665,40 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   }
   if (publisher && w != 0) { wk.m = 0; wk.row0 = 0; wk.base = nullptr; return wk; }
   const float NEG = -__builtin_inff();
-  float v[4];
-  int rank[4];
+  float v[4], v0[4];
   unsigned long long ptrs[4];  // slot addresses of the lane's candidates, fetched alongside the logits
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int e = lane + 64 * r;
     v[r] = (e < E) ? a.r_logits[e] : NEG;
+    v0[r] = v[r];
     ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
-    rank[r] = 0;
   }
+  unsigned long long msel[4] = {0ull, 0ull, 0ull, 0ull};
+  float mx = 0.f, sum_sel = 0.f, my_v = 0.f;  // the last three only matter to the publisher
+  int my_e = 0;
+  for (int j = 0; j < k; ++j) {
+    float bv = v[0];
 #pragma unroll
-  for (int r2 = 0; r2 < 4; ++r2) {
-    if (64 * r2 < E) {
-#pragma unroll 16
-      for (int i = 0; i < 64; ++i) {
-        const float o = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[r2]), i));
-        const int oe = i + 64 * r2;
+    for (int r = 1; r < 4; ++r) bv = fmaxf(bv, v[r]);
+    const float best = wave_max_f32(bv);
+    // the lowest expert id holding the maximum: lowest column r first, then lowest lane
+    int wr = -1, wl = 0;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          if (64 * r < E) {  // uniform: only the logit columns that exist are ranked
-            const int e = lane + 64 * r;
-            rank[r] += (o > v[r] || (o == v[r] && oe < e)) ? 1 : 0;
-          }
-        }
-      }
+    for (int r = 0; r < 4; ++r) {
+      const unsigned long long mr = __ballot(v[r] == best);
+      if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
     }
-  }
-  unsigned long long msel[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) msel[r] = __ballot(lane + 64 * r < E && rank[r] < k);
+    for (int r = 0; r < 4; ++r)
+      if (r == wr) {
+        if (lane == wl) v[r] = NEG;
+        msel[r] |= 1ull << wl;
+      }
+    if (j == 0) mx = best;
+    sum_sel += expf(best - mx);
+    if (lane == j) { my_v = best; my_e = wl + 64 * wr; }
+  }
   // unit u = the u-th smallest selected id
   int cum = 0;
   bool found = false;
@@ -698,31 +719,12 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   wk.m = 1; wk.row0 = u;
   wk.base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
 
-  if (publisher) {  // publish the routing: body of k_topk (weights) and k_dispatch (T = 1)
+  if (publisher) {  // publish the routing: weights as in k_topk, arrays as in k_dispatch (T = 1)
     wk.m = 0;       // no weight tiles for this workgroup
-    // selected logits in choice order (lane j keeps choice j); the row maximum is choice 0
-    float mx = 0.f, sum_sel = 0.f, my_v = 0.f;
-    int my_e = 0;
-#pragma unroll 1
-    for (int j = 0; j < k; ++j) {
-      float val = 0.f; int ee = 0;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const unsigned long long mj = __ballot(lane + 64 * r < E && rank[r] == j);
-        if (mj) {
-          const int src = (int)__builtin_ctzll(mj);
-          val = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[r]), src));
-          ee = src + 64 * r;
-        }
-      }
-      if (j == 0) mx = val;
-      sum_sel += expf(val - mx);
-      if (lane == j) { my_v = val; my_e = ee; }
-    }
     float den = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      if (lane + 64 * r < E) den += expf(v[r] - mx);
+      if (lane + 64 * r < E) den += expf(v0[r] - mx);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
     const float ex = expf(my_v - mx);
