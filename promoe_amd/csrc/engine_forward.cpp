@@ -28,7 +28,18 @@ struct LayerState {
   hipEvent_t ev = nullptr;
   int sub_cursor = 0;
   // routing results of calls that ran without a host round trip, accounted later
-  struct Pending { int layer = -1, max_units = 0; hipEvent_t ev = nullptr; moe_unit *units = nullptr; int *n_active = nullptr; bool busy = false; };
+  struct Pending {
+    int layer = -1, max_units = 0;
+    hipEvent_t ev = nullptr;
+    moe_unit *units = nullptr;
+    int *n_active = nullptr;
+    bool busy = false;
+    // routing stored by the kernel itself into `units`: ready when *seq == seq_expected (no event)
+    int *seq = nullptr;
+    int seq_expected = 0;
+    bool by_seq = false;
+  };
+  int seq_counter = 0;
   static const int kPending = 8;
   Pending pend[kPending];
   int pend_head = 0;
@@ -133,6 +144,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   for (auto &p : s->pend) {
     rc |= halloc(s, &p.units, s->max_units);
     rc |= halloc(s, &p.n_active, 1);
+    rc |= halloc(s, &p.seq, 1);
+    if (p.seq) *p.seq = 0;
     if (hipEventCreateWithFlags(&p.ev, hipEventDisableTiming) != hipSuccess) rc = 1;
   }
   if (rc) return MOE_EHIP;
@@ -148,7 +161,16 @@ int moe_forward_harvest(moe_engine *eng, bool wait) {
   for (int i = 0; i < LayerState::kPending; ++i) {
     LayerState::Pending &p = s->pend[(s->pend_head + i) % LayerState::kPending];  // oldest first
     if (!p.busy) continue;
-    if (wait) { if (hipEventSynchronize(p.ev) != hipSuccess) return MOE_EHIP; }
+    if (p.by_seq) {
+      volatile int *sq = p.seq;
+      if (*sq != p.seq_expected) {
+        if (!wait) break;
+        // the launch that writes it is already in the compute stream
+        if (hipStreamSynchronize((hipStream_t)eng->be->compute_stream()) != hipSuccess) return MOE_EHIP;
+        if (*sq != p.seq_expected) { moe_set_error("routing of layer %d never reached the host", p.layer); return MOE_EHIP; }
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    } else if (wait) { if (hipEventSynchronize(p.ev) != hipSuccess) return MOE_EHIP; }
     else if (hipEventQuery(p.ev) != hipSuccess) { (void)hipGetLastError(); break; }
     const int n = std::min(*p.n_active, p.max_units);
     if (int rc = engine_account_hits(eng, p.layer, p.units, n)) return rc;
@@ -223,18 +245,18 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
-    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
-                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
-                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, st)))
-      return rc;
     LayerState::Pending &p = s->pend[s->pend_head];
     if (p.busy && (rc = moe_forward_harvest(eng, true))) return rc;
     s->pend_head = (s->pend_head + 1) % LayerState::kPending;
-    HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
-    HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
-    HIPC(hipEventRecord(p.ev, st));
-    p.layer = layer; p.max_units = max_units; p.busy = true;
+    // the kernel stores the unit list into the pending slot's pinned memory and then the sequence word
+    const int seq = ++s->seq_counter;
+    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, p.units, p.seq, seq, st)))
+      return rc;
+    *p.n_active = k;
+    p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
       return rc;
@@ -272,7 +294,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
     HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
     HIPC(hipEventRecord(p.ev, st));
-    p.layer = layer; p.max_units = max_units; p.busy = true;
+    p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = false;
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;

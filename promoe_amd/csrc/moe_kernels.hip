@@ -538,6 +538,8 @@ struct GemvArgs {
   int *r_idx; float *r_w;
   int *r_counts, *r_offsets, *r_sorted_pair, *r_pos_of_pair, *r_sorted_tok;
   moe_unit *r_units; int *r_n_active; long long *r_active_ids;
+  // optional copy of the unit list straight into pinned host memory, then a sequence word
+  moe_unit *r_host_units; int *r_host_seq; int r_host_seq_val, r_pad2;
 };
 
 // global-address-space loads (pointers that come out of the slot table are generic
@@ -753,6 +755,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
       moe_unit un; un.expert = my_e; un.m = 1; un.row0 = pos; un.pad = 0;
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
+      if (a.r_host_units) a.r_host_units[pos] = un;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -764,6 +767,10 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
       }
     }
     if (lane == 0) { a.r_offsets[E] = k; *a.r_n_active = k; }
+    if (a.r_host_seq) {  // the host polls the sequence word: units first, system-scope fence, then the word
+      __threadfence_system();
+      if (lane == 0) __hip_atomic_store(a.r_host_seq, a.r_host_seq_val, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
   return wk;
 }
@@ -1507,7 +1514,8 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
                                      int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
                                      float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
-                                     void *h_r, void *h_s, float *part_r, float *part_s, int *err, void *stream) {
+                                     void *h_r, void *h_s, float *part_r, float *part_s, int *err,
+                                     moe_unit *units_host_out, int *seq_host_out, int seq_value, void *stream) {
   if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
       !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
       mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
@@ -1528,6 +1536,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.r_logits = logits; a.r_E = E; a.r_k = k; a.r_mode = mode; a.r_idx = idx; a.r_w = w; a.r_counts = counts;
   a.r_offsets = offsets; a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok;
   a.r_units = units; a.r_n_active = n_active; a.r_active_ids = (long long *)active_ids;
+  a.r_host_units = units_host_out; a.r_host_seq = units_host_out ? seq_host_out : nullptr; a.r_host_seq_val = seq_value;
   // pass 1: w13 + SwiGLU, routing derived in the kernel
   a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, 0, I_sh, I_sh / 16, 0};
   a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
