@@ -120,6 +120,16 @@ int moe_route_decode(const void *x_bf16, const void *wg_bf16, const float *bias,
                      moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
                      unsigned *counter, void *stream);
 
+/* k1b + k2 in one launch (one workgroup) for decode batches: T <= 16, E <= 256, T*k <= 512; same
+ * results, bit for bit, as moe_topk + moe_dispatch.  units_host_out / n_active_host_out /
+ * seq_host_out (optional, pinned HOST memory): the kernel also stores the unit list and its length
+ * there and then, behind a system-scope fence, seq_value into *seq_host_out. */
+int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mode, int *idx, float *w,
+                      int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
+                      moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
+                      moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
+                      void *stream);
+
 /* k3 (decode): int4 grouped SwiGLU expert product through the slot table.
  *   expert_ptr[e] : device address of expert e's slot (0 = not resident -> *err |= 1)
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL

@@ -264,7 +264,28 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     return moe_layer_done(eng, layer);
   }
   static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
-  if (fused_route && T <= 2 && E <= 256 && T * k <= 512) {
+  bool routed_by_tail = false;
+  int tail_seq = 0;
+  if (all_resident && fused_route && T <= 16 && E <= 256 && T * k <= 512) {
+    // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
+    // also hands the unit list to the host through the next pending slot's pinned memory
+    if (!d.gate_bias) {
+      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+    } else {
+      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+      if (d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    }
+    LayerState::Pending &pn = s->pend[s->pend_head];
+    if (pn.busy && (rc = moe_forward_harvest(eng, true))) return rc;
+    tail_seq = ++s->seq_counter;
+    if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
+                                s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                max_units, pn.units, pn.n_active, pn.seq, tail_seq, st)))
+      return rc;
+    routed_by_tail = true;
+  } else if (fused_route && T <= 2 && E <= 256 && T * k <= 512) {
     // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
     // single workgroup behind a device-scope counter, which beats two more launches only
     // while that tail is short (measured: +5 % tokens/s at T=1, -2 % at T=4, -25 % at T=16)
@@ -291,10 +312,15 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     LayerState::Pending &p = s->pend[s->pend_head];
     if (p.busy && (rc = moe_forward_harvest(eng, true))) return rc;
     s->pend_head = (s->pend_head + 1) % LayerState::kPending;
-    HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
-    HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
-    HIPC(hipEventRecord(p.ev, st));
-    p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = false;
+    p.layer = layer; p.max_units = max_units; p.busy = true;
+    if (routed_by_tail) {  // the routing kernel stores the unit list in the slot's pinned memory itself
+      p.by_seq = true; p.seq_expected = tail_seq;
+    } else {
+      HIPC(hipMemcpyAsync(p.units, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
+      HIPC(hipMemcpyAsync(p.n_active, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
+      HIPC(hipEventRecord(p.ev, st));
+      p.by_seq = false;
+    }
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;

@@ -330,56 +330,21 @@ struct RouteArgs {
   int *counts, *offsets, *sorted_pair, *pos_of_pair, *sorted_tok;
   moe_unit *units; int *n_active; long long *active_ids;
   unsigned *counter;
+  moe_unit *host_units; int *host_n_active; int *host_seq; int host_seq_val, pad_;
 };
 
-__global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
-  __shared__ int s_last;
-  __shared__ int s_idx[ROUTE_MAXP];
-  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[4 * 256];
-  __shared__ int s_wsum[4], s_wact[4], s_tot;
+// top-k (one wave per token) and stable dispatch by ONE workgroup of NW waves; the bodies of
+// k_topk and k_dispatch.  With host_units set the unit list also goes straight into pinned host
+// memory, followed behind a system-scope fence by the sequence word the host polls.
+template <int NW>
+static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx, int *s_cnt, int *s_off, int *s_run,
+                                                  int *s_w, int *s_wsum, int *s_wact, int &s_tot) {
+  constexpr int NT = NW * 64;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int H = a.H, E = a.E, T = a.T, k = a.k, P = T * k;
-  // ---- phase 1: one wave per (token, gate row) ------------------------------------------
-  {
-    const int e = blockIdx.x * 4 + w, t = blockIdx.y;
-    if (e < a.Erows) {
-      const uint16_t *xr = a.x + (size_t)t * H;
-      const uint16_t *wr = a.wg + (size_t)e * H;
-      float acc = 0.f;
-      for (int c = 0; c < H; c += 512) {
-        const int kk = c + 8 * lane;
-        if (kk < H) {
-          const uint4 xv = *(const uint4 *)(xr + kk);
-          const uint4 wv = *(const uint4 *)(wr + kk);
-          acc = fmaf(bf16lo(xv.x), bf16lo(wv.x), acc);
-          acc = fmaf(bf16hi(xv.x), bf16hi(wv.x), acc);
-          acc = fmaf(bf16lo(xv.y), bf16lo(wv.y), acc);
-          acc = fmaf(bf16hi(xv.y), bf16hi(wv.y), acc);
-          acc = fmaf(bf16lo(xv.z), bf16lo(wv.z), acc);
-          acc = fmaf(bf16hi(xv.z), bf16hi(wv.z), acc);
-          acc = fmaf(bf16lo(xv.w), bf16lo(wv.w), acc);
-          acc = fmaf(bf16hi(xv.w), bf16hi(wv.w), acc);
-        }
-      }
-#pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
-      if (lane == 0) a.logits[(size_t)t * a.ldl + e] = (a.bias && e < E) ? acc + a.bias[e] : acc;
-    }
-  }
-  // ---- who is last? ------------------------------------------------------------------------
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) {
-    const unsigned prev = atomicAdd(a.counter, 1u);
-    s_last = prev == gridDim.x * gridDim.y - 1u;
-  }
-  __syncthreads();
-  if (!s_last) return;
-  if (tid == 0) atomicExch(a.counter, 0u);
-  __threadfence();
-  // ---- phase 2: top-k, wave w takes tokens w, w+4, ... (body of k_topk) ----------------------
+  const int E = a.E, T = a.T, k = a.k, P = T * k;
+  // ---- phase 2: top-k, wave w takes tokens w, w+NW, ... (body of k_topk) ----------------------
   const float NEG = -__builtin_inff();
-  for (int t = w; t < T; t += 4) {
+  for (int t = w; t < T; t += NW) {
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -427,10 +392,10 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
     }
     if (lane < k) a.w[(size_t)t * k + lane] = wgt;
   }
-  // ---- phase 3: dispatch (k_dispatch with 256 threads; thread e owns expert e) -------------
+  // ---- phase 3: dispatch (k_dispatch with NW waves; thread e owns expert e) -------------
   if (tid < E) { s_cnt[tid] = 0; s_run[tid] = 0; }
   __syncthreads();
-  for (int p = tid; p < P; p += 256) atomicAdd(&s_cnt[s_idx[p]], 1);
+  for (int p = tid; p < P; p += NT) atomicAdd(&s_cnt[s_idx[p]], 1);
   __syncthreads();
   {
     const int c = (tid < E) ? s_cnt[tid] : 0;
@@ -454,24 +419,26 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
         moe_unit u; u.expert = tid; u.m = c; u.row0 = excl; u.pad = 0;
         a.units[uidx] = u;
         a.active_ids[uidx] = tid;
+        if (a.host_units) a.host_units[uidx] = u;
       }
     }
-    if (tid == 255) {
+    if (tid == NT - 1) {
       const int tot_act = ba + sa;
       a.offsets[E] = bc + sc;
       *a.n_active = tot_act < a.max_units ? tot_act : a.max_units;
+      if (a.host_units) *a.host_n_active = tot_act < a.max_units ? tot_act : a.max_units;
       s_tot = tot_act;
     }
     __syncthreads();
-    for (int u = s_tot + tid; u < a.max_units; u += 256) {
+    for (int u = s_tot + tid; u < a.max_units; u += NT) {
       moe_unit z; z.expert = -1; z.m = 0; z.row0 = 0; z.pad = 0;
       a.units[u] = z;
       a.active_ids[u] = -1;
     }
   }
   __syncthreads();
-  for (int base = 0; base < P; base += 256) {
-    for (int i = tid; i < 4 * E; i += 256) s_w[i] = 0;
+  for (int base = 0; base < P; base += NT) {
+    for (int i = tid; i < NW * E; i += NT) s_w[i] = 0;
     __syncthreads();
     const int p = base + tid;
     const int e = (p < P) ? s_idx[p] : -1;
@@ -487,7 +454,7 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
     __syncthreads();
     if (tid < E) {
       int run = s_run[tid];
-      for (int ww = 0; ww < 4; ++ww) {
+      for (int ww = 0; ww < NW; ++ww) {
         const int c = s_w[ww * E + tid];
         s_w[ww * E + tid] = run;
         run += c;
@@ -503,6 +470,67 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
     }
     __syncthreads();
   }
+  if (a.host_units) {
+    __threadfence_system();
+    __syncthreads();
+    if (tid == 0) __hip_atomic_store(a.host_seq, a.host_seq_val, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
+}
+
+__global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
+  __shared__ int s_last;
+  __shared__ int s_idx[ROUTE_MAXP];
+  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[4 * 256];
+  __shared__ int s_wsum[4], s_wact[4], s_tot;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int H = a.H, E = a.E, T = a.T, k = a.k, P = T * k;
+  // ---- phase 1: one wave per (token, gate row) ------------------------------------------
+  {
+    const int e = blockIdx.x * 4 + w, t = blockIdx.y;
+    if (e < a.Erows) {
+      const uint16_t *xr = a.x + (size_t)t * H;
+      const uint16_t *wr = a.wg + (size_t)e * H;
+      float acc = 0.f;
+      for (int c = 0; c < H; c += 512) {
+        const int kk = c + 8 * lane;
+        if (kk < H) {
+          const uint4 xv = *(const uint4 *)(xr + kk);
+          const uint4 wv = *(const uint4 *)(wr + kk);
+          acc = fmaf(bf16lo(xv.x), bf16lo(wv.x), acc);
+          acc = fmaf(bf16hi(xv.x), bf16hi(wv.x), acc);
+          acc = fmaf(bf16lo(xv.y), bf16lo(wv.y), acc);
+          acc = fmaf(bf16hi(xv.y), bf16hi(wv.y), acc);
+          acc = fmaf(bf16lo(xv.z), bf16lo(wv.z), acc);
+          acc = fmaf(bf16hi(xv.z), bf16hi(wv.z), acc);
+          acc = fmaf(bf16lo(xv.w), bf16lo(wv.w), acc);
+          acc = fmaf(bf16hi(xv.w), bf16hi(wv.w), acc);
+        }
+      }
+#pragma unroll
+      for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
+      if (lane == 0) a.logits[(size_t)t * a.ldl + e] = (a.bias && e < E) ? acc + a.bias[e] : acc;
+    }
+  }
+  // ---- who is last? ------------------------------------------------------------------------
+  __threadfence();
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned prev = atomicAdd(a.counter, 1u);
+    s_last = prev == gridDim.x * gridDim.y - 1u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  if (tid == 0) atomicExch(a.counter, 0u);
+  __threadfence();
+  route_tail<4>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
+}
+
+// k1b + k2 in one launch for decode batches whose logits exist already: one workgroup of 16 waves
+__global__ __launch_bounds__(1024) void k_topk_dispatch(const RouteArgs a) {
+  __shared__ int s_idx[ROUTE_MAXP];
+  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[16 * 256];
+  __shared__ int s_wsum[16], s_wact[16], s_tot;
+  route_tail<16>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
 }
 
 // ---------------------------------------------------------------------------
@@ -1643,10 +1671,37 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
   a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
   a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
   a.counter = counter;
+  a.host_units = nullptr; a.host_n_active = nullptr; a.host_seq = nullptr; a.host_seq_val = 0; a.pad_ = 0;
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_route_decode, dim3((E_rows + 3) / 4, T), dim3(256), 0, (hipStream_t)stream, a);
   moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
   return moe_check_launch("k_route_decode");
+}
+
+extern "C" int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mode, int *idx, float *w,
+                                 int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
+                                 moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
+                                 moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
+                                 void *stream) {
+  if (!logits || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok || !units ||
+      !n_active || !active_ids || T <= 0 || T > ROUTE_MAXT || E <= 0 || E > 256 || ldl < E || k <= 0 || k > 32 ||
+      k > E || T * k > ROUTE_MAXP || mode < 0 || mode > 2 || max_units < 0 ||
+      (units_host_out && (!n_active_host_out || !seq_host_out))) {
+    moe_set_error("moe_topk_dispatch: bad argument (T=%d E=%d k=%d)", T, E, k);
+    return MOE_EINVAL;
+  }
+  RouteArgs a;
+  memset(&a, 0, sizeof a);
+  a.logits = (float *)logits; a.T = T; a.E = E; a.Erows = E; a.ldl = ldl; a.k = k; a.mode = mode;
+  while ((1 << a.nbits) < E) ++a.nbits;
+  a.max_units = max_units; a.idx = idx; a.w = w; a.counts = counts; a.offsets = offsets;
+  a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
+  a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
+  a.host_units = units_host_out; a.host_n_active = n_active_host_out; a.host_seq = seq_host_out; a.host_seq_val = seq_value;
+  moe_ktimer_begin(MOE_K_TOPK, (hipStream_t)stream);
+  hipLaunchKernelGGL(k_topk_dispatch, dim3(1), dim3(1024), 0, (hipStream_t)stream, a);
+  moe_ktimer_end(MOE_K_TOPK, (hipStream_t)stream);
+  return moe_check_launch("k_topk_dispatch");
 }
 
 extern "C" int moe_combine(const float *part_r, const float *part_s, const float *topk_w,

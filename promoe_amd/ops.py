@@ -67,6 +67,19 @@ def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispa
     return d
 
 
+def topk_dispatch(logits: torch.Tensor, k: int, E: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
+    """Top-k and dispatch in one launch for T <= 16.  Returns (idx, w, Dispatch)."""
+    T = logits.shape[0]
+    idx = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    d = Dispatch(T, k, E, min(E, T * k), logits.device)
+    check(lib.moe_topk_dispatch(ptr(_dev(logits)), T, E, logits.stride(0), k, mode, ptr(idx), ptr(w), ptr(d.counts),
+                                ptr(d.offsets), ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                ptr(d.n_active), ptr(d.active_ids), d.max_units, 0, 0, 0, 0, cur_stream()),
+          "moe_topk_dispatch")
+    return idx, w, d
+
+
 _route_counter = {}
 
 

@@ -237,3 +237,21 @@ def test_token_decode_routes_in_kernel_like_separate_kernels(cuda, H, I, E, k, m
         na = int(d.n_active.cpu()[0])
         assert torch.equal(d.units[:na], d2.units[:na]) and torch.equal(d.active_ids[:na], d2.active_ids[:na])
         assert torch.equal(y_ref, y)
+
+
+@pytest.mark.parametrize("T,E,k,mode", [(1, 64, 6, 0), (4, 64, 6, 0), (16, 64, 6, 1), (16, 60, 4, 2), (7, 200, 8, 0),
+                                        (16, 8, 2, 2), (3, 256, 32, 0)])
+def test_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode):
+    from promoe_amd import ops
+    print(f"case topk_dispatch T={T} E={E} k={k} mode={mode}", flush=True)
+    rng = np.random.default_rng(T * 131 + E + k)
+    logits = rng.normal(0, 2, (T, E + 1)).astype(np.float32)
+    logits[:, E // 2] = logits[:, 1]          # ties
+    lg = torch.from_numpy(logits).to(cuda)
+    idx, w = ops.topk(lg, k, mode, E=E)
+    d = ops.dispatch(idx, E)
+    idx2, w2, d2 = ops.topk_dispatch(lg[:, :E] if False else lg, k, E, mode) if False else ops.topk_dispatch(lg, k, E, mode)
+    torch.cuda.synchronize()
+    assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+    for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active", "units", "active_ids"):
+        assert torch.equal(getattr(d, name), getattr(d2, name)), name
