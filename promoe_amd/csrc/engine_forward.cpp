@@ -6,6 +6,7 @@
 // resident go out as ONE grouped launch, missed experts follow one by one as their
 // copies land (the returned order of report_one_layer), then combine.
 #include <algorithm>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 
@@ -23,7 +24,8 @@ struct LayerState {
   void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
   // pinned host mirrors
   moe_unit *units_host = nullptr, *units_sub_host = nullptr;
-  int *n_active_host = nullptr, *err_host = nullptr;
+  int *n_active_host = nullptr, *err_host = nullptr, *opt_seq = nullptr;
+  int *err_opt = nullptr;  // error word of launches that are allowed to meet non-resident experts
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
   int sub_cursor = 0;
@@ -141,6 +143,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
   rc |= halloc(s, &s->n_active_host, 1);
   rc |= halloc(s, &s->err_host, 1);
+  rc |= halloc(s, &s->opt_seq, 1);
+  rc |= dalloc(s, &s->err_opt, 1);
   for (auto &p : s->pend) {
     rc |= halloc(s, &p.units, s->max_units);
     rc |= halloc(s, &p.n_active, 1);
@@ -151,6 +155,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   if (rc) return MOE_EHIP;
   HIPC(hipMemset(s->err, 0, sizeof(int)));
   HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
+  HIPC(hipMemset(s->err_opt, 0, sizeof(int)));
+  *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
   return MOE_OK;
 }
@@ -259,6 +265,89 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
+      return rc;
+    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    return moe_layer_done(eng, layer);
+  }
+  // One token, demand fetching only (no prefetch producer that could evict behind our back) and the
+  // fetch thread idle: start the expert kernels on whatever is resident BEFORE the host knows the
+  // routing.  The w13 kernel routes by itself, skips experts whose table entry is 0 and hands the unit
+  // list to the host through pinned memory; the host then runs the cache hooks in the reference's
+  // order (hits were computed already, misses are fetched and computed one by one) while the GPU works.
+  bool optimistic = false;
+  if (!all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && eng->cfg.early_preempt &&
+      eng->cfg.reorder_experts && eng->cfg.num_predict_expert_per_layer == 0 && !eng->predictor_attached &&
+      (size_t)d.H * 2 + 8192 <= 60 * 1024) {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    optimistic = eng->current.e == nullptr && eng->precise_q.empty();
+    for (auto &q : eng->layer_q) optimistic = optimistic && q.empty();
+  }
+  if (optimistic) {
+    if (!d.gate_bias) {
+      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+    } else {
+      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+      if (d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    }
+    const uint64_t *table = nullptr;
+    if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    // what the kernel will find resident: exactly these experts get computed by it
+    std::vector<char> resident_at_launch(E);
+    {
+      std::lock_guard<std::mutex> lk(eng->mu);
+      for (int e = 0; e < E; ++e) resident_at_launch[e] = eng->h_table[(size_t)layer * E + e] != 0;
+    }
+    const int seq = ++s->seq_counter;
+    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->units_host, s->opt_seq, seq, st)))
+      return rc;
+    {  // the routing arrives a few microseconds after the kernel starts
+      volatile int *sq = s->opt_seq;
+      const auto t0 = std::chrono::steady_clock::now();
+      unsigned spins = 0;
+      while (*sq != seq) {
+        if ((++spins & 1023u) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
+          HIPC(hipStreamSynchronize(st));
+          if (*sq != seq) { moe_set_error("routing of layer %d never reached the host", layer); return MOE_EHIP; }
+        }
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    }
+    const int n_act = k;
+    std::vector<int64_t> ids(n_act);
+    std::unordered_map<int, moe_unit> unit_of;
+    for (int u = 0; u < n_act; ++u) { ids[u] = s->units_host[u].expert; unit_of[s->units_host[u].expert] = s->units_host[u]; }
+    if ((rc = moe_report_one_layer(eng, layer, ids.data(), n_act))) return rc;
+    std::vector<int64_t> later, now_ids;
+    {
+      std::lock_guard<std::mutex> lk(eng->mu);
+      for (int i = 0; i < n_act; ++i) {
+        // resident at launch: computed already (and a hit, since nothing could evict it in between);
+        // a missed expert whose copy has landed meanwhile is `launching` too, but still has to be computed
+        if (resident_at_launch[(int)ids[i]]) now_ids.push_back(ids[i]);
+        else later.push_back(ids[i]);
+      }
+      eng->ctr.ready += (uint64_t)now_ids.size();
+    }
+    if (!now_ids.empty() && (rc = moe_release_experts(eng, layer, now_ids.data(), (int64_t)now_ids.size()))) return rc;
+    s->sub_cursor = 0;
+    for (int64_t id : later) {
+      if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
+      if ((rc = moe_flush_table(eng, layer, st))) return rc;
+      moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
+      *slot_h = unit_of[(int)id];
+      HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
+      if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
+      s->sub_cursor++;
+      if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
+    }
+    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
+    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
       return rc;
     if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);

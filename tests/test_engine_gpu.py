@@ -226,3 +226,39 @@ def test_patched_module_mirror_matches_oracle(cuda, fused):
     for key in ("hit", "miss", "evictions"):
         assert c[key] == sim.ctr[key], key
     pm.close()
+
+
+def test_forward_single_token_starts_before_the_host_knows_the_routing(cuda):
+    """Demand fetching only (no prefetch producer): a one-token forward launches the self-routing
+    expert kernel on whatever is resident, learns the routing from pinned memory and serves the
+    misses afterwards.  Outputs, residency and counters must still follow the reference logic."""
+    print("case engine_forward optimistic", flush=True)
+    Lyr, E, k = 3, 16, 4
+    layers = [Int4Layer(H=256, I=384, E=E, I_sh=256, seed=50 + l, zipf=1.2) for l in range(Lyr)]
+    cfg = dict(cache_rate=0.375, cache_policy="lru", num_predict_expert_per_layer=0, reorder_experts=True,
+               early_preempt=True)
+    pm = build_engine(layers, k, cuda, **cfg)
+    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy="lru", num_predict=0, reorder=True, early_preempt=True)
+    worst = 0.0
+    for step in range(12):
+        T = 1 if step % 5 else 3          # mostly single tokens, a few small batches in between
+        for l in range(Lyr):
+            x = O.synth_acts(T, 256, seed=400 + step * Lyr + l)
+            y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            ref = ref_forward(layers[l], x, k, 0)
+            err = np.abs(y.float().cpu().numpy() - ref["out"]).max() / np.abs(ref["out"]).max()
+            worst = max(worst, err)
+            assert err <= TOL, (step, l, T, err)
+            ids = sim.report_one_layer(l, np.unique(ref["idx"]))
+            for e in ids:
+                sim.wait_expert(l, e); sim.expert_launched(l, e)
+            sim.drain()
+            pm.drain()
+            assert [e for e in range(E) if pm.is_in_cache(l, e)] == sim.resident(l), (step, l)
+    c = pm.counters()
+    print(f"  worst max-rel-err {worst:.3e}; counters {c}", flush=True)
+    for key in ("hit", "miss", "evictions", "activated"):
+        assert c[key] == sim.ctr[key], key
+    assert c["miss"] > 0 and c["hit"] > 0 and c["evictions"] > 0
+    pm.close()
