@@ -55,6 +55,32 @@ __global__ __launch_bounds__(256) void k_gate_logits(const uint16_t *__restrict_
   const uint16_t *xr = x + (size_t)t * H;
   const uint16_t *wr = wg + (size_t)e * H;
   float acc = 0.f;
+  if (H <= 4096) {
+    // all loads of the row first (one round trip), then the same fma chain in the same order
+    uint4 xq[8], wq[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int k = c * 512 + 8 * lane;
+      if (k < H) {
+        xq[c] = *(const uint4 *)(xr + k);
+        wq[c] = *(const uint4 *)(wr + k);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int k = c * 512 + 8 * lane;
+      if (k < H) {
+        acc = fmaf(bf16lo(xq[c].x), bf16lo(wq[c].x), acc);
+        acc = fmaf(bf16hi(xq[c].x), bf16hi(wq[c].x), acc);
+        acc = fmaf(bf16lo(xq[c].y), bf16lo(wq[c].y), acc);
+        acc = fmaf(bf16hi(xq[c].y), bf16hi(wq[c].y), acc);
+        acc = fmaf(bf16lo(xq[c].z), bf16lo(wq[c].z), acc);
+        acc = fmaf(bf16hi(xq[c].z), bf16hi(wq[c].z), acc);
+        acc = fmaf(bf16lo(xq[c].w), bf16lo(wq[c].w), acc);
+        acc = fmaf(bf16hi(xq[c].w), bf16hi(wq[c].w), acc);
+      }
+    }
+  } else
   for (int c = 0; c < H; c += 512) {
     const int k = c + 8 * lane;
     if (k < H) {
