@@ -1229,12 +1229,26 @@ __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_
   const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   if (n >= H) return;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int j = 0; j < k; ++j) {
-    const float wj = topk_w[(size_t)t * k + j];
-    const int pos = pos_of_pair[(size_t)t * k + j];
-    const float4 v = *(const float4 *)(part_r + (size_t)pos * H + n);
-    acc.x = fmaf(wj, v.x, acc.x); acc.y = fmaf(wj, v.y, acc.y);
-    acc.z = fmaf(wj, v.z, acc.z); acc.w = fmaf(wj, v.w, acc.w);
+  // eight partial rows at a time: positions and weights first, then the rows, then the
+  // fma chain in pair order (two round trips per eight rows instead of two per row)
+  for (int j0 = 0; j0 < k; j0 += 8) {
+    float wj[8];
+    int pos[8];
+    float4 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int jj = j0 + j < k ? j0 + j : k - 1;
+      wj[j] = topk_w[(size_t)t * k + jj];
+      pos[j] = pos_of_pair[(size_t)t * k + jj];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = *(const float4 *)(part_r + (size_t)pos[j] * H + n);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j0 + j < k) {
+        acc.x = fmaf(wj[j], v[j].x, acc.x); acc.y = fmaf(wj[j], v[j].y, acc.y);
+        acc.z = fmaf(wj[j], v[j].z, acc.z); acc.w = fmaf(wj[j], v[j].w, acc.w);
+      }
   }
   if (part_s) {
     const float g = sg_logit ? 1.f / (1.f + expf(-sg_logit[(size_t)t * sg_stride])) : 1.f;
