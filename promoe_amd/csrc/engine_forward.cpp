@@ -19,6 +19,7 @@ struct LayerState {
   int *idx = nullptr, *counts = nullptr, *offsets = nullptr, *sorted_pair = nullptr, *pos_of_pair = nullptr,
       *sorted_tok = nullptr, *n_active = nullptr, *err = nullptr;
   unsigned *route_counter = nullptr;
+  unsigned char *unit_ws = nullptr;  // resolved units of the one-token path (16 bytes each)
   moe_unit *units = nullptr, *units_sub = nullptr;
   int64_t *active_ids = nullptr;
   void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
@@ -131,6 +132,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->n_active, 1);
   rc |= dalloc(s, &s->err, 1);
   rc |= dalloc(s, &s->route_counter, 1);
+  rc |= dalloc(s, &s->unit_ws, (size_t)16 * std::max(k, 1));
   rc |= dalloc(s, &s->units, s->max_units);
   rc |= dalloc(s, &s->units_sub, (size_t)s->max_units * 2);
   rc |= dalloc(s, &s->active_ids, s->max_units);
@@ -259,7 +261,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, p.units, p.seq, seq, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq, st)))
       return rc;
     *p.n_active = k;
     p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
@@ -304,7 +306,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->units_host, s->opt_seq, seq, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, st)))
       return rc;
     {  // the routing arrives a few microseconds after the kernel starts
       volatile int *sq = s->opt_seq;

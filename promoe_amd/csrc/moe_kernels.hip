@@ -594,6 +594,8 @@ struct GemvArgs {
   moe_unit *r_units; int *r_n_active; long long *r_active_ids;
   // optional copy of the unit list straight into pinned host memory, then a sequence word
   moe_unit *r_host_units; int *r_host_seq; int r_host_seq_val, r_pad2;
+  KUnit *r_kunits;              // routing publisher: resolved units (slot address, rows) for the w2 pass
+  const KUnit *kunits_dev;      // device-side resolved units: one load instead of unit -> table -> address
 };
 
 // global-address-space loads (pointers that come out of the slot table are generic
@@ -651,9 +653,15 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
     if (sh) {
       wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
     } else {
-      const moe_unit ud = a.units[u];
-      wk.m = ud.m; wk.row0 = ud.row0;
-      wk.base = ud.m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
+      if (a.kunits_dev) {
+        const KUnit kd = a.kunits_dev[u];
+        wk.m = kd.m; wk.row0 = kd.row0;
+        wk.base = (const unsigned char *)kd.base;
+      } else {
+        const moe_unit ud = a.units[u];
+        wk.m = ud.m; wk.row0 = ud.row0;
+        wk.base = ud.m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
+      }
     }
   } else {
     // the first 8 units sit at fixed argument offsets: fetched with the rest, picked by scalar selects
@@ -810,6 +818,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
       if (a.r_host_units) a.r_host_units[pos] = un;
+      if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; }
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -1583,7 +1592,8 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
                                      float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
-                                     moe_unit *units_host_out, int *seq_host_out, int seq_value, void *stream) {
+                                     void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
+                                     void *stream) {
   if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
       !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
       mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
@@ -1605,6 +1615,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.r_offsets = offsets; a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok;
   a.r_units = units; a.r_n_active = n_active; a.r_active_ids = (long long *)active_ids;
   a.r_host_units = units_host_out; a.r_host_seq = units_host_out ? seq_host_out : nullptr; a.r_host_seq_val = seq_value;
+  a.r_kunits = (KUnit *)unit_ws;
   // pass 1: w13 + SwiGLU, routing derived in the kernel
   a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, 0, I_sh, I_sh / 16, 0};
   a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
@@ -1629,6 +1640,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z, I_sh, I_sh / 128, I_sh, H, H / 32, 0};
   a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z, I, I / 128, I, H, H / 32, 0};
   a.n_sh_blocks = sh ? H / 32 : 0;
+  a.kunits_dev = (const KUnit *)unit_ws;
   grid = a.n_sh_blocks + k * (H / 32);
   return launch_gemv_t<false>(a, grid, 1, I_sh > I ? I_sh : I, I / 128, s);
 }

@@ -148,7 +148,7 @@ def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, 
                                     ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
                                     ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
                                     ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
-                                    ptr(err), 0, 0, 0, cur_stream()), "moe_decode_token_int4")
+                                    ptr(err), 0, 0, 0, 0, cur_stream()), "moe_decode_token_int4")
     return idx, w, d, part_r, part_s, err, h_r, h_s
 
 
