@@ -156,13 +156,14 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
  * address, row) there and the w2 pass starts from one load instead of unit -> table -> address.
  * units_host_out / seq_host_out (optional, pinned HOST memory): the kernel also stores the k
  * units there and then, behind a system-scope fence, seq_value into *seq_host_out, so a host
- * that polls the word gets the routing without a copy or an event. */
+ * that polls the word gets the routing without a copy or an event.
+ * phases: bit 0 = routing + w13 + SwiGLU, bit 1 = w2 (needs the units of an earlier bit-0 call). */
 int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k, int mode, int H, int I,
                           int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx, float *w,
                           int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                           moe_unit *units, int *n_active, int64_t *active_ids, void *h_r, void *h_s,
                           float *part_r, float *part_s, int *err, void *unit_ws, moe_unit *units_host_out,
-                          int *seq_host_out, int seq_value, void *stream);
+                          int *seq_host_out, int seq_value, int phases, void *stream);
 
 /* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only. */
 int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, int k,

@@ -261,7 +261,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq, 3, st)))
       return rc;
     *p.n_active = k;
     p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
@@ -306,7 +306,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, 3, st)))
       return rc;
     {  // the routing arrives a few microseconds after the kernel starts
       volatile int *sq = s->opt_seq;

@@ -711,7 +711,8 @@ static __device__ __forceinline__ float wave_max_f32(float x) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
 
-static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w) {
+template <int NR>
+static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &a, int lane, int w) {
   GemvWork wk;
   const int n_sh = a.n_sh_blocks;
   const bool sh = (int)blockIdx.x < n_sh;
@@ -729,38 +730,38 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   }
   if (publisher && w != 0) { wk.m = 0; wk.row0 = 0; wk.base = nullptr; return wk; }
   const float NEG = -__builtin_inff();
-  float v[4], v0[4];
-  unsigned long long ptrs[4];  // slot addresses of the lane's candidates, fetched alongside the logits
+  float v[NR], v0[NR];
+  unsigned long long ptrs[NR];  // slot addresses of the lane's candidates, fetched alongside the logits
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+  for (int r = 0; r < NR; ++r) {
     const int e = lane + 64 * r;
     v[r] = (e < E) ? a.r_logits[e] : NEG;
     v0[r] = v[r];
     ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
   }
-  unsigned long long msel[4] = {0ull, 0ull, 0ull, 0ull};
+  unsigned long long msel[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) msel[r] = 0ull;
   float mx = 0.f, sum_sel = 0.f, my_v = 0.f;  // the last three only matter to the publisher
   int my_e = 0;
   for (int j = 0; j < k; ++j) {
     float bv = v[0];
 #pragma unroll
-    for (int r = 1; r < 4; ++r) bv = fmaxf(bv, v[r]);
+    for (int r = 1; r < NR; ++r) bv = fmaxf(bv, v[r]);
     const float best = wave_max_f32(bv);
     // the lowest expert id holding the maximum: lowest column r first, then lowest lane
     int wr = -1, wl = 0;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < NR; ++r) {
       const unsigned long long mr = __ballot(v[r] == best);
       if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < NR; ++r)
       if (r == wr) {
         if (lane == wl) v[r] = NEG;
         msel[r] |= 1ull << wl;
       }
-    if (j == 0) mx = best;
-    sum_sel += expf(best - mx);
     if (lane == j) { my_v = best; my_e = wl + 64 * wr; }
   }
   // unit u = the u-th smallest selected id
@@ -768,7 +769,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   bool found = false;
   unsigned lo = 0, hi = 0;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+  for (int r = 0; r < NR; ++r) {
     const int cnt = __popcll(msel[r]);
     if (!found && u < cum + cnt) {
       unsigned long long mm = msel[r];
@@ -785,9 +786,14 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
 
   if (publisher) {  // publish the routing: weights as in k_topk, arrays as in k_dispatch (T = 1)
     wk.m = 0;       // no weight tiles for this workgroup
+    // sum over the selected logits in choice order (the order of k_topk), maximum = choice 0
+    mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_v), 0));
+#pragma unroll 1
+    for (int j = 0; j < k; ++j)
+      sum_sel += expf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_v), j)) - mx);
     float den = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < NR; ++r)
       if (lane + 64 * r < E) den += expf(v0[r] - mx);
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
@@ -800,14 +806,14 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
       if (a.r_mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
     }
     // dispatch of the k pairs of the one token: position = rank of the expert id among the selected
-    int below[4], cb = 0;
+    int below[NR], cb = 0;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) { below[r] = cb; cb += __popcll(msel[r]); }
+    for (int r = 0; r < NR; ++r) { below[r] = cb; cb += __popcll(msel[r]); }
     if (lane < k) {
       const int r_ = my_e >> 6, l_ = my_e & 63;
       int pos = 0;
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
+      for (int r = 0; r < NR; ++r)
         if (r == r_) pos = below[r] + __popcll(msel[r] & ((1ull << l_) - 1ull));
       a.r_idx[lane] = my_e;
       a.r_w[lane] = wgt;
@@ -821,7 +827,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
       if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < NR; ++r) {
       const int e = lane + 64 * r;
       if (e < E) {
         const bool selb = (msel[r] >> lane) & 1ull;
@@ -836,6 +842,13 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
     }
   }
   return wk;
+}
+
+static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w) {
+  // one instantiation per number of 64-wide logit columns: a 64-expert layer pays for one column only
+  if (a.r_E <= 64) return gemv_resolve_route_n<1>(a, lane, w);
+  if (a.r_E <= 128) return gemv_resolve_route_n<2>(a, lane, w);
+  return gemv_resolve_route_n<4>(a, lane, w);
 }
 
 template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false, bool ROUTE = false>
@@ -1593,7 +1606,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
                                      void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
-                                     void *stream) {
+                                     int phases, void *stream) {
   if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
       !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
       mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
@@ -1627,8 +1640,8 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
     if (ch < 1) ch = 1;
     const size_t lds = gemv_lds(1, H);
     if (lds > 64 * 1024) { moe_set_error("moe_decode_token_int4: H=%d does not fit LDS", H); return MOE_EINVAL; }
-    int rc;
-    switch (ch) {
+    int rc = MOE_OK;
+    if (phases & 1) switch (ch) {
       case 1: rc = launch_gemv_route<1>(a, grid, lds, s); break;
       case 2: rc = launch_gemv_route<2>(a, grid, lds, s); break;
       case 3: rc = launch_gemv_route<3>(a, grid, lds, s); break;
@@ -1636,6 +1649,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
     }
     if (rc) return rc;
   }
+  if (!(phases & 2)) return MOE_OK;
   // pass 2: w2 over the unit list the first pass published
   a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z, I_sh, I_sh / 128, I_sh, H, H / 32, 0};
   a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z, I, I / 128, I, H, H / 32, 0};
