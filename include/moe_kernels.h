@@ -152,18 +152,23 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
  * and publishes it for the w2 pass, moe_combine and the host, so a decode step is
  * moe_gate_logits -> moe_decode_token_int4 -> moe_combine.  E <= 256.  logits: E fp32 values.
  * Every selected expert must be resident (expert_ptr[e] != 0), else *err |= 1.
- * unit_ws (optional): 16*k bytes of device memory; the first pass leaves the resolved units (slot
+ * unit_ws (optional): 32*k bytes of device memory; the first pass leaves the resolved units (slot
  * address, row) there and the w2 pass starts from one load instead of unit -> table -> address.
  * units_host_out / seq_host_out (optional, pinned HOST memory): the kernel also stores the k
  * units there and then, behind a system-scope fence, seq_value into *seq_host_out, so a host
  * that polls the word gets the routing without a copy or an event.
- * phases: bit 0 = routing + w13 + SwiGLU, bit 1 = w2 (needs the units of an earlier bit-0 call). */
+ * phases: bit 0 = routing + w13 + SwiGLU, bit 1 = w2 into partial rows (needs the units of an
+ * earlier bit-0 call), bit 2 = w2 and the weighted combine in ONE launch, straight into y_bf16 [H]
+ * (needs unit_ws of 32*k bytes; shared_gate_logit = the shared expert's gate logit or NULL; every
+ * selected expert resident).  Bits 1 and 2 exclude each other. */
 int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k, int mode, int H, int I,
                           int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx, float *w,
                           int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                           moe_unit *units, int *n_active, int64_t *active_ids, void *h_r, void *h_s,
                           float *part_r, float *part_s, int *err, void *unit_ws, moe_unit *units_host_out,
-                          int *seq_host_out, int seq_value, int phases, void *stream);
+                          int *seq_host_out, int seq_value, int phases, const float *shared_gate_logit,
+                          void *y_bf16, void *stream);
+
 
 /* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only. */
 int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, int k,

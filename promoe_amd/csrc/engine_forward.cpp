@@ -132,7 +132,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->n_active, 1);
   rc |= dalloc(s, &s->err, 1);
   rc |= dalloc(s, &s->route_counter, 1);
-  rc |= dalloc(s, &s->unit_ws, (size_t)16 * std::max(k, 1));
+  rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
   rc |= dalloc(s, &s->units, s->max_units);
   rc |= dalloc(s, &s->units_sub, (size_t)s->max_units * 2);
   rc |= dalloc(s, &s->active_ids, s->max_units);
@@ -212,6 +212,12 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
                                  s->part_r, s->part_s, s->err, units_host, table_host, 3, st);
 }
 
+// the one-token w2 + combine kernel stages the h vectors of all units in LDS
+static bool w2c_fits(const moe_layer_desc &d, int k) {
+  const size_t n_h = (size_t)k * d.I + (size_t)d.I_sh;
+  return d.H % 16 == 0 && n_h * 2 + (n_h / 32) * 4 + 1024 <= 150 * 1024 && k < 64;
+}
+
 extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
   if (!eng) { moe_set_error("null engine"); return MOE_EINVAL; }
   if (!eng->fatal.empty()) { moe_set_error("engine is in a failed state: %s", eng->fatal.c_str()); return MOE_ESTATE; }
@@ -240,6 +246,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                    eng->layer_complete[layer] == E;
   }
   static const bool token_route = !(getenv("MOE_TOKEN_ROUTE") && atoi(getenv("MOE_TOKEN_ROUTE")) == 0);
+  static const bool token_w2c = !(getenv("MOE_TOKEN_W2C") && atoi(getenv("MOE_TOKEN_W2C")) == 0);
   if (all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
     // one token: gate logits, then the w13 kernel routes by itself (no top-k / dispatch launches)
     if (!d.gate_bias) {
@@ -258,15 +265,18 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     s->pend_head = (s->pend_head + 1) % LayerState::kPending;
     // the kernel stores the unit list into the pending slot's pinned memory and then the sequence word
     const int seq = ++s->seq_counter;
+    const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
+    const bool w2c = token_w2c && w2c_fits(d, k);  // w2 and the combine in one launch
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq, 3, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq,
+                                    w2c ? 5 : 3, sg0, y, st)))
       return rc;
     *p.n_active = k;
     p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
-    const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
-    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
+    if (!w2c &&
+        (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
       return rc;
     if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
@@ -306,7 +316,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, 3, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
+                                    nullptr, nullptr, st)))
       return rc;
     {  // the routing arrives a few microseconds after the kernel starts
       volatile int *sq = s->opt_seq;
@@ -336,6 +347,17 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       }
       eng->ctr.ready += (uint64_t)now_ids.size();
     }
+    // the w2 pass goes out now that the routing is known (the w13 kernel is still running): with
+    // every selected expert resident it also combines, otherwise it leaves partial rows for the
+    // experts computed below and the combine after them
+    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
+    const bool w2c = later.empty() && token_w2c && w2c_fits(d, k);
+    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, nullptr, nullptr, 0,
+                                    w2c ? 4 : 2, sgo, y, st)))
+      return rc;
     if (!now_ids.empty() && (rc = moe_release_experts(eng, layer, now_ids.data(), (int64_t)now_ids.size()))) return rc;
     s->sub_cursor = 0;
     for (int64_t id : later) {
@@ -348,8 +370,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       s->sub_cursor++;
       if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
     }
-    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
-    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
+    if (!w2c &&
+        (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
       return rc;
     if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);

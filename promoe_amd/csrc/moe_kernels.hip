@@ -595,6 +595,7 @@ struct GemvArgs {
   // optional copy of the unit list straight into pinned host memory, then a sequence word
   moe_unit *r_host_units; int *r_host_seq; int r_host_seq_val, r_pad2;
   KUnit *r_kunits;              // routing publisher: resolved units (slot address, rows) for the w2 pass
+  float *r_unit_w;              // and the routing weight per unit position
   const KUnit *kunits_dev;      // device-side resolved units: one load instead of unit -> table -> address
 };
 
@@ -824,7 +825,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
       if (a.r_host_units) a.r_host_units[pos] = un;
-      if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; }
+      if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; a.r_unit_w[pos] = wgt; }
     }
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
@@ -1030,6 +1031,151 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
       }
     }
     if (t0 + TMAX < m) __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// k3 (w2) + k5 for ONE token in one launch: a workgroup of 16 waves owns 16 output rows and walks
+// the w2 tiles of those rows over ALL units (the k routed experts and the shared expert), weighting
+// each unit as it accumulates, so the combine needs no launch of its own and no partial rows in memory.
+//   item i < k*G : unit i / G, quantisation group i % G;  items k*G .. : the shared expert's groups
+//   wave w takes items w, w+16, ...; W2C_CHUNK tiles per wave are requested before the activations
+//   (the h vectors of all units) are staged in LDS.
+// ---------------------------------------------------------------------------
+#define W2C_CHUNK 6
+#define W2C_WAVES 16
+struct W2cArgs {
+  const KUnit *kunits;   // resolved routed units (slot address; row = position of the unit's h vector)
+  const float *unit_w;   // routing weight per unit position
+  const uint16_t *h_r, *h_s;
+  const unsigned char *shared_base;
+  const float *sg_logit;  // shared expert's gate logit or NULL
+  long long off_q, off_s, off_z, sh_off_q, sh_off_s, sh_off_z;
+  int k, I, I_sh, H, G, G_sh;
+  uint16_t *y;
+  int *err;
+};
+
+__global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2cArgs a) {
+  extern __shared__ __align__(16) unsigned char wsm[];
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, qd = lane >> 4;
+  const int b = blockIdx.x;  // rows 16b .. 16b+15
+  const int k = a.k, I = a.I, I_sh = a.I_sh, G = a.G, G_sh = a.G_sh;
+  const int n_h = k * I + I_sh;                       // staged activation elements
+  uint16_t *hs = (uint16_t *)wsm;                     // [k][I] then [I_sh]
+  float *xsum = (float *)(wsm + (size_t)n_h * 2);     // sums over 32 consecutive elements
+  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][16]
+  const int zsh = (r & 1) * 4;
+  // the activations are requested first: they depend on nothing, and memory answers a wave in order,
+  // so asked for after the tiles they would arrive after them
+  constexpr int HV = 2;  // vectors per thread held in registers (16 K activations); more go through the loop below
+  const int nvec = n_h >> 3;
+  uint4 hv[HV];
+#pragma unroll
+  for (int j = 0; j < HV; ++j) {
+    const int v = tid + j * 64 * W2C_WAVES;
+    const int el = (v < nvec ? v : 0) * 8;
+    hv[j] = el < k * I ? *(const uint4 *)(a.h_r + el) : *(const uint4 *)(a.h_s + (el - k * I));
+  }
+  // lane u holds unit u's slot address and weight (lane k: the shared expert); read back with readlane
+  u32 ub_lo = 0, ub_hi = 0;
+  float uw = 0.f;
+  if (lane < k) {
+    const unsigned long long ub = a.kunits[lane].base;
+    ub_lo = (u32)ub; ub_hi = (u32)(ub >> 32);
+    uw = a.unit_w[lane];
+  } else if (lane == k) {
+    const unsigned long long ub = (unsigned long long)a.shared_base;
+    ub_lo = (u32)ub; ub_hi = (u32)(ub >> 32);
+    uw = a.sg_logit ? 1.f / (1.f + expf(-a.sg_logit[0])) : 1.f;
+  }
+
+  float acc = 0.f;
+  // item cursor of this wave: unit u (k = the shared expert), group g; a wave's items are W2C_WAVES apart
+  int u = 0, g = w;
+  while (u < k && g >= G) { g -= G; ++u; }
+  bool staged = false;
+  do {  // a wave without items still takes part in the staging barrier
+    u32x4_t wt[W2C_CHUNK];
+    u32 sc[W2C_CHUNK], zz[W2C_CHUNK];
+    float wgt[W2C_CHUNK];
+    int ho[W2C_CHUNK];  // where the item's 128 activations start in the staged vector; -1 = no item
+    // ---- request this chunk's tiles --------------------------------------------------
+#pragma unroll
+    for (int c = 0; c < W2C_CHUNK; ++c) {
+      const bool on = u < k || g < G_sh;
+      const bool shd = u >= k;
+      const int Gu = shd ? G_sh : G;
+      const int ul = on ? u : 0;
+      const u32 lo = __builtin_amdgcn_readlane(ub_lo, ul), hi = __builtin_amdgcn_readlane(ub_hi, ul);
+      wgt[c] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul));
+      const unsigned char *base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+      ho[c] = on && base != nullptr ? (shd ? k * I : u * I) + g * 128 : -1;
+      wt[c] = u32x4_t{0u, 0u, 0u, 0u}; sc[c] = 0; zz[c] = 0;
+      if (on) {  // uniform
+        if (base == nullptr) {  // a selected expert that is not resident
+          if (lane == 0) atomicOr(a.err, 1);
+        } else {
+          const size_t t_idx = (size_t)b * Gu + g;
+          wt[c] = *(g_uint4 *)(base + (shd ? a.sh_off_q : a.off_q) + t_idx * 1024 + lane * 16);
+          sc[c] = *(const __attribute__((address_space(1))) uint16_t *)(base + (shd ? a.sh_off_s : a.off_s) + t_idx * 32 + 2 * r);
+          zz[c] = *(const __attribute__((address_space(1))) unsigned char *)(base + (shd ? a.sh_off_z : a.off_z) + t_idx * 8 + (r >> 1));
+        }
+        g += W2C_WAVES;
+        while (u < k && g >= G) { g -= G; ++u; }
+      }
+    }
+    // ---- first chunk: stage every unit's h vector (+ 32-wide sums) while the tiles travel --------
+    if (!staged) {
+#pragma unroll
+      for (int j = 0; j < HV; ++j) {
+        const int v = tid + j * 64 * W2C_WAVES;
+        float ps = sum8_bf16(hv[j]);
+        ps += __shfl_xor(ps, 1, 64);
+        ps += __shfl_xor(ps, 2, 64);
+        if (v < nvec) {
+          ((uint4 *)hs)[v] = hv[j];
+          if ((tid & 3) == 0) xsum[v >> 2] = ps;
+        }
+      }
+      for (int v = tid + HV * 64 * W2C_WAVES; v < nvec; v += 64 * W2C_WAVES) {
+        const int el = v * 8;
+        const uint4 x4 = el < k * I ? *(const uint4 *)(a.h_r + el) : *(const uint4 *)(a.h_s + (el - k * I));
+        float ps = sum8_bf16(x4);
+        ps += __shfl_xor(ps, 1, 64);
+        ps += __shfl_xor(ps, 2, 64);
+        ((uint4 *)hs)[v] = x4;
+        if ((tid & 3) == 0) xsum[v >> 2] = ps;
+      }
+      __syncthreads();
+      staged = true;
+    }
+    // ---- products: no branch, an absent item has zero weights and a zero scale and reads the first activations
+#pragma unroll
+    for (int c = 0; c < W2C_CHUNK; ++c) {
+      const int hoff = (ho[c] >= 0 ? ho[c] : 0) + qd * 32;  // the lane's 32 activations
+      const uint4 *xp = (const uint4 *)(hs + hoff);
+      const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+      const float xq = xsum[hoff >> 5];
+      const float d0 = dot8_q4(wt[c].x, x0, 0.f), d1 = dot8_q4(wt[c].y, x1, 0.f);
+      const float d2 = dot8_q4(wt[c].z, x2, 0.f), d3 = dot8_q4(wt[c].w, x3, 0.f);
+      const float d = (d0 + d1) + (d2 + d3);
+      const float fs = half_bits_to_f32((uint16_t)sc[c]);
+      const float fz = 128.f + (float)((zz[c] >> zsh) & 15);
+      acc = fmaf(wgt[c] * fs, d - fz * xq, acc);
+    }
+  } while (u < k || g < G_sh);
+  // the four k quarters of the wave, then the waves
+  acc += __shfl_xor(acc, 16, 64);
+  acc += __shfl_xor(acc, 32, 64);
+  if (lane < 16) red[w * 16 + lane] = acc;
+  __syncthreads();
+  if (tid < 16) {
+    float v = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < W2C_WAVES; ++ww) v += red[ww * 16 + tid];
+    a.y[b * 16 + tid] = f32_to_bf16(v);
   }
 }
 
@@ -1606,7 +1752,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
                                      void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
-                                     int phases, void *stream) {
+                                     int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
   if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
       !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
       mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
@@ -1629,6 +1775,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.r_units = units; a.r_n_active = n_active; a.r_active_ids = (long long *)active_ids;
   a.r_host_units = units_host_out; a.r_host_seq = units_host_out ? seq_host_out : nullptr; a.r_host_seq_val = seq_value;
   a.r_kunits = (KUnit *)unit_ws;
+  a.r_unit_w = unit_ws ? (float *)((KUnit *)unit_ws + k) : nullptr;
   // pass 1: w13 + SwiGLU, routing derived in the kernel
   a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, 0, I_sh, I_sh / 16, 0};
   a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
@@ -1648,6 +1795,39 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
       default: rc = launch_gemv_route<4>(a, grid, lds, s); break;
     }
     if (rc) return rc;
+  }
+  if (phases & 4) {  // w2 and the combine in one launch, straight into y
+    if (!unit_ws || !y_bf16 || (H % 16) || k >= 64) {
+      moe_set_error("moe_decode_token_int4: the fused w2 + combine pass needs unit_ws, y and k < 64");
+      return MOE_EINVAL;
+    }
+    W2cArgs c;
+    memset(&c, 0, sizeof c);
+    c.kunits = (const KUnit *)unit_ws; c.unit_w = (const float *)((const KUnit *)unit_ws + k);
+    c.h_r = (const uint16_t *)h_r; c.h_s = (const uint16_t *)h_s; c.shared_base = (const unsigned char *)shared_ptr;
+    c.sg_logit = shared_gate_logit;
+    c.off_q = lr.off2_q; c.off_s = lr.off2_s; c.off_z = lr.off2_z;
+    c.sh_off_q = ls.off2_q; c.sh_off_s = ls.off2_s; c.sh_off_z = ls.off2_z;
+    c.k = k; c.I = I; c.I_sh = sh ? I_sh : 0; c.H = H; c.G = I / 128; c.G_sh = sh ? I_sh / 128 : 0;
+    c.y = (uint16_t *)y_bf16; c.err = err;
+    const size_t n_h = (size_t)k * I + c.I_sh;
+    const size_t lds = n_h * 2 + (n_h / 32) * 4 + W2C_WAVES * 16 * 4;
+    if (lds > 150 * 1024) {
+      moe_set_error("moe_decode_token_int4: fused w2 + combine does not fit LDS (k=%d I=%d)", k, I);
+      return MOE_EINVAL;
+    }
+    static bool attr_set = false;
+    if (lds > 64 * 1024 && !attr_set) {
+      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_w2_combine_token,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                 "hipFuncSetAttribute(k_w2_combine_token)"))
+        return rc;
+      attr_set = true;
+    }
+    moe_ktimer_begin(MOE_K_W2, s);
+    hipLaunchKernelGGL(k_w2_combine_token, dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
+    moe_ktimer_end(MOE_K_W2, s);
+    return moe_check_launch("k_w2_combine_token");
   }
   if (!(phases & 2)) return MOE_OK;
   // pass 2: w2 over the unit list the first pass published

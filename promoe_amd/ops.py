@@ -129,7 +129,7 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
 
 
 def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int, ws=None,
-                      phases: int = 3):
+                      phases: int = 3, unit_ws=None, sg_logit=None, y=None):
     """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
     dev = x.device
     if ws is None:
@@ -149,7 +149,8 @@ def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, 
                                     ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
                                     ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
                                     ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
-                                    ptr(err), 0, 0, 0, 0, phases, cur_stream()), "moe_decode_token_int4")
+                                    ptr(err), ptr(unit_ws), 0, 0, 0, phases, ptr(sg_logit), ptr(y), cur_stream()),
+          "moe_decode_token_int4")
     return idx, w, d, part_r, part_s, err, h_r, h_s
 
 

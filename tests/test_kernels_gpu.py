@@ -239,6 +239,51 @@ def test_token_decode_routes_in_kernel_like_separate_kernels(cuda, H, I, E, k, m
         assert torch.equal(y_ref, y)
 
 
+@pytest.mark.parametrize("H,I,E,k,mode,I_sh,zipf,gated", [
+    (2048, 1408, 16, 6, 0, 2816, 1.2, False), (256, 384, 8, 2, 2, 256, None, True), (256, 256, 60, 4, 1, 512, 1.1, False),
+    (512, 128, 200, 8, 0, 0, None, False), (4096, 14336, 4, 2, 2, 0, None, False), (3584, 2560, 8, 8, 0, 20480, 1.1, True),
+    (256, 128, 4, 1, 0, 0, None, False)])
+def test_token_decode_w2_and_combine_in_one_launch(cuda, H, I, E, k, mode, I_sh, zipf, gated):
+    """One token: phase bit 2 runs w2 over all units and the weighted combine in one launch.  Same
+    routing outputs as the two-launch form; y within bf16 rounding of it (other summation order),
+    and within 2e-2 of the fp32 restatement."""
+    from promoe_amd import ops
+    print(f"case token_w2c H={H} I={I} E={E} k={k} mode={mode} I_sh={I_sh}", flush=True)
+    layer = Int4Layer(H=H, I=I, E=E, I_sh=I_sh, seed=5, zipf=zipf, shared_gate=gated)
+    slots = [torch.from_numpy(s).to(cuda) for s in layer.slots]
+    table = torch.tensor([s.data_ptr() for s in slots], dtype=torch.int64, device=cuda)
+    shared = torch.from_numpy(layer.shared_img).to(cuda) if I_sh else None
+    wg_np = layer.wg if not gated else np.concatenate([layer.wg, layer.shared_gate[None, :]], axis=0)
+    wg = bf16_dev(wg_np, cuda)
+    bias = None if layer.bias is None else torch.from_numpy(
+        np.concatenate([layer.bias, np.zeros(wg_np.shape[0] - E, np.float32)])).to(cuda)
+    unit_ws = torch.zeros(32 * k, dtype=torch.uint8, device=cuda)
+    for seed in range(2):
+        x = O.synth_acts(1, H, seed=seed + 20)
+        xd = bf16_dev(x, cuda)
+        logits = ops.gate_logits(xd, wg, bias)
+        sg = logits[:, E] if gated else None
+        idx, w, d, pr, ps, err, _, _ = ops.decode_token_int4(xd, logits, E, k, mode, table, shared, H, I, I_sh)
+        y_ref = ops.combine(pr, ps, w, d.pos_of_pair, sg, 1, H, k)
+        y = torch.full((1, H), float("nan"), dtype=torch.bfloat16, device=cuda)
+        idx2, w2, d2, _, _, err2, _, _ = ops.decode_token_int4(xd, logits, E, k, mode, table, shared, H, I, I_sh,
+                                                               phases=5, unit_ws=unit_ws, sg_logit=sg, y=y)
+        torch.cuda.synchronize()
+        assert int(err.cpu()[0]) == 0 and int(err2.cpu()[0]) == 0
+        assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+        assert torch.equal(d.units[:k], d2.units[:k])
+        a, b = y.float().cpu().numpy(), y_ref.float().cpu().numpy()
+        assert np.isfinite(a).all()
+        assert np.abs(a - b).max() <= 1e-2 * np.abs(b).max(), (np.abs(a - b).max(), np.abs(b).max())
+        lg = O.gate_logits_ordered(x, layer.wg)
+        if layer.bias is not None:
+            lg = (lg + layer.bias[None, :]).astype(np.float32)
+        ref = O.moe_forward(x, layer.wg, layer.experts_fp32, k, mode, shared=layer.shared_fp32,
+                            shared_gate=layer.shared_gate, logits=lg)
+        assert np.array_equal(idx2.cpu().numpy(), ref["idx"])
+        assert np.abs(a - ref["out"]).max() <= TOL * np.abs(ref["out"]).max()
+
+
 @pytest.mark.parametrize("T,E,k,mode", [(1, 64, 6, 0), (4, 64, 6, 0), (16, 64, 6, 1), (16, 60, 4, 2), (7, 200, 8, 0),
                                         (16, 8, 2, 2), (3, 256, 32, 0)])
 def test_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode):
