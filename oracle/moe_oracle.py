@@ -212,6 +212,32 @@ def dequant_int4(qweight, scales, qzeros, N: int, K: int) -> np.ndarray:
 #   128 bytes of nibbles.   w = d*sc_j*q - dmin*m_j
 # Nibble order (ggml): for each 64-weight chunk c (0..3), bytes qs[32c .. 32c+31]:
 #   low nibbles are weights 64c+0..31 (sub-block 2c), high nibbles 64c+32..63 (2c+1).
+def dequant_gptq(qweight, qzeros, scales, g_idx=None, zero_plus_one: bool = True) -> np.ndarray:
+    """AutoGPTQ checkpoint tensors of one linear layer -> fp32 weight [N, K] (out x in).
+
+    Restates the published AutoGPTQ 4-bit convention (the library itself is not part of the
+    reference tree: the reference only moves these buffers, utils/__init__.py:39-60):
+    qweight int32 [K/8, N] packs 8 inputs per word, low nibble first; qzeros int32 [G, N/8] packs 8
+    outputs per word; format "gptq" stores zero - 1 and adds the one back modulo 16; scales [G, N];
+    w[k, n] = (q[k, n] - zero[g_idx[k], n]) * scales[g_idx[k], n].  Plain loops over the nibbles on
+    purpose (the product code uses a vectorised transpose)."""
+    qw = np.asarray(qweight).view(np.uint32)
+    qz = np.asarray(qzeros).view(np.uint32)
+    sc = np.asarray(scales, np.float16).astype(np.float32)
+    K, N = qw.shape[0] * 8, qw.shape[1]
+    G = qz.shape[0]
+    gi = np.arange(K) // (K // G) if g_idx is None else np.asarray(g_idx).reshape(-1)
+    w = np.zeros((N, K), np.float32)
+    for k in range(K):
+        q = (qw[k // 8, :] >> np.uint32(4 * (k % 8))) & 0xF                    # [N]
+        g = int(gi[k])
+        z = np.array([(qz[g, n // 8] >> np.uint32(4 * (n % 8))) & 0xF for n in range(N)], np.int64)
+        if zero_plus_one:
+            z = (z + 1) & 0xF
+        w[:, k] = (q.astype(np.float32) - z.astype(np.float32)) * sc[g, :]
+    return w
+
+
 # --------------------------------------------------------------------------
 QK_K = 256
 Q4K_BYTES = 144
