@@ -139,6 +139,26 @@ int moe_attach_predictor(moe_engine *eng, int attached);
  * p[n_layers, num_expert] for layers starting_layer.. (policy "nn") */
 int moe_update_priority(moe_engine *eng, const float *p, int n_layers, int starting_layer);
 
+/* ---- built-in predictor: what the reference's SepPredictor + PredictWorker do (predictor.cpp:496-607,
+ * worker.cpp:6-77) with one linear model per (source layer -> destination layer) pair, scored on
+ * the GPU.  Source layer l (0..L; L = the last layer's output) predicts the layers of its window
+ * (build_predict_layer_mapping, predictor.cpp:8-46, from layer_predict_interval,
+ * layer_predict_max_window, limit_layer_0_window and
+ * layer_predict_replace_first_input_with_last_output).  When a decode step (B = S = 1) reports the
+ * hidden state of layer l (moe_report_layer_logits; moe_forward does it with every block's input), the
+ * scores x . W^T + b of every destination layer are computed on the compute stream; a host thread
+ * ranks the top num_predict_expert_per_layer experts (ties: lower id), feeds the softmax of the scores
+ * to the NN policy (moe_update_priority) and issues the prefetch requests.  Prefill steps issue empty
+ * requests.  Starting the predictor attaches it (see moe_attach_predictor). ---- */
+/* first[l], last[l] for l = 0..L: destination layers [first, last) of source layer l */
+int moe_predictor_windows(moe_engine *eng, int *first, int *last);
+/* model of one pair: w bf16 [num_expert, H] and bias fp32 [num_expert] or NULL, device memory the caller
+ * keeps alive (host memory on the host backend); dst must lie in the window of src */
+int moe_predictor_set_model(moe_engine *eng, int src, int dst, const void *w, const float *bias, int H);
+/* after moe_launch: needs a model for every pair of every window, and every layer covered once */
+int moe_predictor_start(moe_engine *eng);
+int moe_predictor_stats(moe_engine *eng, uint64_t *n_jobs, uint64_t *n_requests);
+
 /* ---- Belady policy hooks: CacheOracle / set_cur_seq (adapter.cpp:62-70, cache.cpp:592-644) ---- */
 int moe_oracle_load(moe_engine *eng, const int64_t *entry_metas, int64_t n_entries,
                     const int32_t *prefill_len, int64_t n_seq, const int32_t *prefill_sel,

@@ -315,6 +315,27 @@ def load_oracle(L, E, entry_metas, prefill_len, prefill_sel, decode_sel):
     return out
 
 
+def predict_layer_mapping(L, interval, window, limit_layer_0_window, cross_token):
+    """Destination layers [first, last) each source layer 0..L predicts (predictor.cpp:8-46)."""
+    pl = [0] * (L + 1)
+    stop = 0
+    for l in range(0, L, max(interval, 1)):
+        w = window
+        if l == 0 and limit_layer_0_window != -1:
+            w = limit_layer_0_window
+        pl[l] = stop
+        pl[l + 1] = min(l % L + w, L)
+        stop = pl[l + 1]
+    for l in range(1, L + 1):
+        if pl[l] < pl[l - 1]:
+            pl[l] = pl[l - 1]
+    ret = [(pl[l], pl[l + 1]) for l in range(L)] + [(0, 0)]
+    if cross_token:
+        ret[L] = ret[0]
+        ret[0] = (0, 0)
+    return ret
+
+
 # ---------------------------------------------------------------- cache + scheduler
 class CacheSim:
     """Experts are keyed (layer, expert)."""

@@ -52,6 +52,10 @@ _sig("moe_route_decode", [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp,
 _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_topk_dispatch", [vp, i32, i32, i32, i32, i32] + [vp] * 10 + [i32, vp, vp, vp, i32, vp])
 _sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])
+_sig("moe_predictor_windows", [vp, vp, vp])
+_sig("moe_predictor_set_model", [vp, i32, i32, vp, vp, i32])
+_sig("moe_predictor_start", [vp])
+_sig("moe_predictor_stats", [vp, vp, vp])
 _sig("moe_q4k_layout_make", [i32, i32, C.POINTER(Int4Layout)])
 _sig("moe_experts_decode_q4k", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_prefill_workspace_bytes", [i32, i32, i32], C.c_int64)

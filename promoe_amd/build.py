@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmoe_engine.so")
 
 HIP_SOURCES = ["moe_kernels.hip", "moe_prefill.hip"]
-CXX_SOURCES = ["moe_common.cpp", "engine_cfg.cpp", "engine_core.cpp", "engine_forward.cpp", "backends.cpp"]
+CXX_SOURCES = ["moe_common.cpp", "engine_cfg.cpp", "engine_core.cpp", "engine_forward.cpp", "engine_predict.cpp", "backends.cpp"]
 
 # -packed-fp32-ops: keep hipcc from forming v_pk_*_f32 out of scalar float code.
 HIP_FLAGS = [

@@ -579,6 +579,7 @@ moe_engine::~moe_engine() {
   cv_work.notify_all();
   cv_state.notify_all();
   cv_sem.notify_all();
+  moe_predictor_free(this);
   if (fetch_thread.joinable()) fetch_thread.join();
   if (fw) { moe_forward_free(fw); fw = nullptr; }
 }
@@ -792,11 +793,12 @@ extern "C" int moe_expert_num_ready(moe_engine *eng, int layer, int expert) {
 // ---------------------------------------------------------------------------
 extern "C" int moe_report_layer_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H) {
   ENG_GUARD(eng);
-  (void)hidden; (void)B; (void)H;
   if (layer < 0 || layer > eng->cfg.num_layer) { moe_set_error("bad layer %d", layer); return MOE_EINVAL; }
-  std::lock_guard<std::mutex> lk(eng->mu);
-  if (layer == 0) eng->s_seqlen.push_back((uint64_t)S);  // prefetcher.cpp:452-455
-  return MOE_OK;
+  {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    if (layer == 0) eng->s_seqlen.push_back((uint64_t)S);  // prefetcher.cpp:452-455
+  }
+  return moe_predictor_on_logits(eng, layer, hidden, B, S, H);  // prefetcher.cpp:451-452
 }
 
 static int report_one_layer_locked(moe_engine *eng, int layer, int64_t *ids, int64_t n,

@@ -233,7 +233,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   const int ldl = E + 1;
   int rc;
   // hook order of the reference (utils/hooks.py:216-223)
-  if (layer == 0 && (rc = moe_report_layer_logits(eng, 0, x, 1, T, d.H))) return rc;
+  // the layer hook's pre_forward: this block's input (decode: what the built-in predictor reads)
+  if ((rc = moe_report_layer_logits(eng, layer, x, 1, T, d.H))) return rc;
   const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
   if ((rc = moe_forward_harvest(eng, false))) return rc;
   // Every expert of the layer resident, and the layer's slot group can hold them all: there
@@ -242,8 +243,9 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   bool all_resident = false;
   {
     std::lock_guard<std::mutex> lk(eng->mu);
+    // (with a predictor attached the hooks' budget / progress bookkeeping has to run: no short cut)
     all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
-                   eng->layer_complete[layer] == E;
+                   eng->layer_complete[layer] == E && !eng->predictor_attached;
   }
   static const bool token_route = !(getenv("MOE_TOKEN_ROUTE") && atoi(getenv("MOE_TOKEN_ROUTE")) == 0);
   static const bool token_w2c = !(getenv("MOE_TOKEN_W2C") && atoi(getenv("MOE_TOKEN_W2C")) == 0);
@@ -278,7 +280,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (!w2c &&
         (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
       return rc;
-    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
   // One token, demand fetching only (no prefetch producer that could evict behind our back) and the
@@ -373,7 +375,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (!w2c &&
         (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
       return rc;
-    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
   static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
@@ -441,7 +443,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
       return rc;
-    if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
   // the active expert list comes back to the host
@@ -500,7 +502,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k, st)))
     return rc;
   // MoeLayerHook.post_forward (utils/hooks.py:220-223)
-  if ((rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+  if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
   return moe_layer_done(eng, layer);
 }
 

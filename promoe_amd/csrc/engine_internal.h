@@ -158,6 +158,7 @@ Backend *moe_make_host_backend();
 struct Series { std::vector<uint64_t> v; };
 
 struct LayerState;  // forward workspace, engine_forward.cpp
+struct PredictorState;  // built-in predictor, engine_predict.cpp
 
 struct moe_engine {
   moe_cfg cfg;
@@ -206,12 +207,15 @@ struct moe_engine {
   // fused forward
   std::vector<moe_layer_desc> layer_desc;
   LayerState *fw = nullptr;
+  PredictorState *pred = nullptr;
 
   ~moe_engine();
 };
 
 int engine_fail(moe_engine *eng, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void moe_forward_free(LayerState *);
+void moe_predictor_free(moe_engine *eng);
+int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H);
 // account demand hits of experts that were launched without a host round trip
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);
 // collect the routing results of earlier moe_forward calls (wait: block until all are in)

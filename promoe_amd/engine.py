@@ -152,8 +152,8 @@ class PrefetchMngr:
 
     def report_moe_layer_logits(self, layer_id: int, hidden=None, seq_len: int | None = None):
         if hidden is not None:
-            B, S, H = (hidden.shape if hidden.dim() == 3 else (1,) + tuple(hidden.shape))
-            p = hidden.data_ptr()
+            B, S, H = (hidden.shape if len(hidden.shape) == 3 else (1,) + tuple(hidden.shape))
+            p = hidden.ctypes.data if isinstance(hidden, np.ndarray) else hidden.data_ptr()
         else:
             B, S, H, p = 1, int(seq_len or 1), 0, 0
         check(lib.moe_report_layer_logits(self._h, layer_id, p, B, S, H), "report_moe_layer_logits")
@@ -202,6 +202,30 @@ class PrefetchMngr:
 
     def attach_predictor(self, attached: bool = True):
         check(lib.moe_attach_predictor(self._h, int(attached)), "attach_predictor")
+
+    # -- built-in predictor (linear model per source -> destination layer pair) --
+    def predictor_windows(self):
+        """[(first, last)] for source layers 0..L: the destination layers each one predicts."""
+        n = int(self.metas.num_layer) + 1
+        a, b = (C.c_int * n)(), (C.c_int * n)()
+        check(lib.moe_predictor_windows(self._h, a, b), "predictor_windows")
+        return list(zip(a, b))
+
+    def set_predictor_model(self, src: int, dst: int, w, bias=None):
+        """w bf16 [E, H] (device tensor; numpy uint16 bit patterns on the host backend), bias fp32 [E] or None."""
+        self._keep.append((w, bias))
+        H = int(w.shape[1])
+        wp = w.ctypes.data if isinstance(w, np.ndarray) else L.ptr(w)
+        bp = None if bias is None else (bias.ctypes.data if isinstance(bias, np.ndarray) else L.ptr(bias))
+        check(lib.moe_predictor_set_model(self._h, src, dst, wp, bp, H), "set_predictor_model")
+
+    def start_predictor(self):
+        check(lib.moe_predictor_start(self._h), "start_predictor")
+
+    def predictor_stats(self) -> dict:
+        a, b = C.c_uint64(), C.c_uint64()
+        check(lib.moe_predictor_stats(self._h, C.byref(a), C.byref(b)), "predictor_stats")
+        return {"jobs": a.value, "requests": b.value}
 
     def update_priority(self, p: np.ndarray, starting_layer: int = 0):
         p = np.ascontiguousarray(p, dtype=np.float32)

@@ -262,3 +262,44 @@ def test_forward_single_token_starts_before_the_host_knows_the_routing(cuda):
         assert c[key] == sim.ctr[key], key
     assert c["miss"] > 0 and c["hit"] > 0 and c["evictions"] > 0
     pm.close()
+
+
+def test_builtin_predictor_prefetches_what_the_next_layers_route_to(cuda):
+    """Models of the pairs (src -> dst) = the gate of dst, and every layer of a token sees the same
+    hidden state: the predictions are the true routings, so layers 1.. find their experts prefetched.
+    Outputs stay those of the oracle; demand misses drop against the same run without a predictor."""
+    print("case engine_predictor", flush=True)
+    Lyr, E, k, H = 4, 16, 2, 256
+    layers = [Int4Layer(H=H, I=128, E=E, I_sh=0, seed=30 + l) for l in range(Lyr)]
+    xs = [O.synth_acts(1, H, seed=700 + t) for t in range(12)]
+
+    def run(with_predictor):
+        pm = build_engine(layers, k, cuda, cache_rate=0.25, cache_policy="lru", num_predict_expert_per_layer=k,
+                          layer_predict_interval=1, layer_predict_max_window=2, limit_layer_0_window=2)
+        if with_predictor:
+            for src, (a, b) in enumerate(pm.predictor_windows()):
+                for dst in range(a, b):
+                    pm.set_predictor_model(src, dst, torch.from_numpy(layers[dst].wg).to(torch.bfloat16).to(cuda), None)
+            pm.start_predictor()
+        worst = 0.0
+        for x in xs:
+            xd = torch.from_numpy(x).to(torch.bfloat16).to(cuda)
+            for l in range(Lyr):
+                y = pm.forward(l, xd)
+                torch.cuda.synchronize()
+                ref = ref_forward(layers[l], x, k, 0)
+                worst = max(worst, float(np.abs(y.float().cpu().numpy() - ref["out"]).max() / np.abs(ref["out"]).max()))
+        pm.drain()
+        c = pm.counters()
+        st = pm.predictor_stats() if with_predictor else None
+        pm.close()
+        return worst, c, st
+
+    w0, c0, _ = run(False)
+    w1, c1, st = run(True)
+    assert w0 <= TOL and w1 <= TOL
+    assert st["jobs"] == len(xs) * 3 and st["requests"] == len(xs) * Lyr
+    assert c1["prefetch_hit"] > 0
+    assert c1["miss"] * 2 < c0["miss"]
+    print(f"  demand misses {c0['miss']} -> {c1['miss']}, ready {c0['ready']} -> {c1['ready']}, "
+          f"prefetch hits {c1['prefetch_hit']}", flush=True)

@@ -1,0 +1,113 @@
+"""Built-in predictor on the host backend: layer windows against the restated mapping, and the
+request / budget / progress protocol with models whose predictions are known."""
+import numpy as np
+import pytest
+
+from oracle import cache_oracle as CO
+from oracle import moe_oracle as O
+from promoe_amd import _lib as L
+from promoe_amd import engine as EG
+
+
+def make(Lyr, E, k, **cfg):
+    m = EG.ModuleMeta(Lyr, E)
+    m.init_param_list(["w"])
+    d = {"num_expert_per_token": str(k)}
+    d.update({a: str(b) for a, b in cfg.items()})
+    m.init_from_map(d)
+    m.handle_uninited_configs()
+    pm = EG.PrefetchMngr(m, backend=L.BACKEND_HOST)
+    for l in range(Lyr):
+        for e in range(E):
+            pm.add_one_expert_param(np.full(64, l * E + e, np.uint8), l, e, "w")
+    pm.init_gpu_mem_buffer()
+    pm.launch_thread()
+    return pm
+
+
+@pytest.mark.parametrize("Lyr,interval,window,limit0,cross", [(4, 1, 2, 2, False), (6, 1, 3, 1, False), (6, 2, 3, -1, False),
+                                                              (5, 1, 1, 1, False), (4, 1, 2, 2, True), (27, 1, 3, 3, False)])
+def test_windows_follow_the_reference_mapping(Lyr, interval, window, limit0, cross):
+    pm = make(Lyr, 4, 2, layer_predict_interval=interval, layer_predict_max_window=window, limit_layer_0_window=limit0,
+              layer_predict_replace_first_input_with_last_output=cross, predict_input_mode="moe_layer_logits")
+    got = pm.predictor_windows()
+    want = CO.predict_layer_mapping(Lyr, interval, window, int(pm.metas.limit_layer_0_window), cross)
+    assert got == want
+    pm.close()
+
+
+def test_known_windows():
+    # hand-derived from predictor.cpp:8-46: L=4, interval 1, window 2, layer 0 window 2
+    assert CO.predict_layer_mapping(4, 1, 2, 2, False) == [(0, 2), (2, 3), (3, 4), (4, 4), (0, 0)]
+    # cross-token: the last output predicts what layer 0's input did, layer 0 predicts nothing
+    assert CO.predict_layer_mapping(4, 1, 2, 2, True) == [(0, 0), (2, 3), (3, 4), (4, 4), (0, 2)]
+    # window 1: every layer predicts itself only
+    assert CO.predict_layer_mapping(3, 1, 1, 1, False) == [(0, 1), (1, 2), (2, 3), (0, 0)]
+
+
+def _bf16(a):
+    return O.f32_to_bf16_bits(np.ascontiguousarray(a, np.float32))
+
+
+def test_requests_follow_the_models_and_the_protocol_keeps_in_step():
+    Lyr, E, k, H = 4, 8, 2, 64
+    rng = np.random.default_rng(0)
+    pm = make(Lyr, E, k, cache_rate=0.5, cache_policy="lru", num_predict_expert_per_layer=2,
+              layer_predict_interval=1, layer_predict_max_window=2, limit_layer_0_window=2,
+              predict_input_mode="moe_layer_logits")
+    wins = pm.predictor_windows()
+    assert wins == [(0, 2), (2, 3), (3, 4), (4, 4), (0, 0)]
+    with pytest.raises(L.MoeError):
+        pm.set_predictor_model(1, 1, _bf16(np.zeros((E, H))))          # layer 1 predicts layer 2 only
+    # model of (src, dst): one-hot rows, so that the score of expert e is x[dst * E + e]
+    for src, (a, b) in enumerate(wins):
+        for dst in range(a, b):
+            w = np.zeros((E, H), np.float32)
+            w[np.arange(E), dst * E + np.arange(E)] = 1.0
+            pm.set_predictor_model(src, dst, _bf16(w), None)
+    pm.start_predictor()
+    want = {}
+    for tok in range(6):
+        x = np.zeros(H, np.float32)
+        chosen = {}
+        for l in range(Lyr):
+            top = rng.choice(E, size=2, replace=False)
+            x[l * E + top[0]] = 3.0; x[l * E + top[1]] = 2.0           # ranked: top[0] then top[1]
+            chosen[l] = [int(top[0]), int(top[1])]
+        xb = _bf16(x.reshape(1, 1, H))
+        for l in range(Lyr):
+            pm.report_moe_layer_logits(l, xb)
+            ids = np.array(sorted(chosen[l]), np.int64)
+            order = pm.report_one_layer(l, ids)                        # waits for the layer's request
+            for e in order:
+                pm.report_one_expert(l, int(e)); pm.one_expert_done(l, int(e))
+            pm.one_moe_layer_done(l)
+        pm.drain()
+        want[tok] = chosen
+    st = pm.predictor_stats()
+    assert st["jobs"] == 6 * 3 and st["requests"] == 6 * Lyr           # sources 0, 1, 2 have windows; 4 layers per token
+    c = pm.counters()
+    # layers 1..3 are requested before they run: their experts are prefetched, only layer 0 (predicted
+    # from its own input, a moment before use) and evictions can miss
+    assert c["prefetch_hit"] + c["prefetch_miss"] > 0
+    assert c["ready"] >= 6 * 3 * k * 0.9
+    # a prefill step: empty requests, nothing to wait for
+    pm.report_moe_layer_logits(0, None, seq_len=5)
+    for l in range(Lyr):
+        if l:
+            pm.report_moe_layer_logits(l, None, seq_len=5)
+        ids = np.arange(4, dtype=np.int64)
+        for e in pm.report_one_layer(l, ids):
+            pm.report_one_expert(l, int(e)); pm.one_expert_done(l, int(e))
+        pm.one_moe_layer_done(l)
+    assert pm.predictor_stats()["requests"] == 7 * Lyr
+    pm.close()
+
+
+def test_start_needs_every_model():
+    pm = make(3, 4, 2, layer_predict_interval=1, layer_predict_max_window=1, limit_layer_0_window=1,
+              predict_input_mode="moe_layer_logits")
+    pm.set_predictor_model(0, 0, _bf16(np.zeros((4, 16))))
+    with pytest.raises(L.MoeError, match="no model"):
+        pm.start_predictor()
+    pm.close()
