@@ -1035,14 +1035,17 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
 }
 
 // ---------------------------------------------------------------------------
-// k3 (w2) + k5 for ONE token in one launch: a workgroup of 16 waves owns 16 output rows and walks
+// k3 (w2) + k5 for ONE token in one launch: a workgroup of 16 waves owns 8 output rows and walks
 // the w2 tiles of those rows over ALL units (the k routed experts and the shared expert), weighting
 // each unit as it accumulates, so the combine needs no launch of its own and no partial rows in memory.
 //   item i < k*G : unit i / G, quantisation group i % G;  items k*G .. : the shared expert's groups
-//   wave w takes items w, w+16, ...; W2C_CHUNK tiles per wave are requested before the activations
-//   (the h vectors of all units) are staged in LDS.
+//   A tile holds 16 rows; the workgroup wants 8 of them, so a wave reads the halves of TWO items with
+//   one load: lanes whose tile row is 0..7 take item 2s, the others item 2s + 1, each its row & 7 of
+//   the workgroup's half.  Wave w takes the item pairs s = w, w+16, ...; W2C_CHUNK loads per wave are
+//   requested before the activations (the h vectors of all units) are staged in LDS.
+//   H/8 workgroups: twice the compute units of a 16-row split, which is what the load latency wants.
 // ---------------------------------------------------------------------------
-#define W2C_CHUNK 6
+#define W2C_CHUNK 3
 #define W2C_WAVES 16
 struct W2cArgs {
   const KUnit *kunits;   // resolved routed units (slot address; row = position of the unit's h vector)
@@ -1060,13 +1063,15 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   extern __shared__ __align__(16) unsigned char wsm[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
-  const int b = blockIdx.x;  // rows 16b .. 16b+15
+  const int b16 = blockIdx.x >> 1, half = blockIdx.x & 1;  // rows 16*b16 + 8*half .. + 7
+  const bool second = r >= 8;                               // this lane works on the pair's second item
+  const int rr = 8 * half + (r & 7);                        // its row inside the 16-row tile
   const int k = a.k, I = a.I, I_sh = a.I_sh, G = a.G, G_sh = a.G_sh;
   const int n_h = k * I + I_sh;                       // staged activation elements
   uint16_t *hs = (uint16_t *)wsm;                     // [k][I] then [I_sh]
   float *xsum = (float *)(wsm + (size_t)n_h * 2);     // sums over 32 consecutive elements
-  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][16]
-  const int zsh = (r & 1) * 4;
+  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][8]
+  const int zsh = (rr & 1) * 4;
   // the activations are requested first: they depend on nothing, and memory answers a wave in order,
   // so asked for after the tiles they would arrive after them
   constexpr int HV = 2;  // vectors per thread held in registers (16 K activations); more go through the loop below
@@ -1092,37 +1097,49 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   }
 
   float acc = 0.f;
-  // item cursor of this wave: unit u (k = the shared expert), group g; a wave's items are W2C_WAVES apart
-  int u = 0, g = w;
+  // cursor of the wave's current pair: first item = unit u (k = the shared expert), group g
+  int u = 0, g = 2 * w;
   while (u < k && g >= G) { g -= G; ++u; }
   bool staged = false;
   do {  // a wave without items still takes part in the staging barrier
     u32x4_t wt[W2C_CHUNK];
     u32 sc[W2C_CHUNK], zz[W2C_CHUNK];
     float wgt[W2C_CHUNK];
-    int ho[W2C_CHUNK];  // where the item's 128 activations start in the staged vector; -1 = no item
+    int ho[W2C_CHUNK];  // where the lane's item keeps its 128 activations in the staged vector
     // ---- request this chunk's tiles --------------------------------------------------
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
-      const bool on = u < k || g < G_sh;
-      const bool shd = u >= k;
+      // second item of the pair = the next item
+      int u2 = u, g2 = g + 1;
+      if (u2 < k && g2 >= G) { g2 -= G; ++u2; }
+      const bool on1 = u < k || g < G_sh, on2 = u2 < k || g2 < G_sh;
+      const int ul1 = on1 ? u : 0, ul2 = on2 ? u2 : 0;
+      const u32 lo1 = __builtin_amdgcn_readlane(ub_lo, ul1), hi1 = __builtin_amdgcn_readlane(ub_hi, ul1);
+      const u32 lo2 = __builtin_amdgcn_readlane(ub_lo, ul2), hi2 = __builtin_amdgcn_readlane(ub_hi, ul2);
+      const float w1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul1));
+      const float w2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul2));
+      const unsigned long long base1 = ((unsigned long long)hi1 << 32) | lo1, base2 = ((unsigned long long)hi2 << 32) | lo2;
+      if ((on1 && base1 == 0ull) || (on2 && base2 == 0ull)) {  // uniform: a selected expert that is not resident
+        if (lane == 0) atomicOr(a.err, 1);
+      }
+      // the lane's own item
+      const bool on = second ? (on2 && base2 != 0ull) : (on1 && base1 != 0ull);
+      const int lu = second ? u2 : u, lg = second ? g2 : g;
+      const bool shd = lu >= k;
+      const unsigned long long base = second ? base2 : base1;
       const int Gu = shd ? G_sh : G;
-      const int ul = on ? u : 0;
-      const u32 lo = __builtin_amdgcn_readlane(ub_lo, ul), hi = __builtin_amdgcn_readlane(ub_hi, ul);
-      wgt[c] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul));
-      const unsigned char *base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
-      ho[c] = on && base != nullptr ? (shd ? k * I : u * I) + g * 128 : -1;
+      wgt[c] = second ? w2 : w1;
+      ho[c] = on ? (shd ? k * I : lu * I) + lg * 128 : 0;
       wt[c] = u32x4_t{0u, 0u, 0u, 0u}; sc[c] = 0; zz[c] = 0;
-      if (on) {  // uniform
-        if (base == nullptr) {  // a selected expert that is not resident
-          if (lane == 0) atomicOr(a.err, 1);
-        } else {
-          const size_t t_idx = (size_t)b * Gu + g;
-          wt[c] = *(g_uint4 *)(base + (shd ? a.sh_off_q : a.off_q) + t_idx * 1024 + lane * 16);
-          sc[c] = *(const __attribute__((address_space(1))) uint16_t *)(base + (shd ? a.sh_off_s : a.off_s) + t_idx * 32 + 2 * r);
-          zz[c] = *(const __attribute__((address_space(1))) unsigned char *)(base + (shd ? a.sh_off_z : a.off_z) + t_idx * 8 + (r >> 1));
-        }
-        g += W2C_WAVES;
+      if (on) {
+        const unsigned char *bp = (const unsigned char *)base;
+        const size_t t_idx = (size_t)b16 * Gu + lg;
+        wt[c] = *(g_uint4 *)(bp + (shd ? a.sh_off_q : a.off_q) + t_idx * 1024 + (qd * 16 + rr) * 16);
+        sc[c] = *(const __attribute__((address_space(1))) uint16_t *)(bp + (shd ? a.sh_off_s : a.off_s) + t_idx * 32 + 2 * rr);
+        zz[c] = *(const __attribute__((address_space(1))) unsigned char *)(bp + (shd ? a.sh_off_z : a.off_z) + t_idx * 8 + (rr >> 1));
+      }
+      if (on1) {  // next pair of this wave
+        g += 2 * W2C_WAVES;
         while (u < k && g >= G) { g -= G; ++u; }
       }
     }
@@ -1154,7 +1171,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
     // ---- products: no branch, an absent item has zero weights and a zero scale and reads the first activations
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
-      const int hoff = (ho[c] >= 0 ? ho[c] : 0) + qd * 32;  // the lane's 32 activations
+      const int hoff = ho[c] + qd * 32;  // the lane's 32 activations
       const uint4 *xp = (const uint4 *)(hs + hoff);
       const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
       const float xq = xsum[hoff >> 5];
@@ -1166,16 +1183,17 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
       acc = fmaf(wgt[c] * fs, d - fz * xq, acc);
     }
   } while (u < k || g < G_sh);
-  // the four k quarters of the wave, then the waves
+  // the two items of the pairs, the four k quarters of the wave, then the waves
+  acc += __shfl_xor(acc, 8, 64);
   acc += __shfl_xor(acc, 16, 64);
   acc += __shfl_xor(acc, 32, 64);
-  if (lane < 16) red[w * 16 + lane] = acc;
+  if (lane < 8) red[w * 8 + lane] = acc;
   __syncthreads();
-  if (tid < 16) {
+  if (tid < 8) {
     float v = 0.f;
 #pragma unroll
-    for (int ww = 0; ww < W2C_WAVES; ++ww) v += red[ww * 16 + tid];
-    a.y[b * 16 + tid] = f32_to_bf16(v);
+    for (int ww = 0; ww < W2C_WAVES; ++ww) v += red[ww * 8 + tid];
+    a.y[b16 * 16 + 8 * half + tid] = f32_to_bf16(v);
   }
 }
 
@@ -1825,7 +1843,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
       attr_set = true;
     }
     moe_ktimer_begin(MOE_K_W2, s);
-    hipLaunchKernelGGL(k_w2_combine_token, dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
+    hipLaunchKernelGGL(k_w2_combine_token, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
     moe_ktimer_end(MOE_K_W2, s);
     return moe_check_launch("k_w2_combine_token");
   }
