@@ -1059,18 +1059,21 @@ struct W2cArgs {
   int *err;
 };
 
+// NI = items a wave reads with one load = 16 / (rows per workgroup)
+template <int NI>
 __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2cArgs a) {
   extern __shared__ __align__(16) unsigned char wsm[];
+  constexpr int RW = 16 / NI;  // rows of this workgroup
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
-  const int b16 = blockIdx.x >> 1, half = blockIdx.x & 1;  // rows 16*b16 + 8*half .. + 7
-  const bool second = r >= 8;                               // this lane works on the pair's second item
-  const int rr = 8 * half + (r & 7);                        // its row inside the 16-row tile
+  const int b16 = blockIdx.x / NI, part = blockIdx.x % NI;  // rows 16*b16 + RW*part .. + RW-1
+  const int mine = r / RW;                                  // which item of the group this lane works on
+  const int rr = RW * part + (r % RW);                      // its row inside the 16-row tile
   const int k = a.k, I = a.I, I_sh = a.I_sh, G = a.G, G_sh = a.G_sh;
   const int n_h = k * I + I_sh;                       // staged activation elements
   uint16_t *hs = (uint16_t *)wsm;                     // [k][I] then [I_sh]
   float *xsum = (float *)(wsm + (size_t)n_h * 2);     // sums over 32 consecutive elements
-  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][8]
+  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][RW]
   const int zsh = (rr & 1) * 4;
   // the activations are requested first: they depend on nothing, and memory answers a wave in order,
   // so asked for after the tiles they would arrive after them
@@ -1097,8 +1100,8 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   }
 
   float acc = 0.f;
-  // cursor of the wave's current pair: first item = unit u (k = the shared expert), group g
-  int u = 0, g = 2 * w;
+  // cursor of the wave's current group of NI items: first item = unit u (k = the shared expert), group g
+  int u = 0, g = NI * w;
   while (u < k && g >= G) { g -= G; ++u; }
   bool staged = false;
   do {  // a wave without items still takes part in the staging barrier
@@ -1109,26 +1112,28 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
     // ---- request this chunk's tiles --------------------------------------------------
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
-      // second item of the pair = the next item
-      int u2 = u, g2 = g + 1;
-      if (u2 < k && g2 >= G) { g2 -= G; ++u2; }
-      const bool on1 = u < k || g < G_sh, on2 = u2 < k || g2 < G_sh;
-      const int ul1 = on1 ? u : 0, ul2 = on2 ? u2 : 0;
-      const u32 lo1 = __builtin_amdgcn_readlane(ub_lo, ul1), hi1 = __builtin_amdgcn_readlane(ub_hi, ul1);
-      const u32 lo2 = __builtin_amdgcn_readlane(ub_lo, ul2), hi2 = __builtin_amdgcn_readlane(ub_hi, ul2);
-      const float w1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul1));
-      const float w2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul2));
-      const unsigned long long base1 = ((unsigned long long)hi1 << 32) | lo1, base2 = ((unsigned long long)hi2 << 32) | lo2;
-      if ((on1 && base1 == 0ull) || (on2 && base2 == 0ull)) {  // uniform: a selected expert that is not resident
-        if (lane == 0) atomicOr(a.err, 1);
+      // the group's items are consecutive; pick the lane's own while walking them (all uniform but the selects)
+      int uj = u, gj = g;
+      bool on = false, any_missing = false;
+      int lu = 0, lg = 0;
+      unsigned long long base = 0ull;
+      float lw = 0.f;
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const bool onj = uj < k || gj < G_sh;
+        const int ul = onj ? uj : 0;
+        const u32 lo = __builtin_amdgcn_readlane(ub_lo, ul), hi = __builtin_amdgcn_readlane(ub_hi, ul);
+        const float wj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul));
+        const unsigned long long bj = ((unsigned long long)hi << 32) | lo;
+        any_missing = any_missing || (onj && bj == 0ull);
+        if (mine == j) { on = onj && bj != 0ull; lu = uj; lg = gj; base = bj; lw = wj; }
+        ++gj;  // next item
+        if (uj < k && gj >= G) { gj -= G; ++uj; }
       }
-      // the lane's own item
-      const bool on = second ? (on2 && base2 != 0ull) : (on1 && base1 != 0ull);
-      const int lu = second ? u2 : u, lg = second ? g2 : g;
+      if (any_missing && lane == 0) atomicOr(a.err, 1);  // a selected expert that is not resident
       const bool shd = lu >= k;
-      const unsigned long long base = second ? base2 : base1;
       const int Gu = shd ? G_sh : G;
-      wgt[c] = second ? w2 : w1;
+      wgt[c] = lw;
       ho[c] = on ? (shd ? k * I : lu * I) + lg * 128 : 0;
       wt[c] = u32x4_t{0u, 0u, 0u, 0u}; sc[c] = 0; zz[c] = 0;
       if (on) {
@@ -1138,8 +1143,8 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
         sc[c] = *(const __attribute__((address_space(1))) uint16_t *)(bp + (shd ? a.sh_off_s : a.off_s) + t_idx * 32 + 2 * rr);
         zz[c] = *(const __attribute__((address_space(1))) unsigned char *)(bp + (shd ? a.sh_off_z : a.off_z) + t_idx * 8 + (rr >> 1));
       }
-      if (on1) {  // next pair of this wave
-        g += 2 * W2C_WAVES;
+      if (u < k || g < G_sh) {  // next group of this wave
+        g += NI * W2C_WAVES;
         while (u < k && g >= G) { g -= G; ++u; }
       }
     }
@@ -1183,17 +1188,18 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
       acc = fmaf(wgt[c] * fs, d - fz * xq, acc);
     }
   } while (u < k || g < G_sh);
-  // the two items of the pairs, the four k quarters of the wave, then the waves
-  acc += __shfl_xor(acc, 8, 64);
+  // the items of the groups, the four k quarters of the wave, then the waves
+#pragma unroll
+  for (int m = RW; m < 16; m <<= 1) acc += __shfl_xor(acc, m, 64);
   acc += __shfl_xor(acc, 16, 64);
   acc += __shfl_xor(acc, 32, 64);
-  if (lane < 8) red[w * 8 + lane] = acc;
+  if (lane < RW) red[w * RW + lane] = acc;
   __syncthreads();
-  if (tid < 8) {
+  if (tid < RW) {
     float v = 0.f;
 #pragma unroll
-    for (int ww = 0; ww < W2C_WAVES; ++ww) v += red[ww * 8 + tid];
-    a.y[b16 * 16 + 8 * half + tid] = f32_to_bf16(v);
+    for (int ww = 0; ww < W2C_WAVES; ++ww) v += red[ww * RW + tid];
+    a.y[b16 * 16 + RW * part + tid] = f32_to_bf16(v);
   }
 }
 
@@ -1834,16 +1840,20 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
       moe_set_error("moe_decode_token_int4: fused w2 + combine does not fit LDS (k=%d I=%d)", k, I);
       return MOE_EINVAL;
     }
+    static const int ni_env = getenv("MOE_W2C_SPLIT") ? atoi(getenv("MOE_W2C_SPLIT")) : 0;
+    const int ni = ni_env == 1 || ni_env == 2 || ni_env == 4 ? ni_env : 2;
     static bool attr_set = false;
     if (lds > 64 * 1024 && !attr_set) {
-      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_w2_combine_token,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                 "hipFuncSetAttribute(k_w2_combine_token)"))
-        return rc;
+      for (const void *f : {(const void *)k_w2_combine_token<1>, (const void *)k_w2_combine_token<2>, (const void *)k_w2_combine_token<4>})
+        if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                   "hipFuncSetAttribute(k_w2_combine_token)"))
+          return rc;
       attr_set = true;
     }
     moe_ktimer_begin(MOE_K_W2, s);
-    hipLaunchKernelGGL(k_w2_combine_token, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+    if (ni == 1) hipLaunchKernelGGL(k_w2_combine_token<1>, dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
+    else if (ni == 2) hipLaunchKernelGGL(k_w2_combine_token<2>, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+    else hipLaunchKernelGGL(k_w2_combine_token<4>, dim3(H / 4), dim3(64 * W2C_WAVES), lds, s, c);
     moe_ktimer_end(MOE_K_W2, s);
     return moe_check_launch("k_w2_combine_token");
   }
