@@ -27,6 +27,26 @@ static __device__ __forceinline__ float dot2bf(u32 a, u32 b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
                                          __builtin_bit_cast(bf16x2_t, b), c, false);
 }
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
+static __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
+}
+// A unit list for the host: stores with both scope bits set go past the caches straight to the pinned
+// host buffer; once they have completed (host_stores_done) the sequence word the host polls may follow.
+// No cache write-back or invalidate is involved, unlike a system-scope fence.
+static __device__ __forceinline__ void host_store_unit(moe_unit *dst, int i, int expert, int m, int row0) {
+  const u32x4_t v = {(u32)expert, (u32)m, (u32)row0, 0u};
+  __builtin_amdgcn_raw_buffer_store_b128(v, make_rsrc(dst, 0x7fffffffu), i * 16, 0, 17 /* sc0 | sc1 */);
+}
+static __device__ __forceinline__ void host_store_i32(int *dst, int v) {
+  __builtin_amdgcn_raw_buffer_store_b32((u32)v, make_rsrc(dst, 0x7fffffffu), 0, 0, 17);
+}
+static __device__ __forceinline__ void host_stores_done() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);  // every outstanding memory operation of this wave has completed
+}
 static __device__ __forceinline__ float half_bits_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
@@ -445,14 +465,14 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
         moe_unit u; u.expert = tid; u.m = c; u.row0 = excl; u.pad = 0;
         a.units[uidx] = u;
         a.active_ids[uidx] = tid;
-        if (a.host_units) a.host_units[uidx] = u;
+        if (a.host_units) host_store_unit(a.host_units, uidx, tid, c, excl);
       }
     }
     if (tid == NT - 1) {
       const int tot_act = ba + sa;
       a.offsets[E] = bc + sc;
       *a.n_active = tot_act < a.max_units ? tot_act : a.max_units;
-      if (a.host_units) *a.host_n_active = tot_act < a.max_units ? tot_act : a.max_units;
+      if (a.host_units) host_store_i32(a.host_n_active, tot_act < a.max_units ? tot_act : a.max_units);
       s_tot = tot_act;
     }
     __syncthreads();
@@ -497,9 +517,9 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
     __syncthreads();
   }
   if (a.host_units) {
-    __threadfence_system();
+    host_stores_done();
     __syncthreads();
-    if (tid == 0) __hip_atomic_store(a.host_seq, a.host_seq_val, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (tid == 0) __hip_atomic_store(a.host_seq, a.host_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
   }
 }
 
@@ -601,7 +621,6 @@ struct GemvArgs {
 
 // global-address-space loads (pointers that come out of the slot table are generic
 // to the compiler and would otherwise become flat_load)
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const u32x4_t g_uint4;
 typedef __attribute__((address_space(1))) const unsigned int g_u32;
 static __device__ __forceinline__ uint4 ldg_u4(const void *p) {
@@ -614,11 +633,6 @@ static __device__ __forceinline__ float sum8_bf16(const uint4 &v) {
          bf16hi(v.w);
 }
 
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-// buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
-static __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
-}
 static __device__ __forceinline__ uint4 bload16(rsrc_t r, int voff, int soff) {
   const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
   return make_uint4(v.x, v.y, v.z, v.w);
@@ -824,7 +838,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       moe_unit un; un.expert = my_e; un.m = 1; un.row0 = pos; un.pad = 0;
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
-      if (a.r_host_units) a.r_host_units[pos] = un;
+      if (a.r_host_units) host_store_unit(a.r_host_units, pos, my_e, 1, pos);
       if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; a.r_unit_w[pos] = wgt; }
     }
 #pragma unroll
@@ -837,9 +851,9 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       }
     }
     if (lane == 0) { a.r_offsets[E] = k; *a.r_n_active = k; }
-    if (a.r_host_seq) {  // the host polls the sequence word: units first, system-scope fence, then the word
-      __threadfence_system();
-      if (lane == 0) __hip_atomic_store(a.r_host_seq, a.r_host_seq_val, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    if (a.r_host_seq) {  // the host polls the sequence word: it follows once the unit stores have completed
+      host_stores_done();
+      if (lane == 0) __hip_atomic_store(a.r_host_seq, a.r_host_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
   return wk;
