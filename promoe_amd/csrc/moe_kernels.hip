@@ -379,6 +379,24 @@ struct RouteArgs {
   moe_unit *host_units; int *host_n_active; int *host_seq; int host_seq_val, pad_;
 };
 
+// maximum over the 64 lanes of a wave, built from DPP row shifts and broadcasts (no LDS traffic)
+static __device__ __forceinline__ float wave_max_f32(float x) {
+  // inclusive max-scan inside each row of 16 lanes, then rows 0->1, 2->3, then 1->3: lane 63 holds the result
+#define WMAX_STEP(ctrl, rmask)                                                                          \
+  {                                                                                                     \
+    const int xi = __builtin_bit_cast(int, x);                                                          \
+    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, ctrl, rmask, 0xf, false))); \
+  }
+  WMAX_STEP(0x111, 0xf)  // row_shr:1
+  WMAX_STEP(0x112, 0xf)  // row_shr:2
+  WMAX_STEP(0x114, 0xf)  // row_shr:4
+  WMAX_STEP(0x118, 0xf)  // row_shr:8
+  WMAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+  WMAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef WMAX_STEP
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
 // top-k (one wave per token) and stable dispatch by ONE workgroup of NW waves; the bodies of
 // k_topk and k_dispatch.  With host_units set the unit list also goes straight into pinned host
 // memory, followed behind a system-scope fence by the sequence word the host polls.
@@ -398,9 +416,7 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
       // written by other workgroups of this launch: read at device scope, past the L1
       v[r] = (e < E) ? __hip_atomic_load(a.logits + (size_t)t * a.ldl + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : NEG;
     }
-    float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    const float mx = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
     float den = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
@@ -409,18 +425,16 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
     for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
     float sel_v = 0.f, sum_sel = 0.f;
     for (int j = 0; j < k; ++j) {
-      float bv = v[0];
-      int bi = lane;
+      // the maximum, then the lowest expert id that holds it: lowest column first, then lowest lane
+      const float bv = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+      int wr = -1, wl = 0;
 #pragma unroll
-      for (int r = 1; r < 4; ++r) {
-        if (v[r] > bv) { bv = v[r]; bi = lane + 64 * r; }
+      for (int r = 0; r < 4; ++r) {
+        const unsigned long long mr = __ballot(v[r] == bv);
+        if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
       }
-#pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) {
-        const float ov = __shfl_xor(bv, m, 64);
-        const int oi = __shfl_xor(bi, m, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-      }
+      if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
+      const int bi = wl + 64 * wr;
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         if (bi == lane + 64 * r) v[r] = NEG;
@@ -709,23 +723,6 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
 // lowest expert id that holds the maximum - the order and the tie rule of k_topk.  One spare
 // workgroup publishes the routing (indices, weights, dispatch arrays, unit list) for the
 // later kernels and the host.
-static __device__ __forceinline__ float wave_max_f32(float x) {
-  // inclusive max-scan inside each row of 16 lanes, then rows 0->1, 2->3, then 1->3: lane 63 holds the result
-#define WMAX_STEP(ctrl, rmask)                                                                          \
-  {                                                                                                     \
-    const int xi = __builtin_bit_cast(int, x);                                                          \
-    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, ctrl, rmask, 0xf, false))); \
-  }
-  WMAX_STEP(0x111, 0xf)  // row_shr:1
-  WMAX_STEP(0x112, 0xf)  // row_shr:2
-  WMAX_STEP(0x114, 0xf)  // row_shr:4
-  WMAX_STEP(0x118, 0xf)  // row_shr:8
-  WMAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
-  WMAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
-#undef WMAX_STEP
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
-}
-
 template <int NR>
 static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &a, int lane, int w) {
   GemvWork wk;
@@ -771,6 +768,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       const unsigned long long mr = __ballot(v[r] == best);
       if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
     }
+    if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
 #pragma unroll
     for (int r = 0; r < NR; ++r)
       if (r == wr) {
