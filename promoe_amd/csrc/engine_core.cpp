@@ -509,6 +509,28 @@ static void resolve_using(moe_engine *eng, Expert *v, std::unique_lock<std::mute
     if (st == kReady) { v->status = kIdle; return; }
     if (st == kIdle) return;
     if (st == kUsing) {
+      if (v->seq_ptr) {
+        // released against a sequence word: it normally arrives with the caller's next launch; if it
+        // does not (the caller stopped, or took another path), an event recorded now proves the same
+        const volatile int *sp = v->seq_ptr;
+        const int need = v->seq_need;
+        lk.unlock();
+        const auto t0 = std::chrono::steady_clock::now();
+        bool reached = false;
+        while (!(reached = (int)((unsigned)*sp - (unsigned)need) >= 0) &&
+               std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(100)) {}
+        if (!reached) {
+          lk.lock();
+          if (!eng->proof_event) eng->proof_event = eng->be->event_create();
+          void *pe = eng->proof_event;
+          if (pe) eng->be->event_record(pe, eng->be->compute_stream());
+          lk.unlock();
+          if (pe) eng->be->event_sync(pe);
+        }
+        lk.lock();
+        if (v->status.load() == kUsing && v->seq_ptr == sp && v->seq_need == need) { v->seq_ptr = nullptr; v->status = kReady; }
+        continue;
+      }
       void *ev = v->event;
       if (ev) { lk.unlock(); eng->be->event_sync(ev); lk.lock(); }
       if (v->status.load() == kUsing) v->status = kReady;
@@ -774,7 +796,10 @@ extern "C" int moe_expert_status(moe_engine *eng, int layer, int expert) {
   if (!eng || check_le(eng, layer, expert)) return MOE_EINVAL;
   std::lock_guard<std::mutex> lk(eng->mu);
   Expert *e = eng->ex(layer, expert);
-  if (e->status.load() == kUsing && (!e->event || eng->be->event_done(e->event))) e->status = kReady;
+  if (e->status.load() == kUsing && (e->seq_ptr ? e->seq_reached() : (!e->event || eng->be->event_done(e->event)))) {
+    e->seq_ptr = nullptr;
+    e->status = kReady;
+  }
   return e->status.load();
 }
 extern "C" int moe_is_in_cache(moe_engine *eng, int layer, int expert) {
@@ -874,6 +899,7 @@ extern "C" int moe_expert_launched(moe_engine *eng, int layer, int expert) {
             expert, e->status.load());
   if (!e->own_event) e->own_event = eng->be->event_create();
   e->event = e->own_event;
+  e->seq_ptr = nullptr;
   if (e->event) eng->be->event_record(e->event, eng->be->compute_stream());
   e->status = kUsing;
   eng->cv_state.notify_all();
@@ -940,6 +966,25 @@ extern "C" int moe_release_experts(moe_engine *eng, int layer, const int64_t *id
       if (ev) eng->be->event_record(ev, eng->be->compute_stream());
     }
     x->event = ev;
+    x->seq_ptr = nullptr;
+    x->status = kUsing;
+  }
+  eng->cv_state.notify_all();
+  return MOE_OK;
+}
+
+int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need) {
+  ENG_GUARD(eng);
+  if (int rc = check_le(eng, layer, 0)) return rc;
+  std::lock_guard<std::mutex> lk(eng->mu);
+  for (int64_t i = 0; i < n; ++i) {
+    if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
+    Expert *x = eng->ex(layer, (int)ids[i]);
+    ENG_CHECK(eng, x->status.load() == kLaunching, "transfer launching->using, but expert %d.%d is in state %d", layer,
+              (int)ids[i], x->status.load());
+    x->event = nullptr;
+    x->seq_ptr = seq_ptr;
+    x->seq_need = seq_need;
     x->status = kUsing;
   }
   eng->cv_state.notify_all();
@@ -961,6 +1006,7 @@ extern "C" int moe_release_layer(moe_engine *eng, int layer) {
       if (ev) eng->be->event_record(ev, eng->be->compute_stream());
     }
     x->event = ev;
+    x->seq_ptr = nullptr;
     x->status = kUsing;
   }
   eng->cv_state.notify_all();

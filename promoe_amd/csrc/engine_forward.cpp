@@ -360,7 +360,11 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                     s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, nullptr, nullptr, 0,
                                     w2c ? 4 : 2, sgo, y, st)))
       return rc;
-    if (!now_ids.empty() && (rc = moe_release_experts(eng, layer, now_ids.data(), (int64_t)now_ids.size()))) return rc;
+    // no event in the stream (one costs the step about 4 us of GPU time): the experts count as in use until
+    // the routing word of a LATER one-token step arrives, whose kernel starts behind everything queued here
+    if (!now_ids.empty() &&
+        (rc = moe_release_experts_seq(eng, layer, now_ids.data(), (int64_t)now_ids.size(), s->opt_seq, seq + 1)))
+      return rc;
     s->sub_cursor = 0;
     for (int64_t id : later) {
       if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;

@@ -67,6 +67,11 @@ struct Expert {
   std::atomic<int> status{kIdle};
   void *event = nullptr;      // (not owned) event recorded after the last launch that reads the slot
   void *own_event = nullptr;  // per-expert event of the stepwise API (prefetcher.cpp:263)
+  // alternative to `event`: the launches that read the slot are over once *seq_ptr has reached seq_need
+  // (a word a LATER kernel of the same stream stores into host memory when it starts)
+  const volatile int *seq_ptr = nullptr;
+  int seq_need = 0;
+  bool seq_reached() const { return !seq_ptr || (int)((unsigned)*seq_ptr - (unsigned)seq_need) >= 0; }
   size_t total_alloc() const { size_t t = 0; for (auto &c : chunks) t += c.alloc; return t; }
 };
 
@@ -177,6 +182,7 @@ struct moe_engine {
   std::vector<char> table_dirty;  // per layer
   std::vector<void *> dummy_bufs;
   std::vector<void *> layer_event;  // one per layer, used by moe_release_layer
+  void *proof_event = nullptr;      // recorded by the fetch thread when a sequence word does not come
   std::vector<int> layer_complete;  // fully fetched resident experts per layer
 
   // NN / MIN policy state (cache.hpp:262-266)
@@ -216,6 +222,8 @@ int engine_fail(moe_engine *eng, const char *fmt, ...) __attribute__((format(pri
 void moe_forward_free(LayerState *);
 void moe_predictor_free(moe_engine *eng);
 int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H);
+// launching -> using without an event: the experts count as in use until *seq_ptr reaches seq_need
+int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need);
 // account demand hits of experts that were launched without a host round trip
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);
 // collect the routing results of earlier moe_forward calls (wait: block until all are in)

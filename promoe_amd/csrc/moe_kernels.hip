@@ -799,6 +799,26 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
 
   if (publisher) {  // publish the routing: weights as in k_topk, arrays as in k_dispatch (T = 1)
     wk.m = 0;       // no weight tiles for this workgroup
+    // position of a pair = rank of its expert id among the selected
+    int below[NR], cb = 0;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) { below[r] = cb; cb += __popcll(msel[r]); }
+    int pos = 0;
+    {
+      const int r_ = my_e >> 6, l_ = my_e & 63;
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+        if (r == r_) pos = below[r] + __popcll(msel[r] & ((1ull << l_) - 1ull));
+    }
+    // a host that waits for the routing gets it first: the unit list, then (once those stores have
+    // completed) the sequence word it polls; weights and dispatch arrays follow
+    if (a.r_host_units) {
+      if (lane < k) host_store_unit(a.r_host_units, pos, my_e, 1, pos);
+      if (a.r_host_seq) {
+        host_stores_done();
+        if (lane == 0) __hip_atomic_store(a.r_host_seq, a.r_host_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+    }
     // sum over the selected logits in choice order (the order of k_topk), maximum = choice 0
     mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_v), 0));
 #pragma unroll 1
@@ -818,16 +838,8 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       wgt = ex / den;
       if (a.r_mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
     }
-    // dispatch of the k pairs of the one token: position = rank of the expert id among the selected
-    int below[NR], cb = 0;
-#pragma unroll
-    for (int r = 0; r < NR; ++r) { below[r] = cb; cb += __popcll(msel[r]); }
+    // dispatch of the k pairs of the one token
     if (lane < k) {
-      const int r_ = my_e >> 6, l_ = my_e & 63;
-      int pos = 0;
-#pragma unroll
-      for (int r = 0; r < NR; ++r)
-        if (r == r_) pos = below[r] + __popcll(msel[r] & ((1ull << l_) - 1ull));
       a.r_idx[lane] = my_e;
       a.r_w[lane] = wgt;
       a.r_sorted_pair[pos] = lane;
@@ -836,7 +848,6 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       moe_unit un; un.expert = my_e; un.m = 1; un.row0 = pos; un.pad = 0;
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
-      if (a.r_host_units) host_store_unit(a.r_host_units, pos, my_e, 1, pos);
       if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; a.r_unit_w[pos] = wgt; }
     }
 #pragma unroll
@@ -849,10 +860,6 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       }
     }
     if (lane == 0) { a.r_offsets[E] = k; *a.r_n_active = k; }
-    if (a.r_host_seq) {  // the host polls the sequence word: it follows once the unit stores have completed
-      host_stores_done();
-      if (lane == 0) __hip_atomic_store(a.r_host_seq, a.r_host_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
   }
   return wk;
 }
