@@ -401,27 +401,45 @@ def main():
     # ---- the configured cache rate: 24 of 64 experts per layer resident, LRU ------------
     cache_run = None
     if not a.no_cache_run:
-        pm2 = stack.engine(16, cache_rate=0.375, cache_policy="lru", num_predict_expert_per_layer=0,
-                           reorder_experts=True, early_preempt=True)
-        xs = stack.acts(T, 64, seed=3)
-        xs_out = torch.empty_like(xs[0])
-        n2 = 40 * L_
-        for i in range(10 * L_):              # fill the slots along the Zipf popularity
-            pm2.forward(i % L_, xs[(i // L_) % len(xs)], out=xs_out)
-        torch.cuda.synchronize()
-        c0 = pm2.counters()
-        t0 = time.perf_counter()
-        for i in range(n2):
-            pm2.forward(i % L_, xs[(10 + i // L_) % len(xs)], out=xs_out)
-        torch.cuda.synchronize()
-        d3 = time.perf_counter() - t0
-        c2 = pm2.counters()
-        hit, miss = c2["hit"] - c0["hit"], c2["miss"] - c0["miss"]
-        cache_run = {"cache_rate": 0.375, "policy": "lru", "tokens_per_s": T * n2 / d3, "ms_per_step": d3 / n2 * 1e3,
-                     "hit_rate": hit / max(hit + miss, 1), "h2d_GB": (c2["h2d_bytes"] - c0["h2d_bytes"]) / 1e9,
-                     "h2d_GBps": (c2["h2d_bytes"] - c0["h2d_bytes"]) / d3 / 1e9, "steps": n2,
-                     "misses": miss, "wait_us_per_miss": (c2["wait_us"] - c0["wait_us"]) / max(miss, 1)}
-        pm2.close()
+        def cache_leg(predict):
+            cfg = dict(cache_rate=0.375, cache_policy="lru", reorder_experts=True, early_preempt=True,
+                       num_predict_expert_per_layer=k if predict else 0)
+            if predict:
+                cfg.update(layer_predict_interval=1, layer_predict_max_window=10, limit_layer_0_window=10)
+            pm2 = stack.engine(16, **cfg)
+            if predict:
+                # the built-in predictor with the destination layer's gate as the model of every pair; this
+                # bench feeds ONE hidden state to all layers of a token, so these predictions are exact: what
+                # prefetching can hide when the predictor is right
+                for src, (f0, f1) in enumerate(pm2.predictor_windows()):
+                    for dst in range(f0, f1):
+                        pm2.set_predictor_model(src, dst, stack.gate_w[dst], stack.gate_bias[dst])
+                pm2.start_predictor()
+            xs2 = stack.acts(T, 64, seed=3)
+            out2 = torch.empty_like(xs2[0])
+            n2 = 40 * L_
+            for i in range(10 * L_):              # fill the slots along the Zipf popularity
+                pm2.forward(i % L_, xs2[(i // L_) % len(xs2)], out=out2)
+            torch.cuda.synchronize()
+            c0 = pm2.counters()
+            t0 = time.perf_counter()
+            for i in range(n2):
+                pm2.forward(i % L_, xs2[(10 + i // L_) % len(xs2)], out=out2)
+            torch.cuda.synchronize()
+            d3 = time.perf_counter() - t0
+            c2 = pm2.counters()
+            pm2.close()
+            dl = {kk: c2[kk] - c0[kk] for kk in ("hit", "miss", "prefetch_hit", "prefetch_miss", "ready", "unready",
+                                                 "wait_us", "h2d_bytes")}
+            return {"cache_rate": 0.375, "policy": "lru", "tokens_per_s": T * n2 / d3, "ms_per_step": d3 / n2 * 1e3,
+                    "hit_rate": dl["hit"] / max(dl["hit"] + dl["miss"], 1), "h2d_GB": dl["h2d_bytes"] / 1e9,
+                    "h2d_GBps": dl["h2d_bytes"] / d3 / 1e9, "steps": n2, "misses": dl["miss"],
+                    "wait_us_per_miss": dl["wait_us"] / max(dl["miss"], 1) if not predict else None,
+                    "prefetch_hits": dl["prefetch_hit"], "prefetch_copies": dl["prefetch_miss"],
+                    "ready_rate": dl["ready"] / max(dl["ready"] + dl["unready"], 1), "wait_us_total": dl["wait_us"]}
+        cache_run = cache_leg(False)
+        if T == 1:
+            cache_run["with_predictor"] = cache_leg(True)
 
     prefill = None
     if not a.no_prefill:

@@ -557,6 +557,9 @@ static void fetch_thread_main(moe_engine *eng) {
     }
     Expert *e = eng->current.e;
     const int start = eng->current.start, stop = eng->current.stop;
+    // a kernel may be reading any slot of this group through a table snapshot: the slot stays as it is
+    // until the caller has seen that kernel's selection and protected what it uses
+    while (eng->group_of(e->layer).guard > 0 && !eng->exiting) eng->cv_state.wait_for(lk, std::chrono::microseconds(50));
     if (Expert *v = eng->current.wait_victim) {
       resolve_using(eng, v, lk);
       if (v->slot == e->slot && !in_cache(eng, v)) { set_table(eng, v, false); v->slot = -1; }
@@ -790,6 +793,30 @@ extern "C" int moe_flush_table(moe_engine *eng, int layer, void *stream) {
   eng->table_dirty[layer] = 0;
   const size_t o = (size_t)layer * eng->cfg.num_expert;
   return eng->be->flush_table(eng->d_table + o, eng->h_table + o, eng->cfg.num_expert, stream);
+}
+
+int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resident_out) {
+  ENG_GUARD(eng);
+  if (int rc = check_le(eng, layer, 0)) return rc;
+  if (!eng->slots_ready) { moe_set_error("slots not initialised"); return MOE_ESTATE; }
+  std::lock_guard<std::mutex> lk(eng->mu);
+  const size_t o = (size_t)layer * eng->cfg.num_expert;
+  if (eng->table_dirty[layer]) {
+    eng->table_dirty[layer] = 0;
+    if (int rc = eng->be->flush_table(eng->d_table + o, eng->h_table + o, eng->cfg.num_expert, stream)) return rc;
+  }
+  for (int e = 0; e < eng->cfg.num_expert; ++e) resident_out[e] = eng->h_table[o + e] != 0;
+  eng->group_of(layer).guard++;
+  return MOE_OK;
+}
+
+void moe_guard_release(moe_engine *eng, int layer) {
+  {
+    std::lock_guard<std::mutex> lk(eng->mu);
+    Group &g = eng->group_of(layer);
+    if (g.guard > 0) g.guard--;
+  }
+  eng->cv_state.notify_all();
 }
 
 extern "C" int moe_expert_status(moe_engine *eng, int layer, int expert) {

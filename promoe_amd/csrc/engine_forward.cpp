@@ -283,19 +283,14 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
-  // One token, demand fetching only (no prefetch producer that could evict behind our back) and the
-  // fetch thread idle: start the expert kernels on whatever is resident BEFORE the host knows the
-  // routing.  The w13 kernel routes by itself, skips experts whose table entry is 0 and hands the unit
-  // list to the host through pinned memory; the host then runs the cache hooks in the reference's
-  // order (hits were computed already, misses are fetched and computed one by one) while the GPU works.
-  bool optimistic = false;
-  if (!all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && eng->cfg.early_preempt &&
-      eng->cfg.reorder_experts && eng->cfg.num_predict_expert_per_layer == 0 && !eng->predictor_attached &&
-      (size_t)d.H * 2 + 8192 <= 60 * 1024) {
-    std::lock_guard<std::mutex> lk(eng->mu);
-    optimistic = eng->current.e == nullptr && eng->precise_q.empty();
-    for (auto &q : eng->layer_q) optimistic = optimistic && q.empty();
-  }
+  // One token that may meet non-resident experts: start the expert kernels on whatever is resident BEFORE
+  // the host knows the routing.  The w13 kernel routes by itself, skips experts whose table entry is 0 and
+  // hands the unit list to the host through pinned memory; the host then runs the cache hooks in the
+  // reference's order (hits were computed already, misses are fetched and computed one by one) while the GPU
+  // works.  From the table snapshot until the hooks have marked the hits, the layer's slot group is guarded:
+  // prefetch and demand traffic may evict, but no copy into one of its slots starts.
+  const bool optimistic = !all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 &&
+                          eng->cfg.early_preempt && eng->cfg.reorder_experts && (size_t)d.H * 2 + 8192 <= 60 * 1024;
   if (optimistic) {
     if (!d.gate_bias) {
       if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
@@ -307,13 +302,14 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     }
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
-    if ((rc = moe_flush_table(eng, layer, st))) return rc;
     // what the kernel will find resident: exactly these experts get computed by it
     std::vector<char> resident_at_launch(E);
-    {
-      std::lock_guard<std::mutex> lk(eng->mu);
-      for (int e = 0; e < E; ++e) resident_at_launch[e] = eng->h_table[(size_t)layer * E + e] != 0;
-    }
+    if ((rc = moe_flush_table_guarded(eng, layer, st, resident_at_launch.data()))) return rc;
+    struct GuardRelease {  // on every way out, errors included
+      moe_engine *eng; int layer; bool armed;
+      void release() { if (armed) { armed = false; moe_guard_release(eng, layer); } }
+      ~GuardRelease() { release(); }
+    } guard{eng, layer, true};
     const int seq = ++s->seq_counter;
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
@@ -342,13 +338,20 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     {
       std::lock_guard<std::mutex> lk(eng->mu);
       for (int i = 0; i < n_act; ++i) {
-        // resident at launch: computed already (and a hit, since nothing could evict it in between);
-        // a missed expert whose copy has landed meanwhile is `launching` too, but still has to be computed
-        if (resident_at_launch[(int)ids[i]]) now_ids.push_back(ids[i]);
-        else later.push_back(ids[i]);
+        // resident at launch and still there (now `launching`: nobody overwrites it): computed already.
+        // A missed expert whose copy has landed meanwhile is `launching` too, but still has to be computed;
+        // so has one that a prefetch evicted between the snapshot and now (its slot was intact while the
+        // guard stood, but is free to be overwritten from here on).
+        Expert *ex = eng->ex(layer, (int)ids[i]);
+        if (resident_at_launch[(int)ids[i]] && ex->status.load() == kLaunching && ex->num_ready == eng->cfg.num_per_expert_param &&
+            eng->h_table[(size_t)layer * E + ids[i]] != 0)
+          now_ids.push_back(ids[i]);
+        else
+          later.push_back(ids[i]);
       }
       eng->ctr.ready += (uint64_t)now_ids.size();
     }
+    guard.release();
     // the w2 pass goes out now that the routing is known (the w13 kernel is still running): with
     // every selected expert resident it also combines, otherwise it leaves partial rows for the
     // experts computed below and the combine after them

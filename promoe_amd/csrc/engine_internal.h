@@ -131,6 +131,9 @@ struct Group {
   std::unique_ptr<Policy> policy;
   std::vector<int> unused;  // free slot indices; taken from the back
   size_t full_len = 0;
+  // > 0 while a kernel runs on a snapshot of the slot table whose selection the host does not know yet:
+  // evictions go on, but no copy into a slot of this group starts (fetch thread waits)
+  int guard = 0;
 };
 
 struct CopyTask {
@@ -223,6 +226,10 @@ void moe_forward_free(LayerState *);
 void moe_predictor_free(moe_engine *eng);
 int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H);
 // launching -> using without an event: the experts count as in use until *seq_ptr reaches seq_need
+// slot table of `layer` to the device (if changed) and the same residency as a byte vector, taken in one
+// critical section together with raising the group's guard; moe_guard_release lowers it again
+int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resident_out);
+void moe_guard_release(moe_engine *eng, int layer);
 int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need);
 // account demand hits of experts that were launched without a host round trip
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);
