@@ -1060,7 +1060,12 @@ extern "C" int moe_prefetch_layer(moe_engine *eng, int layer, const int64_t *ids
   eng->budget--;
   // PrefetchLayerTask (prefetcher.cpp:585-611)
   if (!eng->layer_q[layer].empty()) { moe_set_error("prefetch request for layer %d while its queue is not empty", layer); return MOE_ESTATE; }
-  if (eng->current.e && eng->current.e->layer == layer) { moe_set_error("prefetch request for layer %d while a copy of that layer is in flight", layer); return MOE_ESTATE; }
+  if (eng->current.e && eng->current.e->layer == layer) {
+    moe_set_error("prefetch request for layer %d while a copy of that layer is in flight (expert %d, chunks %d..%d, %s, guard %d, progress %ld, budget %ld)",
+                  layer, eng->current.e->idx, eng->current.start, eng->current.stop, eng->current.precise ? "demand" : "speculative",
+                  eng->group_of(layer).guard, eng->progress, eng->budget);
+    return MOE_ESTATE;
+  }
   if (layer == 0 && eng->cfg.limit_layer_0_num_predict != -1) n = std::min<int64_t>(n, eng->cfg.limit_layer_0_num_predict);
   const int P = eng->cfg.num_per_expert_param;
   for (int64_t i = 0; i < n; ++i) {

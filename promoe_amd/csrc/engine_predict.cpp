@@ -11,6 +11,7 @@
 // scores are x . W^T + b, computed by the gate-logits kernel on the compute stream right behind the
 // layer input; the host thread sees them through pinned memory and an event.
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstring>
 #include <deque>
@@ -141,6 +142,12 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
         std::partial_sort(order.begin(), order.begin() + n, order.end(),
                           [&](int a, int b) { return s[a] > s[b] || (s[a] == s[b] && a < b); });
         ids.assign(order.begin(), order.begin() + n);
+      }
+      {  // a request may not overlap a copy of its own layer (prefetcher.cpp:585-611 checks it): the copy in
+         // flight is a leftover of the layer's previous turn and is over in a moment
+        std::unique_lock<std::mutex> lk(eng->mu);
+        for (int spin = 0; spin < 200 && !eng->exiting && eng->current.e && eng->current.e->layer == dst; ++spin)
+          eng->cv_state.wait_for(lk, std::chrono::microseconds(100));
       }
       const int rc = moe_prefetch_layer(eng, dst, ids.data(), n, 1);
       if (rc == MOE_ESTATE && eng->exiting) return;

@@ -303,3 +303,34 @@ def test_builtin_predictor_prefetches_what_the_next_layers_route_to(cuda):
     assert c1["miss"] * 2 < c0["miss"]
     print(f"  demand misses {c0['miss']} -> {c1['miss']}, ready {c0['ready']} -> {c1['ready']}, "
           f"prefetch hits {c1['prefetch_hit']}", flush=True)
+
+
+def test_one_token_path_under_wrong_prefetches(cuda):
+    """A predictor with random models keeps evicting experts the tokens are about to use, while the one-token
+    path launches its kernels on table snapshots: the outputs must stay the oracle's (the slot-group guard and
+    the late classification of evicted experts are what this exercises)."""
+    print("case engine_wrong_prefetch", flush=True)
+    Lyr, E, k, H = 3, 16, 4, 256
+    layers = [Int4Layer(H=H, I=128, E=E, I_sh=128, seed=60 + l, zipf=1.1) for l in range(Lyr)]
+    pm = build_engine(layers, k, cuda, cache_rate=0.3, cache_policy="lru", num_predict_expert_per_layer=k,
+                      layer_predict_interval=1, layer_predict_max_window=2, limit_layer_0_window=2)
+    g = torch.Generator().manual_seed(5)
+    for src, (a, b) in enumerate(pm.predictor_windows()):
+        for dst in range(a, b):
+            pm.set_predictor_model(src, dst, torch.randn(E, H, generator=g).to(torch.bfloat16).to(cuda), None)
+    pm.start_predictor()
+    worst = 0.0
+    for t in range(30):
+        for l in range(Lyr):
+            x = O.synth_acts(1, H, seed=900 + t * Lyr + l)
+            y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            ref = ref_forward(layers[l], x, k, 0)
+            worst = max(worst, float(np.abs(y.float().cpu().numpy() - ref["out"]).max() / np.abs(ref["out"]).max()))
+    pm.drain()
+    c = pm.counters()
+    pm.close()
+    print(f"  worst rel err {worst:.3e}, misses {c['miss']}, prefetch copies {c['prefetch_miss']}, evictions {c['evictions']}",
+          flush=True)
+    assert worst <= TOL
+    assert c["prefetch_miss"] > 0 and c["evictions"] > 0 and c["miss"] > 0
