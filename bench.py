@@ -379,7 +379,7 @@ def main():
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this kernel at this
                 # workload (T=1, 27 layers), scaled by a copy kernel of known size; not measurable in-process
-                "traffic": 24252314 if (T == 1 and L_ == 27) else None,
+                "traffic": 24245555 if (T == 1 and L_ == 27) else None,
                 "algorithmic_bytes_per_launch": w13_bytes_k, "avg_launch_us": w13_us,
                 "distinct_routed_experts_per_launch": D_k,
                 "method": "%d back-to-back launches between one HIP event pair" % n_k}
