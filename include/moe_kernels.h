@@ -123,7 +123,7 @@ int moe_route_decode(const void *x_bf16, const void *wg_bf16, const float *bias,
 /* k1b + k2 in one launch (one workgroup) for decode batches: T <= 16, E <= 256, T*k <= 512; same
  * results, bit for bit, as moe_topk + moe_dispatch.  units_host_out / n_active_host_out /
  * seq_host_out (optional, pinned HOST memory): the kernel also stores the unit list and its length
- * there and then, behind a system-scope fence, seq_value into *seq_host_out. */
+ * there and then, once those stores have completed, seq_value into *seq_host_out. */
 int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mode, int *idx, float *w,
                       int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                       moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
@@ -155,7 +155,7 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
  * unit_ws (optional): 32*k bytes of device memory; the first pass leaves the resolved units (slot
  * address, row) there and the w2 pass starts from one load instead of unit -> table -> address.
  * units_host_out / seq_host_out (optional, pinned HOST memory): the kernel also stores the k
- * units there and then, behind a system-scope fence, seq_value into *seq_host_out, so a host
+ * units there and then, once those stores have completed, seq_value into *seq_host_out, so a host
  * that polls the word gets the routing without a copy or an event.
  * phases: bit 0 = routing + w13 + SwiGLU, bit 1 = w2 into partial rows (needs the units of an
  * earlier bit-0 call), bit 2 = w2 and the weighted combine in ONE launch, straight into y_bf16 [H]

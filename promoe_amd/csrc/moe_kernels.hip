@@ -399,7 +399,7 @@ static __device__ __forceinline__ float wave_max_f32(float x) {
 
 // top-k (one wave per token) and stable dispatch by ONE workgroup of NW waves; the bodies of
 // k_topk and k_dispatch.  With host_units set the unit list also goes straight into pinned host
-// memory, followed behind a system-scope fence by the sequence word the host polls.
+// memory, followed (once those stores have completed) by the sequence word the host polls.
 template <int NW>
 static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx, int *s_cnt, int *s_off, int *s_run,
                                                   int *s_w, int *s_wsum, int *s_wact, int &s_tot) {

@@ -1,0 +1,17 @@
+// Stand-ins for the GPU entry points of the library in the host-only sanitizer builds: the engine
+// refers to them, the host backend never calls them.
+#include <cstdint>
+#include <cstdio>
+
+#define STUB(name) extern "C" int name(...) { fprintf(stderr, "kernel entry " #name " called in the host-only build\n"); return -1; }
+STUB(moe_gate_logits)
+STUB(moe_topk)
+STUB(moe_dispatch)
+STUB(moe_route_decode)
+STUB(moe_topk_dispatch)
+STUB(moe_experts_decode_int4)
+STUB(moe_decode_token_int4)
+STUB(moe_experts_decode_q4k)
+STUB(moe_experts_prefill)
+STUB(moe_combine)
+extern "C" int64_t moe_prefill_workspace_bytes(...) { return 0; }
