@@ -585,12 +585,14 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
   route_tail<4>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
 }
 
-// k1b + k2 in one launch for decode batches whose logits exist already: one workgroup of 16 waves
-__global__ __launch_bounds__(1024) void k_topk_dispatch(const RouteArgs a) {
+// k1b + k2 in one launch for decode batches whose logits exist already: one workgroup of NW waves
+// (a wave per token in the top-k phase: 4 waves are enough for T <= 4 and their barriers are cheaper)
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void k_topk_dispatch(const RouteArgs a) {
   __shared__ int s_idx[ROUTE_MAXP];
-  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[16 * 256];
-  __shared__ int s_wsum[16], s_wact[16], s_tot;
-  route_tail<16>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
+  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[NW * 256];
+  __shared__ int s_wsum[NW], s_wact[NW], s_tot;
+  route_tail<NW>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
 }
 
 // ---------------------------------------------------------------------------
@@ -1992,7 +1994,8 @@ extern "C" int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int
   a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
   a.host_units = units_host_out; a.host_n_active = n_active_host_out; a.host_seq = seq_host_out; a.host_seq_val = seq_value;
   moe_ktimer_begin(MOE_K_TOPK, (hipStream_t)stream);
-  hipLaunchKernelGGL(k_topk_dispatch, dim3(1), dim3(1024), 0, (hipStream_t)stream, a);
+  if (T <= 4) hipLaunchKernelGGL(k_topk_dispatch<4>, dim3(1), dim3(256), 0, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(k_topk_dispatch<16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, a);
   moe_ktimer_end(MOE_K_TOPK, (hipStream_t)stream);
   return moe_check_launch("k_topk_dispatch");
 }
