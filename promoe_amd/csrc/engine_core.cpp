@@ -1044,6 +1044,14 @@ extern "C" int moe_release_layer(moe_engine *eng, int layer) {
 // prefetch request hook
 // ---------------------------------------------------------------------------
 extern "C" int moe_prefetch_layer(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking) {
+  return moe_prefetch_layer_over(eng, layer, ids, n, blocking, false);
+}
+
+// over_copy: accept the request although a copy of the same layer is still in flight.  The copy is a leftover
+// of the layer's previous turn; the new tasks queue up behind it, and one that names the same expert is dropped
+// as a duplicate when its turn comes.  The hook above refuses, as the reference does; the built-in predictor
+// cannot: the copy may be held back by the slot-group guard of a forward that itself waits for this request.
+int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking, bool over_copy) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
   if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_prefetch_layer: bad ids"); return MOE_EINVAL; }
@@ -1060,7 +1068,7 @@ extern "C" int moe_prefetch_layer(moe_engine *eng, int layer, const int64_t *ids
   eng->budget--;
   // PrefetchLayerTask (prefetcher.cpp:585-611)
   if (!eng->layer_q[layer].empty()) { moe_set_error("prefetch request for layer %d while its queue is not empty", layer); return MOE_ESTATE; }
-  if (eng->current.e && eng->current.e->layer == layer) {
+  if (!over_copy && eng->current.e && eng->current.e->layer == layer) {
     moe_set_error("prefetch request for layer %d while a copy of that layer is in flight (expert %d, chunks %d..%d, %s, guard %d, progress %ld, budget %ld)",
                   layer, eng->current.e->idx, eng->current.start, eng->current.stop, eng->current.precise ? "demand" : "speculative",
                   eng->group_of(layer).guard, eng->progress, eng->budget);

@@ -230,6 +230,7 @@ int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int 
 // critical section together with raising the group's guard; moe_guard_release lowers it again
 int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resident_out);
 void moe_guard_release(moe_engine *eng, int layer);
+int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking, bool over_copy);
 int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need);
 // account demand hits of experts that were launched without a host round trip
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);

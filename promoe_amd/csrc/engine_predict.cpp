@@ -143,13 +143,17 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
                           [&](int a, int b) { return s[a] > s[b] || (s[a] == s[b] && a < b); });
         ids.assign(order.begin(), order.begin() + n);
       }
-      {  // a request may not overlap a copy of its own layer (prefetcher.cpp:585-611 checks it): the copy in
-         // flight is a leftover of the layer's previous turn and is over in a moment
+      {  // a copy of this layer still in flight is a leftover of the layer's previous turn and normally over
+         // in a moment: give it that moment, so that the new tasks do not queue behind it for nothing
         std::unique_lock<std::mutex> lk(eng->mu);
-        for (int spin = 0; spin < 200 && !eng->exiting && eng->current.e && eng->current.e->layer == dst; ++spin)
-          eng->cv_state.wait_for(lk, std::chrono::microseconds(100));
+        const auto t0 = std::chrono::steady_clock::now();
+        while (!eng->exiting && eng->current.e && eng->current.e->layer == dst &&
+               std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(500))
+          eng->cv_state.wait_for(lk, std::chrono::microseconds(50));
       }
-      const int rc = moe_prefetch_layer(eng, dst, ids.data(), n, 1);
+      // ... but not for ever: the copy may be waiting for the slot-group guard of the very forward that waits
+      // for this request
+      const int rc = moe_prefetch_layer_over(eng, dst, ids.data(), n, 1, true);
       if (rc == MOE_ESTATE && eng->exiting) return;
       if (rc != MOE_OK) {  // keep the layer's progress in step so that report_one_layer does not wait for ever
         predictor_fail(eng, p, "prefetch_layer");

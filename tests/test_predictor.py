@@ -111,3 +111,39 @@ def test_start_needs_every_model():
     with pytest.raises(L.MoeError, match="no model"):
         pm.start_predictor()
     pm.close()
+
+
+def test_request_over_a_leftover_copy_of_the_same_layer(monkeypatch):
+    """Layer 0 is predicted from its own input, so a wrong prediction's copy can still be running when the
+    next token asks for layer 0 again.  The hook refuses such a request (as the reference does); the
+    built-in predictor queues it behind the copy instead of failing the forward."""
+    monkeypatch.setenv("MOE_HOST_COPY_DELAY_US", "100000")             # every copy takes 100 ms
+    Lyr, E, k, H = 2, 8, 2, 64
+    pm = make(Lyr, E, k, cache_rate=0.5, cache_policy="lru", num_predict_expert_per_layer=2,
+              layer_predict_interval=1, layer_predict_max_window=2, limit_layer_0_window=2,
+              predict_input_mode="moe_layer_logits")
+    assert pm.predictor_windows() == [(0, 2), (2, 2), (0, 0)]
+    for l in range(Lyr):                                               # warm the cache: experts 0..3 of each layer
+        for e in pm.report_one_layer(l, np.arange(4, dtype=np.int64)):
+            pm.report_one_expert(l, int(e)); pm.one_expert_done(l, int(e))
+        pm.one_moe_layer_done(l)
+    pm.drain()
+    absent = [[e for e in range(E) if pm.expert_status(l, e) == "idle"] for l in range(Lyr)]
+    assert all(len(a) == 4 for a in absent)
+    for dst in range(Lyr):                                             # always predict two experts that are not cached
+        w = np.zeros((E, H), np.float32)
+        w[absent[dst][0], 0] = 2.0; w[absent[dst][1], 0] = 1.0
+        pm.set_predictor_model(0, dst, _bf16(w), None)
+    pm.start_predictor()
+    xb = _bf16(np.ones((1, 1, H), np.float32))
+    for tok in range(3):                                               # the tokens only use cached experts: no demand copy to wait for
+        for l in range(Lyr):
+            pm.report_moe_layer_logits(l, xb)
+            cached = [e for e in range(E) if pm.expert_status(l, e) in ("ready", "using")][:k]
+            assert len(cached) == k
+            for e in pm.report_one_layer(l, np.array(cached, np.int64)):
+                pm.report_one_expert(l, int(e)); pm.one_expert_done(l, int(e))
+            pm.one_moe_layer_done(l)
+    pm.drain()
+    assert pm.predictor_stats()["requests"] == 3 * Lyr
+    pm.close()
