@@ -1234,6 +1234,11 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
 // Per tile (one quantisation group): D_g = sum (128+q) x ; acc += s_row (D_g - (128+z_row) X_tok,g).
 // ---------------------------------------------------------------------------
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+// two fp16 scales and their two zero nibbles (bits 0..7 of z) -> (s0, -s0 (128 + z0), s1, -s1 (128 + z1))
+static __device__ __forceinline__ float4 scale_zero_pair(u32 sc, u32 z) {
+  const float s0 = half_bits_to_f32((uint16_t)sc), s1 = half_bits_to_f32((uint16_t)(sc >> 16));
+  return make_float4(s0, -s0 * (128.f + (float)(z & 15)), s1, -s1 * (128.f + (float)((z >> 4) & 15)));
+}
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 static __device__ __forceinline__ bf16x8_t deq8_bf16(u32 w) {
@@ -1248,7 +1253,9 @@ static __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &x) {
 }
 
 template <bool SWIGLU, int CH, bool DEVUNITS>
-__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW) {
+__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW_R, const int RPW_S) {
+  constexpr int NP = 1, NB = 2 * NP;  // block pairs / 16-row blocks per iteration
+  constexpr int PF = 4;               // activation pieces in flight while staging
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
@@ -1263,40 +1270,44 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
     return;
   }
   const int K = c.K, G = c.G;
+  // block pairs of this workgroup: the shared expert sees every token, so its workgroups take fewer
+  const int RPW = (int)blockIdx.x < a.n_sh_blocks ? RPW_S : RPW_R;
   const int XS = K * 2 + 16;  // padded row stride (bytes): 16 token rows hit 16 distinct bank quads
   unsigned char *xs = smem;                                           // [TB][XS]
   float *xsum = (float *)(smem + (size_t)TB * XS);                    // [TB][G]
-  uint16_t *s_sc = (uint16_t *)(xsum + (((size_t)TB * G + 3) & ~(size_t)3));  // [2][G][16] fp16, 16-B aligned
-  unsigned char *s_zz = (unsigned char *)(s_sc + 2 * G * 16);         // [2][G][8]
-  float *red = (float *)(s_zz + 2 * G * 8);                           // [4][2][16 rows][16 tok]
+  // per (block, group, row): scale s and -s (128 + zero), so that a row's update is two fma's
+  float *s_f = xsum + (((size_t)TB * G + 3) & ~(size_t)3);            // [NB][G][16][2], 16-B aligned
+  float *red = s_f + NB * G * 32;                                     // [4][NB][16 rows][16 tok]
 
   const int GPW = (G - w + 3) >> 2;
   const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
   const int vec_per_row = K >> 3;
-  const int n_sc = 2 * G * 8, n_zz = 2 * G * 2;
+  const int n_sc = NB * G * 8;  // scale dwords (two rows each) of one iteration
 
   for (int t0 = 0; t0 < m; t0 += TB) {
     const int mc = (m - t0) < TB ? (m - t0) : TB;
-   // RPW consecutive (gate,up) / (row,row) block pairs per workgroup: the activations are
-   // staged once and the fixed per-workgroup cost is spread over more weight tiles
-   for (int pp = 0; pp < RPW; ++pp) {
+   // RPW consecutive (gate,up) / (row,row) block pairs per workgroup: the activations are staged
+   // once and the fixed per-workgroup cost is spread over more weight tiles
+   for (int pp = 0; pp < RPW; pp += NP) {
     const int b = wk.b * RPW + pp;
     const int rbA = 2 * b;
-    const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, 2u * G * 1024u);
-    const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, 2u * G * 32u);
-    const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, 2u * G * 8u);
+    const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
+    const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
+    const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
     // ---- straight-line load section ------------------------------------------------------
     const int row_first = row0 + t0;
     const int arow0 = c.gather ? c.gather[row_first] : row_first;
     const uint4 xv0 = bload16(rx, (tid < vec_per_row ? tid : 0) * 16, arow0 * c.act_stride * 2);
+    // scale dword e = (block, group, row pair j) and the zero dword that holds its two nibbles
+    const int zoff = ((tid >> 3) * 2 + ((tid & 7) >> 2)) * 4;
     const u32 msc0 = bload4(rs, tid * 4, 0), msc1 = bload4(rs, tid * 4, 1024);
-    const u32 mzz = bload4(rz, tid * 4, 0);
-    uint4 wa[CH], wb[CH];
+    const u32 mz0 = bload4(rz, zoff, 0), mz1 = bload4(rz, zoff, 256);
+    uint4 wt[CH][NB];
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       const int g = j < GPW ? w + 4 * j : 0;
-      wa[j] = bload16(rq, lane * 16, g * 1024);
-      wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+#pragma unroll
+      for (int n = 0; n < NB; ++n) wt[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
     }
     // ---- stage x rows (+ per-group sums over 128 values = 16 consecutive vectors) ----------
     if (pp == 0) {
@@ -1308,10 +1319,10 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
         if ((tid & 15) == 0) xsum[tid >> 4] = ps;
       }
     }
-    if (tid < n_sc) ((u32 *)s_sc)[tid] = msc0;
-    if (tid + 256 < n_sc) ((u32 *)s_sc)[tid + 256] = msc1;
-    if (tid < n_zz) ((u32 *)s_zz)[tid] = mzz;
-    // remaining (row, 256-vector chunk) pieces, four loads in flight at a time; piece 0 is
+    const int zsh = 8 * (tid & 3);  // the pair's nibbles inside its zero dword
+    if (tid < n_sc) ((float4 *)s_f)[tid] = scale_zero_pair(msc0, mz0 >> zsh);
+    if (tid + 256 < n_sc) ((float4 *)s_f)[tid + 256] = scale_zero_pair(msc1, mz1 >> zsh);
+    // remaining (row, 256-vector chunk) pieces, PF loads in flight at a time; piece 0 is
     // the early load above
     if (pp == 0) {
       const int cpr = (vec_per_row + 255) >> 8;  // chunks per row
@@ -1319,36 +1330,44 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
       // row index of every token of this pass, one per lane (lanes >= mc repeat the last)
       const int grow = row_first + (lane < mc ? lane : mc - 1);
       const int arow_l = c.gather ? c.gather[grow] : grow;
-      for (int pb = 1; pb < total; pb += 4) {
-        uint4 xb[4];
+      for (int pb = 1; pb < total; pb += PF) {
+        uint4 xb[PF];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int pi = pb + q < total ? pb + q : 0;
-          const int t = pi / cpr, ch = pi - t * cpr;
-          const int v = tid + 256 * ch;
-          const int arow = __builtin_amdgcn_readlane(arow_l, t);
-          xb[q] = bload16(rx, (v < vec_per_row ? v : 0) * 16, arow * c.act_stride * 2);
+        for (int q = 0; q < PF; ++q) {
+          // groups of four past the end are skipped (uniform branch); inside a group the index is clamped
+          if ((q & 3) == 0 || pb + (q & ~3) < total) {
+            const int pi = pb + q < total ? pb + q : 0;
+            const int t = pi / cpr, ch = pi - t * cpr;
+            const int v = tid + 256 * ch;
+            const int arow = __builtin_amdgcn_readlane(arow_l, t);
+            xb[q] = bload16(rx, (v < vec_per_row ? v : 0) * 16, arow * c.act_stride * 2);
+          } else {
+            xb[q] = make_uint4(0u, 0u, 0u, 0u);
+          }
         }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < PF; ++q) {
           const int pi = pb + q;
+          if (pi >= total) break;
           const int t = pi / cpr, ch = pi - t * cpr;
           const int v = tid + 256 * ch;
           float ps = sum8_bf16(xb[q]);
           ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
           ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
-          if (pi < total && v < vec_per_row) {
+          if (v < vec_per_row) {
             *(uint4 *)(xs + (size_t)t * XS + (size_t)v * 16) = xb[q];
             if ((tid & 15) == 0) xsum[t * G + (v >> 4)] = ps;
           }
         }
       }
     }
-    for (int i = tid + 512; i < n_sc; i += 256) ((u32 *)s_sc)[i] = bload4(rs, i * 4, 0);
-    for (int i = tid + 256; i < n_zz; i += 256) ((u32 *)s_zz)[i] = bload4(rz, i * 4, 0);
+    for (int i = tid + 512; i < n_sc; i += 256)
+      ((float4 *)s_f)[i] = scale_zero_pair(bload4(rs, i * 4, 0), bload4(rz, zoff + (i >> 8) * 256, 0) >> zsh);
     __syncthreads();
 
-    f32x4_t accA = {0.f, 0.f, 0.f, 0.f}, accB = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int tok = r < mc ? r : mc - 1;  // lanes past the last token repeat it (ignored later)
     const unsigned char *xrow = xs + (size_t)tok * XS + qd * 64;
 
@@ -1357,72 +1376,73 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
           const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
-          wa[j] = bload16(rq, lane * 16, g * 1024);
-          wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+#pragma unroll
+          for (int n = 0; n < NB; ++n) wt[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
         }
       }
 #pragma unroll
       for (int j = 0; j < CH; ++j) {
-        const bool valid = jc + j < GPW;
-        const int g = valid ? w + 4 * (jc + j) : 0;
-        const uint4 *xp = (const uint4 *)(xrow + g * 256);
-        const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
-        const float xg = xsum[tok * G + g];
-        // scales / zeros of the 4 rows this lane owns in D: rows 4qd..4qd+3
-        const uint2 sA = *(const uint2 *)(s_sc + g * 16 + 4 * qd);
-        const uint2 sB = *(const uint2 *)(s_sc + (G + g) * 16 + 4 * qd);
-        const u32 zA = *(const uint16_t *)(s_zz + g * 8 + 2 * qd);
-        const u32 zB = *(const uint16_t *)(s_zz + (G + g) * 8 + 2 * qd);
-        f32x4_t dA = {0.f, 0.f, 0.f, 0.f}, dB = {0.f, 0.f, 0.f, 0.f};
-        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].x), as_bf16x8(x0), dA, 0, 0, 0);
-        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].x), as_bf16x8(x0), dB, 0, 0, 0);
-        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].y), as_bf16x8(x1), dA, 0, 0, 0);
-        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].y), as_bf16x8(x1), dB, 0, 0, 0);
-        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].z), as_bf16x8(x2), dA, 0, 0, 0);
-        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].z), as_bf16x8(x2), dB, 0, 0, 0);
-        dA = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wa[j].w), as_bf16x8(x3), dA, 0, 0, 0);
-        dB = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wb[j].w), as_bf16x8(x3), dB, 0, 0, 0);
-        const float vs = valid ? 1.f : 0.f;  // a clamped (duplicate) tile contributes nothing
-        const u32 sAw[2] = {sA.x, sA.y}, sBw[2] = {sB.x, sB.y};
+        if (jc + j < GPW) {  // (uniform: a partial last chunk holds a clamped, duplicate tile)
+          const int g = w + 4 * (jc + j);
+          const uint4 *xp = (const uint4 *)(xrow + g * 256);
+          const bf16x8_t x0 = as_bf16x8(xp[0]), x1 = as_bf16x8(xp[1]), x2 = as_bf16x8(xp[2]), x3 = as_bf16x8(xp[3]);
+          const float xg = xsum[tok * G + g];
+          f32x4_t d[NB];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float fsa = vs * half_bits_to_f32((uint16_t)(sAw[i >> 1] >> (16 * (i & 1))));
-          const float fsb = vs * half_bits_to_f32((uint16_t)(sBw[i >> 1] >> (16 * (i & 1))));
-          const float fza = 128.f + (float)((zA >> (4 * i)) & 15);
-          const float fzb = 128.f + (float)((zB >> (4 * i)) & 15);
-          accA[i] = fmaf(fsa, dA[i] - fza * xg, accA[i]);
-          accB[i] = fmaf(fsb, dB[i] - fzb * xg, accB[i]);
+          for (int n = 0; n < NB; ++n) d[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].x), x0, d[n], 0, 0, 0);
+#pragma unroll
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].y), x1, d[n], 0, 0, 0);
+#pragma unroll
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].z), x2, d[n], 0, 0, 0);
+#pragma unroll
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].w), x3, d[n], 0, 0, 0);
+#pragma unroll
+          for (int n = 0; n < NB; ++n) {
+            // (s, -s (128 + z)) of the 4 rows this lane owns in D: rows 4qd..4qd+3
+            const float4 *sf = (const float4 *)(s_f + ((n * G + g) * 16 + 4 * qd) * 2);
+            const float4 f0 = sf[0], f1 = sf[1];
+            acc[n][0] = fmaf(f0.x, d[n][0], fmaf(f0.y, xg, acc[n][0]));
+            acc[n][1] = fmaf(f0.z, d[n][1], fmaf(f0.w, xg, acc[n][1]));
+            acc[n][2] = fmaf(f1.x, d[n][2], fmaf(f1.y, xg, acc[n][2]));
+            acc[n][3] = fmaf(f1.z, d[n][3], fmaf(f1.w, xg, acc[n][3]));
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // cross-wave reduction: red[w][ab][row][tok]
+    // cross-wave reduction: red[w][block][row][tok]
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      red[((w * 2 + 0) * 16 + 4 * qd + i) * 16 + r] = accA[i];
-      red[((w * 2 + 1) * 16 + 4 * qd + i) * 16 + r] = accB[i];
-    }
+    for (int n = 0; n < NB; ++n)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[((w * NB + n) * 16 + 4 * qd + i) * 16 + r] = acc[n][i];
     __syncthreads();
     {
       const int row = tid >> 4, t = tid & 15;  // 256 threads = 16 rows x 16 tokens
-      float va = 0.f, vb = 0.f;
+      float v[NB];
 #pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
-        va += red[((ww * 2 + 0) * 16 + row) * 16 + t];
-        vb += red[((ww * 2 + 1) * 16 + row) * 16 + t];
+      for (int n = 0; n < NB; ++n) {
+        v[n] = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < 4; ++ww) v[n] += red[((ww * NB + n) * 16 + row) * 16 + t];
       }
       if (t < mc) {
-        if (SWIGLU) {
-          const float hv = va / (1.f + expf(-va)) * vb;
-          ((uint16_t *)c.out)[(size_t)(row_first + t) * c.out_stride + b * 16 + row] = f32_to_bf16(hv);
-        } else {
-          float *o = (float *)c.out + (size_t)(row_first + t) * c.out_stride + 2 * b * 16 + row;
-          o[0] = va;
-          o[16] = vb;
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+          const float va = v[2 * q], vb = v[2 * q + 1];
+          if (SWIGLU) {
+            const float hv = va / (1.f + expf(-va)) * vb;
+            ((uint16_t *)c.out)[(size_t)(row_first + t) * c.out_stride + (b + q) * 16 + row] = f32_to_bf16(hv);
+          } else {
+            float *o = (float *)c.out + (size_t)(row_first + t) * c.out_stride + 2 * (b + q) * 16 + row;
+            o[0] = va;
+            o[16] = vb;
+          }
         }
       }
     }
-    if (pp + 1 < RPW) __syncthreads();
+    if (pp + NP < RPW) __syncthreads();
    }
     if (t0 + TB < m) __syncthreads();
   }
@@ -1641,22 +1661,30 @@ static int launch_gemv_q4k(const GemvArgs &a, int grid, int T, int Kmax, hipStre
   }
 }
 
-static size_t gemv_mfma_lds(int tb, int K) {
+// nb: 16-row blocks per iteration (2, or 4 in the 16-token form)
+static size_t gemv_mfma_lds(int tb, int K, int nb) {
   const size_t G = K / 128;
-  return (size_t)tb * (K * 2 + 16) + (((size_t)tb * G + 3) & ~(size_t)3) * 4 + 2 * G * 32 + 2 * G * 8 +
-         (size_t)4 * 2 * 256 * 4;
+  return (size_t)tb * (K * 2 + 16) + (((size_t)tb * G + 3) & ~(size_t)3) * 4 + nb * G * 128 +
+         (size_t)4 * nb * 256 * 4;
 }
 
 template <bool SW, int CH>
 static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t lds, hipStream_t s) {
-  // block pairs per workgroup: enough workgroups to fill the chip twice, then fewer, larger ones
   GemvArgs a = a_in;
+  const int units = a.cls[1].nblk > 0 ? (grid_in - a.n_sh_blocks) / a.cls[1].nblk : 0;
+  // routed block pairs per workgroup: enough workgroups to fill the chip twice, then fewer, larger ones
   int rpw = 1;
-  while (rpw < 4 && grid_in / (rpw * 2) >= 1024 && a.cls[1].nblk % (rpw * 2) == 0 &&
-         (a.n_sh_blocks == 0 || (a.cls[0].nblk % (rpw * 2) == 0)))
-    rpw *= 2;
-  a.cls[0].nblk /= rpw; a.cls[1].nblk /= rpw; a.n_sh_blocks /= rpw;
-  const int grid = grid_in / rpw;
+  while (rpw < 4 && units * a.cls[1].nblk / (rpw * 2) >= 1024 && a.cls[1].nblk % (rpw * 2) == 0) rpw *= 2;
+  // the shared expert's workgroups stage every token row.  With a reduction longer than the routed
+  // experts' (w2 of a wide shared expert) they are the long ones of the launch and keep one pair each:
+  // four pairs each cost the 16-token step of a 2048 x 2816 shared expert about 8 us.  Otherwise they
+  // take what the routed ones take (more, smaller workgroups only add staging traffic).
+  int rpw_s = 1;
+  if (a.n_sh_blocks > 0 && a.cls[0].K <= a.cls[1].K)
+    while (rpw_s < rpw && a.cls[0].nblk % (rpw_s * 2) == 0) rpw_s *= 2;
+  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= rpw_s; a.n_sh_blocks /= rpw_s; }
+  a.cls[1].nblk /= rpw;
+  const int grid = a.n_sh_blocks + units * a.cls[1].nblk;
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma<SW, CH, true>,
@@ -1671,8 +1699,8 @@ static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t ld
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, true>), dim3(grid), dim3(256), lds, s, a, tb, rpw);
-  else hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, false>), dim3(grid), dim3(256), lds, s, a, tb, rpw);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, true>), dim3(grid), dim3(256), lds, s, a, tb, rpw, rpw_s);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma<SW, CH, false>), dim3(grid), dim3(256), lds, s, a, tb, rpw, rpw_s);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4_mfma");
 }
@@ -1698,8 +1726,11 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
   if (mode == 2 || (mode == 0 && T > 1)) {
     int tb = 1;
     while (tb < T && tb < 16) tb <<= 1;
-    while (tb > 1 && gemv_mfma_lds(tb, Kmax) > 150 * 1024) tb >>= 1;
-    const size_t lds = gemv_mfma_lds(tb, Kmax);
+    while (tb > 1 && gemv_mfma_lds(tb, Kmax, 2) > 150 * 1024) tb >>= 1;
+    // sixteen token rows that leave room for one workgroup per CU only: eight rows and two workgroups
+    // are faster when that fits (units with more than eight tokens take a second pass)
+    if (tb == 16 && gemv_mfma_lds(16, Kmax, 2) > 80 * 1024 && gemv_mfma_lds(8, Kmax, 2) <= 80 * 1024) tb = 8;
+    const size_t lds = gemv_mfma_lds(tb, Kmax, 2);
     if (lds > 150 * 1024) { moe_set_error("k_gemv_int4_mfma: K=%d does not fit LDS", Kmax); return MOE_EINVAL; }
     switch (ch) {
       case 1: return launch_gemv_mfma<SW, 1>(a, grid, tb, lds, s);
