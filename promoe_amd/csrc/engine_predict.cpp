@@ -29,7 +29,13 @@ struct PredictorState {
   std::vector<std::pair<int, int>> window;          // [L + 1]: destination layers [first, second) of source l
   std::map<std::pair<int, int>, PredictModel> models;
   int max_win = 0, H = 0;
-  float *scores_dev = nullptr, *scores_host = nullptr;  // [L + 1][max_win][E]
+  // [L + 1][max_win][E].  Device backend: pinned host memory; the score kernel stores into it through
+  // scores_dev, its device-side address (no copy in the stream), the thread reads it after the event
+  float *scores_dev = nullptr, *scores_host = nullptr;
+  // device backend: the models of one source layer stacked into one [n_dst * E, H] matrix (and bias
+  // vector, if any of them has one), so that a report costs one launch whatever the window
+  std::vector<void *> stack_w;
+  std::vector<float *> stack_b;
   std::vector<void *> events;                            // one per source layer
   std::thread th;
   std::mutex mu;
@@ -189,10 +195,35 @@ extern "C" int moe_predictor_start(moe_engine *eng) {
   if (p->host_math) {
     p->scores_host = new float[n]();
   } else {
-    if (moe_check_hip(hipMalloc((void **)&p->scores_dev, n * sizeof(float)), "hipMalloc(predictor scores)")) return MOE_EHIP;
     if (moe_check_hip(hipHostMalloc((void **)&p->scores_host, n * sizeof(float), hipHostMallocDefault), "hipHostMalloc(predictor scores)"))
       return MOE_EHIP;
+    if (moe_check_hip(hipHostGetDevicePointer((void **)&p->scores_dev, p->scores_host, 0), "hipHostGetDevicePointer(predictor scores)"))
+      return MOE_EHIP;
     for (int l = 0; l <= L; ++l) p->events.push_back(eng->be->event_create());
+    p->stack_w.assign(L + 1, nullptr);
+    p->stack_b.assign(L + 1, nullptr);
+    const size_t wb = (size_t)E * p->H * 2;
+    for (int src = 0; src <= L; ++src) {
+      const auto win = p->window[src];
+      const int nd = win.second - win.first;
+      if (nd <= 0) continue;
+      bool any_bias = false;
+      for (int dst = win.first; dst < win.second; ++dst) any_bias |= p->models[{src, dst}].bias != nullptr;
+      if (moe_check_hip(hipMalloc(&p->stack_w[src], wb * nd), "hipMalloc(predictor models)")) return MOE_EHIP;
+      if (any_bias) {
+        if (moe_check_hip(hipMalloc((void **)&p->stack_b[src], (size_t)nd * E * sizeof(float)), "hipMalloc(predictor bias)")) return MOE_EHIP;
+        if (moe_check_hip(hipMemset(p->stack_b[src], 0, (size_t)nd * E * sizeof(float)), "hipMemset(predictor bias)")) return MOE_EHIP;
+      }
+      for (int dst = win.first; dst < win.second; ++dst) {
+        const PredictModel &m = p->models[{src, dst}];
+        const size_t i = (size_t)(dst - win.first);
+        if (moe_check_hip(hipMemcpy((char *)p->stack_w[src] + i * wb, m.w, wb, hipMemcpyDeviceToDevice), "hipMemcpy(predictor model)"))
+          return MOE_EHIP;
+        if (m.bias && moe_check_hip(hipMemcpy(p->stack_b[src] + i * E, m.bias, (size_t)E * sizeof(float), hipMemcpyDeviceToDevice),
+                                    "hipMemcpy(predictor bias)"))
+          return MOE_EHIP;
+      }
+    }
   }
   p->started = true;
   p->th = std::thread(predictor_loop, eng, p);
@@ -211,19 +242,18 @@ int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int 
   if (decode) {
     if (!hidden || H != p->H) { moe_set_error("predictor: layer %d reported a hidden state of width %d, the models take %d", layer, H, p->H); return MOE_EINVAL; }
     const int E = eng->cfg.num_expert;
-    for (int dst = win.first; dst < win.second; ++dst) {
-      const PredictModel &m = p->models[{layer, dst}];
-      const size_t off = ((size_t)layer * p->max_win + (dst - win.first)) * E;
-      if (p->host_math) {
+    if (p->host_math) {
+      for (int dst = win.first; dst < win.second; ++dst) {
+        const PredictModel &m = p->models[{layer, dst}];
+        const size_t off = ((size_t)layer * p->max_win + (dst - win.first)) * E;
         host_scores((const uint16_t *)hidden, (const uint16_t *)m.w, m.bias, p->scores_host + off, H, E);
-      } else if (int rc = moe_gate_logits(hidden, m.w, m.bias, p->scores_dev + off, 1, H, E, E, eng->be->compute_stream())) {
-        return rc;
       }
-    }
-    if (!p->host_math) {
-      const size_t off = (size_t)layer * p->max_win * E, nb = (size_t)(win.second - win.first) * E * sizeof(float);
-      if (int rc = moe_check_hip(hipMemcpyAsync(p->scores_host + off, p->scores_dev + off, nb, hipMemcpyDeviceToHost,
-                                                (hipStream_t)eng->be->compute_stream()), "hipMemcpyAsync(predictor scores)"))
+    } else {
+      // one launch for the whole window: the stacked models' rows are the window's (dst, expert) pairs in order
+      const size_t off = (size_t)layer * p->max_win * E;
+      const int rows = (win.second - win.first) * E;
+      if (int rc = moe_gate_logits(hidden, p->stack_w[layer], p->stack_b[layer], p->scores_dev + off, 1, H, rows, rows,
+                                   eng->be->compute_stream()))
         return rc;
       if (eng->be->event_record(p->events[layer], eng->be->compute_stream()) != 0) return MOE_EHIP;
     }
@@ -256,7 +286,8 @@ void moe_predictor_free(moe_engine *eng) {
   if (p->th.joinable()) p->th.join();
   if (p->host_math) delete[] p->scores_host;
   else {
-    if (p->scores_dev) (void)hipFree(p->scores_dev);
+    for (void *w : p->stack_w) if (w) (void)hipFree(w);
+    for (float *b : p->stack_b) if (b) (void)hipFree(b);
     if (p->scores_host) (void)hipHostFree(p->scores_host);
   }
   delete p;
