@@ -152,8 +152,9 @@ int moe_update_priority(moe_engine *eng, const float *p, int n_layers, int start
  * requests.  Starting the predictor attaches it (see moe_attach_predictor). ---- */
 /* first[l], last[l] for l = 0..L: destination layers [first, last) of source layer l */
 int moe_predictor_windows(moe_engine *eng, int *first, int *last);
-/* model of one pair: w bf16 [num_expert, H] and bias fp32 [num_expert] or NULL, device memory the caller
- * keeps alive (host memory on the host backend); dst must lie in the window of src */
+/* model of one pair: w bf16 [num_expert, H] and bias fp32 [num_expert] or NULL, device memory (host memory on
+ * the host backend) that stays valid until moe_predictor_start, which copies the models of a source layer
+ * into one matrix (the host backend keeps reading the caller's memory); dst must lie in the window of src */
 int moe_predictor_set_model(moe_engine *eng, int src, int dst, const void *w, const float *bias, int H);
 /* after moe_launch: needs a model for every pair of every window, and every layer covered once */
 int moe_predictor_start(moe_engine *eng);
