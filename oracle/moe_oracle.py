@@ -24,7 +24,9 @@ Pinning status (what fixes each function, beyond re-typing a formula)
 * dispatch: == numpy stable argsort; bijection/count invariants; brute force.
 * int4 g128: pack->unpack round trip, closed form w=(q-z)*s, hand-built blocks.
 * q4_K: hand-built known-answer super-blocks (all-zero, single nibble, max scale).
-* swiglu_expert / moe_forward: reduce to torch F.linear/F.silu in fp32.
+* swiglu_expert / moe_forward: reduce to torch F.linear/F.silu in fp32; the whole
+  layer is checked against stock transformers' Qwen2-MoE, Mixtral and DeepSeek-V2
+  sparse blocks run in fp32 (tests/test_oracle_vs_transformers.py).
 * The exact bf16<->fp32 cast order of the external patched module is NOT pinned
   by anything in the reference ("parity unpinned" for that detail); it is covered
   by the 2e-2 output tolerance against this fp32 path.
