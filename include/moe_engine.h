@@ -159,6 +159,10 @@ int moe_predictor_set_model(moe_engine *eng, int src, int dst, const void *w, co
 /* after moe_launch: needs a model for every pair of every window, and every layer covered once */
 int moe_predictor_start(moe_engine *eng);
 int moe_predictor_stats(moe_engine *eng, uint64_t *n_jobs, uint64_t *n_requests);
+/* waits until the predictor thread has worked off every report so far (its counters lag the hooks by a
+ * moment); 0 = idle, 1 = still busy after timeout_ms (it may be waiting for the run-ahead budget, which only
+ * further layers release).  No counterpart in the reference, whose worker is joined at exit only. */
+int moe_predictor_wait_idle(moe_engine *eng, int timeout_ms);
 
 /* ---- Belady policy hooks: CacheOracle / set_cur_seq (adapter.cpp:62-70, cache.cpp:592-644) ---- */
 int moe_oracle_load(moe_engine *eng, const int64_t *entry_metas, int64_t n_entries,

@@ -39,7 +39,8 @@ struct PredictorState {
   std::vector<void *> events;                            // one per source layer
   std::thread th;
   std::mutex mu;
-  std::condition_variable cv;
+  std::condition_variable cv, cv_idle;
+  bool busy = false;                                     // a job is being processed
   std::deque<PredictJob> q;
   bool exit = false, started = false, host_math = false;
   uint64_t n_jobs = 0, n_requests = 0;
@@ -127,6 +128,7 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
       if (p->exit) return;
       job = p->q.front();
       p->q.pop_front();
+      p->busy = true;
     }
     const auto win = p->window[job.src];
     bool decode = job.seq_len == 1;
@@ -172,6 +174,8 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
     }
     std::lock_guard<std::mutex> lk(p->mu);
     p->n_jobs++;
+    p->busy = false;
+    p->cv_idle.notify_all();
   }
 }
 
@@ -265,6 +269,15 @@ int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int 
   }
   p->cv.notify_all();
   return MOE_OK;
+}
+
+extern "C" int moe_predictor_wait_idle(moe_engine *eng, int timeout_ms) {
+  if (!eng || !eng->pred) { moe_set_error("moe_predictor_wait_idle: no predictor"); return MOE_ESTATE; }
+  PredictorState *p = eng->pred;
+  std::unique_lock<std::mutex> lk(p->mu);
+  const bool idle = p->cv_idle.wait_for(lk, std::chrono::milliseconds(timeout_ms < 0 ? 0 : timeout_ms),
+                                        [&] { return p->exit || (p->q.empty() && !p->busy); });
+  return idle ? MOE_OK : 1;
 }
 
 extern "C" int moe_predictor_stats(moe_engine *eng, uint64_t *n_jobs, uint64_t *n_requests) {

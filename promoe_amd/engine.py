@@ -222,7 +222,9 @@ class PrefetchMngr:
     def start_predictor(self):
         check(lib.moe_predictor_start(self._h), "start_predictor")
 
-    def predictor_stats(self) -> dict:
+    def predictor_stats(self, settle_ms: int = 2000) -> dict:
+        """Counters of the predictor thread, read once it has worked off the reports so far (or after settle_ms)."""
+        lib.moe_predictor_wait_idle(self._h, settle_ms)
         a, b = C.c_uint64(), C.c_uint64()
         check(lib.moe_predictor_stats(self._h, C.byref(a), C.byref(b)), "predictor_stats")
         return {"jobs": a.value, "requests": b.value}
