@@ -170,7 +170,8 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
     q4k = fmt == L.FMT_Q4K
     mk = synth.random_q4k_images if q4k else synth.random_int4_images
     lay = LY.q4k_layout if q4k else LY.int4_layout
-    if T > 16:   # the rule of moe_forward: token groups above 16 rows take the matrix-core kernels
+    tiles = T > ops.gemv_max_tokens(fmt)   # the rule of moe_forward: larger token groups take the matrix-core tile kernels
+    if tiles:
         def run_experts(x, d_, table, sh, H_, I_, I_sh_, phases=3, ws=None):
             return ops.experts_prefill(x, d_, table, sh, H_, I_, I_sh_, fmt, phases=phases, ws=ws)
     else:
@@ -234,8 +235,8 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
     return {"workload": name, "tokens": T, "layers_in_rotation": layers, "tokens_per_s": T / t_layer,
             "us_per_layer": t_layer * 1e6, "distinct_routed_experts_per_step": D,
             "algorithmic_bytes_per_step": step_bytes, "layer_GBps": step_bytes / t_layer / 1e9,
-            "roofline": {"bound": "hbm", "kernel": ("k_prefill_int4 (w13 + SwiGLU)" if T > 16 else
-                                                    "k_gemv_int4%s (w13 + SwiGLU)" % ("<q4_K>" if q4k else ("_mfma" if T > 1 else ""))),
+            "roofline": {"bound": "hbm", "kernel": ("k_prefill_int4 (w13 + SwiGLU)" if tiles else
+                                                    "k_gemv_int4%s (w13 + SwiGLU)" % ("<q4_K>" if q4k else ("_mfma_kc" if (T > 16 or H > 2048) and T > 1 else ("_mfma" if T > 1 else "")))),
                          "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
                          "algorithmic_bytes_per_launch": w13_bytes, "avg_launch_us": t_w13 * 1e6,
                          "method": "%d back-to-back launches between one HIP event pair" % steps}}
@@ -293,7 +294,7 @@ def main():
           (L_, E, stack.expert_bytes * L_ * E / 1e9, time.perf_counter() - t_setup), file=sys.stderr, flush=True)
 
     # ---- steady-state hits: every expert resident -------------------------------------
-    pm = stack.engine(16, cache_rate=1.0, cache_policy="lru")
+    pm = stack.engine(max(16, T), cache_rate=1.0, cache_policy="lru")
     import numpy as np
     for l in range(L_):                      # bring every expert into its slot
         pm.acquire_layer(l, np.arange(E, dtype=np.int64))

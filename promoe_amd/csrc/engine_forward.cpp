@@ -188,10 +188,14 @@ int moe_forward_harvest(moe_engine *eng, bool wait) {
 }
 
 // Expert product of one launch group.  Token groups of prefill size (and every bf16 layer)
-// go to the matrix-core kernels, decode batches to the bandwidth-bound GEMV kernels.
+// go to the matrix-core tile kernels, decode batches to the bandwidth-bound GEMV kernels.
 static bool use_prefill(const moe_layer_desc &d, int T) {
   if (d.fmt == MOE_FMT_BF16) return true;
-  return T > 16 && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
+  // int4-g128: up to 64 tokens the grouped launch is bound by the weight stream and the GEMV kernels
+  // (operand 128 + q, scale and zero applied after the products) stream it faster than the tile kernels,
+  // which dequantise every weight completely (measured on the 2048 x 1408 and 4096 x 14336 shapes)
+  const int gemv_tmax = d.fmt == MOE_FMT_INT4_G128 ? 64 : 16;
+  return T > gemv_tmax && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
 }
 
 static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
@@ -388,7 +392,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
   bool routed_by_tail = false;
   int tail_seq = 0;
-  if (all_resident && fused_route && T <= 16 && E <= 256 && T * k <= 512) {
+  if (all_resident && fused_route && T <= 32 && E <= 256 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory
     if (!d.gate_bias) {

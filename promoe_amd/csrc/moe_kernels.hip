@@ -365,7 +365,7 @@ __global__ __launch_bounds__(DISP_THREADS) void k_dispatch(
 // stable dispatch on its own.  Three launches become one, and the logits are still spread
 // over as many workgroups as before.  The counter must be zero at launch and is left zero.
 // ---------------------------------------------------------------------------
-#define ROUTE_MAXT 16
+#define ROUTE_MAXT 64
 #define ROUTE_MAXP 512
 struct RouteArgs {
   const uint16_t *x, *wg;
@@ -1449,6 +1449,212 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 }
 
 // ---------------------------------------------------------------------------
+// k3, matrix-core form for long reductions and for up to 32 rows per pass.  Same tiles, same
+// products and the same scale/zero correction as k_gemv_int4_mfma, different work split:
+//   * a wave owns one block pair (gate/up blocks, or two row blocks) over the whole reduction, so
+//     there is no cross-wave reduction; a workgroup = four adjacent pairs of one unit;
+//   * the activations are staged CG groups (CG x 128 columns) at a time, double-buffered, one
+//     barrier per chunk, so the LDS footprint does not grow with K (two workgroups per CU at any K);
+//   * the weight tiles of the next four groups and the activations and scales of the next chunk
+//     are in flight while the current ones are worked on;
+//   * NT = 2: two 16-token column blocks per pass share every dequantised weight tile.
+// ---------------------------------------------------------------------------
+template <bool SWIGLU, bool DEVUNITS, int NT, int CG>
+__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
+  constexpr int NB = 2, WS = 4;        // 16-row blocks per wave, groups per weight step
+  constexpr int TBK = 16 * NT;         // token rows per pass
+  constexpr int XSC = CG * 256 + 16;   // padded row stride of a staged chunk (bytes)
+  constexpr int XV = CG * 16;          // 16-byte vectors per row and chunk
+  constexpr int NPC = TBK * XV / 256;  // vectors per thread and chunk
+  constexpr int NSD = NB * CG * 8 / 64;  // scale dwords (two rows each) per lane and chunk
+  constexpr int SPC = CG / WS;         // weight steps per chunk
+  static_assert(CG % WS == 0 && (SPC == 1 || SPC == 2) && NPC >= 1 && NSD >= 1, "chunk shape");
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, qd = lane >> 4;
+
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  const GemvClass &c = wk.c;
+  const int m = wk.m, row0 = wk.row0;
+  const unsigned char *base = wk.base;
+  if (m <= 0) return;
+  if (base == nullptr) {
+    if (tid == 0) atomicOr(a.err, 1);
+    return;
+  }
+  const int K = c.K, G = c.G;
+  unsigned char *xs = smem;                                   // [2][TBK][XSC]
+  float *xsum = (float *)(smem + (size_t)2 * TBK * XSC);      // [2][TBK][CG]
+  float *sfw = xsum + 2 * TBK * CG + w * (NB * CG * 32);      // this wave's [NB][CG][16 rows][2]
+
+  const int b = wk.b * 4 + w;  // the wave's block pair
+  const int rbA = 2 * b;
+  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
+  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
+  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
+  const int NCH = (G + CG - 1) / CG;  // activation chunks
+  const int NS = (G + WS - 1) / WS;   // weight steps
+
+  for (int t0 = 0; t0 < m; t0 += TBK) {
+    const int mc = (m - t0) < TBK ? (m - t0) : TBK;
+    const int row_first = row0 + t0;
+    // byte offset of the activation row behind each of this thread's vectors (rows past the
+    // last token repeat it; they are staged but never read)
+    int xoff[NPC];
+#pragma unroll
+    for (int i = 0; i < NPC; ++i) {
+      const int row = (tid + 256 * i) / XV;
+      const int gr = row_first + (row < mc ? row : mc - 1);
+      xoff[i] = (c.gather ? c.gather[gr] : gr) * c.act_stride * 2;
+    }
+    uint4 xr[NPC];
+    u32 scr[NSD], zr[NSD];
+    // loads of one chunk: activations, scale dwords and the zero dwords that hold their nibbles
+    // (groups past the end of the reduction: zero activations, zero scales)
+    auto load_chunk = [&](const int ch) {
+#pragma unroll
+      for (int i = 0; i < NPC; ++i) {
+        const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
+        const bool in = kv * 8 < K;
+        const uint4 v = bload16(rx, xoff[i] + (in ? kv * 16 : 0), 0);
+        xr[i] = in ? v : make_uint4(0u, 0u, 0u, 0u);
+      }
+#pragma unroll
+      for (int i = 0; i < NSD; ++i) {
+        const int e = lane + 64 * i;
+        const int n = e / (CG * 8), g = ch * CG + ((e % (CG * 8)) >> 3), j = e & 7;
+        const bool ok = g < G;
+        scr[i] = bload4(rs, ok ? ((n * G + g) * 8 + j) * 4 : 0x7ffffff0, 0);
+        zr[i] = bload4(rz, ok ? (n * G + g) * 8 + (j >> 2) * 4 : 0x7ffffff0, 0);
+      }
+    };
+    auto load_w = [&](const int s, uint4 (&wt_)[WS][NB]) {
+#pragma unroll
+      for (int j = 0; j < WS; ++j) {
+        const int g = s * WS + j < G ? s * WS + j : G - 1;
+#pragma unroll
+        for (int n = 0; n < NB; ++n) wt_[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
+      }
+    };
+    f32x4_t acc[NB][NT];
+#pragma unroll
+    for (int n = 0; n < NB; ++n)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[n][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    int tokl[NT];  // lanes past the last token repeat it (their columns are not stored)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) tokl[t] = 16 * t + r < mc ? 16 * t + r : mc - 1;
+
+    // registers -> LDS for chunk ch, barrier, then the next chunk's loads
+    auto chunk_begin = [&](const int ch) {
+      const int cb = ch & 1;
+#pragma unroll
+      for (int i = 0; i < NPC; ++i) {
+        const int p = tid + 256 * i;
+        const int row = p / XV, v = p & (XV - 1);
+        float ps = sum8_bf16(xr[i]);
+        ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
+        ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
+        *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xr[i];
+        if ((tid & 15) == 0) xsum[(cb * TBK + row) * CG + (v >> 4)] = ps;
+      }
+#pragma unroll
+      for (int i = 0; i < NSD; ++i) {
+        const int e = lane + 64 * i;
+        ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
+      }
+      __syncthreads();
+      if (ch + 1 < NCH) load_chunk(ch + 1);
+    };
+    // weight step s (four groups) on the tiles in cur; the next step's tiles go to nxt first
+    auto step = [&](const int s, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
+      if (s + 1 < NS) load_w(s + 1, nxt);
+      const int cb = (s / SPC) & 1;
+#pragma unroll
+      for (int j = 0; j < WS; ++j) {
+        if (s * WS + j < G) {  // uniform
+          const int gq = (s % SPC) * WS + j;
+          bf16x8_t xv[NT][4];
+          float xg[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const uint4 *xp = (const uint4 *)(xs + ((size_t)cb * TBK + tokl[t]) * XSC + gq * 256 + qd * 64);
+            xv[t][0] = as_bf16x8(xp[0]); xv[t][1] = as_bf16x8(xp[1]);
+            xv[t][2] = as_bf16x8(xp[2]); xv[t][3] = as_bf16x8(xp[3]);
+            xg[t] = xsum[(cb * TBK + tokl[t]) * CG + gq];
+          }
+#pragma unroll
+          for (int n = 0; n < NB; ++n) {
+            const bf16x8_t w0 = deq8_bf16(cur[j][n].x), w1 = deq8_bf16(cur[j][n].y);
+            const bf16x8_t w2 = deq8_bf16(cur[j][n].z), w3 = deq8_bf16(cur[j][n].w);
+            // (s, -s (128 + z)) of the 4 rows this lane owns in D: rows 4qd..4qd+3
+            const float4 *sf = (const float4 *)(sfw + ((n * CG + gq) * 16 + 4 * qd) * 2);
+            const float4 f0 = sf[0], f1 = sf[1];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              f32x4_t d = f32x4_t{0.f, 0.f, 0.f, 0.f};
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, xv[t][0], d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, xv[t][1], d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2, xv[t][2], d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w3, xv[t][3], d, 0, 0, 0);
+              acc[n][t][0] = fmaf(f0.x, d[0], fmaf(f0.y, xg[t], acc[n][t][0]));
+              acc[n][t][1] = fmaf(f0.z, d[1], fmaf(f0.w, xg[t], acc[n][t][1]));
+              acc[n][t][2] = fmaf(f1.x, d[2], fmaf(f1.y, xg[t], acc[n][t][2]));
+              acc[n][t][3] = fmaf(f1.z, d[3], fmaf(f1.w, xg[t], acc[n][t][3]));
+            }
+          }
+        }
+      }
+    };
+
+    uint4 wA[WS][NB], wB[WS][NB];
+    load_chunk(0);
+    load_w(0, wA);
+    if constexpr (SPC == 2) {
+      for (int ch = 0; ch < NCH; ++ch) {
+        chunk_begin(ch);
+        step(2 * ch, wA, wB);
+        if (2 * ch + 1 < NS) step(2 * ch + 1, wB, wA);
+      }
+    } else {
+      for (int ch = 0; ch < NCH; ch += 2) {
+        chunk_begin(ch);
+        step(ch, wA, wB);
+        if (ch + 1 < NCH) {
+          chunk_begin(ch + 1);
+          step(ch + 1, wB, wA);
+        }
+      }
+    }
+    // every lane holds 4 consecutive rows of both blocks for one token per column block
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (16 * t + r < mc) {
+        const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
+        if (SWIGLU) {
+          u32 h[2];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
+            const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
+            const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
+            h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
+          }
+          *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
+        } else {
+#pragma unroll
+          for (int n = 0; n < NB; ++n)
+            *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
+                make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
+        }
+      }
+    }
+    if (t0 + TBK < m) __syncthreads();  // the next pass restages chunk buffer 0
+  }
+}
+
+// ---------------------------------------------------------------------------
 // k5 combine
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_r,
@@ -1523,7 +1729,9 @@ extern "C" int moe_gate_logits(const void *x, const void *wg, const float *bias,
   }
   if (T == 0) return MOE_OK;
   const size_t tile_lds = (size_t)GATE_TT * H * 2;
-  if (T > 16 && H <= 4096 && tile_lds <= 150 * 1024) {
+  // up to 128 tokens a wave per (token, gate row) is faster than the token-tile kernel (8 us against 18 us
+  // at 128 tokens, 2048 columns, 64 rows)
+  if (T > 128 && H <= 4096 && tile_lds <= 150 * 1024) {
     static bool attr_set = false;
     if (tile_lds > 64 * 1024 && !attr_set) {
       if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gate_logits_tile,
@@ -1705,6 +1913,44 @@ static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t ld
   return moe_check_launch("k_gemv_int4_mfma");
 }
 
+static size_t gemv_mfma_kc_lds(int nt, int cg) {
+  return (size_t)2 * 16 * nt * (cg * 256 + 16) + (size_t)2 * 16 * nt * cg * 4 + (size_t)4 * 2 * cg * 32 * 4;
+}
+
+// chunked-K form: a workgroup takes four block pairs of a unit (both classes' pair counts are
+// multiples of four: I and H are multiples of 128)
+template <bool SW, int NT, int CG>
+static int launch_gemv_mfma_kc(const GemvArgs &a_in, int grid_in, hipStream_t s) {
+  GemvArgs a = a_in;
+  const int units = a.cls[1].nblk > 0 ? (grid_in - a.n_sh_blocks) / a.cls[1].nblk : 0;
+  if ((a.n_sh_blocks > 0 && a.cls[0].nblk % 4) || (units > 0 && a.cls[1].nblk % 4)) {
+    moe_set_error("k_gemv_int4_mfma_kc: block pairs per unit not a multiple of 4");
+    return MOE_EINVAL;
+  }
+  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= 4; a.n_sh_blocks /= 4; }
+  a.cls[1].nblk /= 4;
+  const int grid = a.n_sh_blocks + units * a.cls[1].nblk;
+  const size_t lds = gemv_mfma_kc_lds(NT, CG);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NT, CG>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NT, CG>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
+      return MOE_EHIP;
+    }
+    attr_set = true;
+  }
+  moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NT, CG>), dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NT, CG>), dim3(grid), dim3(256), lds, s, a);
+  moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
+  return moe_check_launch("k_gemv_int4_mfma_kc");
+}
+
 // 0: dot2 GEMV for T == 1, matrix-core form otherwise (default); 1: always dot2; 2: always MFMA
 static int gemv_mode() {
   static int mode = -1;
@@ -1724,6 +1970,13 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
   if (ch < 1) ch = 1;
   const int mode = gemv_mode();
   if (mode == 2 || (mode == 0 && T > 1)) {
+    // chunked-K form: reductions too long for two workgroups per CU with the whole rows staged, and
+    // batches of more than 16 tokens (measured on the 4096 x 14336 and 2048 x 1408 shapes: the w2 pass
+    // gains from 32-token passes above 32 tokens, the w13 pass does not)
+    if (Kmax > 2048 || T > 16) {
+      if (!SW && T > 32) return launch_gemv_mfma_kc<SW, 2, 4>(a, grid, s);
+      return launch_gemv_mfma_kc<SW, 1, 8>(a, grid, s);
+    }
     int tb = 1;
     while (tb < T && tb < 16) tb <<= 1;
     while (tb > 1 && gemv_mfma_lds(tb, Kmax, 2) > 150 * 1024) tb >>= 1;

@@ -99,7 +99,7 @@ class SparseMoeBlock:
         one.__dict__.update(d.__dict__)
         one.units, one.max_units = unit_row, unit_row.shape[0]
         sh = self.shared if with_shared else None
-        if self.fmt == L.FMT_BF16 or x.shape[0] > 16:
+        if self.fmt == L.FMT_BF16 or x.shape[0] > ops.gemv_max_tokens(self.fmt):
             return ops.experts_prefill(x, one, table, sh, self.H, self.I, self.I_sh, self.fmt, ws=ws)
         return ops.experts_decode_int4(x, one, table, sh, self.H, self.I, self.I_sh,
                                        ws=None if ws is None else ws[:5]) + (None,)

@@ -11,6 +11,12 @@ from . import _lib as L
 from ._lib import lib, ptr, cur_stream, check
 
 
+def gemv_max_tokens(fmt: int) -> int:
+    """Largest token group moe_forward sends to the GEMV kernels; larger ones (and every bf16 layer) take
+    the matrix-core tile kernels."""
+    return 64 if fmt == L.FMT_INT4_G128 else 16
+
+
 def _dev(t):
     assert t.is_cuda and t.is_contiguous(), "expected a contiguous device tensor"
     return t

@@ -76,7 +76,7 @@ def test_hip_layer_forward_matches_fixture(cuda, kind):
         idx, w = ops.topk(logits, k, 0, E=E)
         assert np.array_equal(idx.cpu().numpy(), f["idx_T%d" % T])
         d = ops.dispatch(idx, E)
-        if kind == "bf16" or T > 16:
+        if kind == "bf16" or T > ops.gemv_max_tokens(fmt):
             part_r, part_s, err = ops.experts_prefill(x, d, table, shared, H, I, I_sh, fmt)[:3]
         elif kind == "q4k":
             part_r, part_s, err = ops.experts_decode_q4k(x, d, table, shared, H, I, I_sh)[:3]

@@ -148,7 +148,17 @@ def test_decode_layer_small_variants(cuda):
     check_layer(Int4Layer(H=384, I=640, E=4, I_sh=128, seed=6), 3, 2, 0, cuda)
 
 
-@pytest.mark.parametrize("T", [1, 4, 16])
+@pytest.mark.parametrize("T", [3, 16, 20, 40, 64])
+def test_decode_layer_long_reduction(cuda, T):
+    """Reductions longer than 2048 and batches of more than 16 tokens take the chunked-K GEMV: group counts
+    that leave a partial last chunk and an odd number of weight steps (G = 18, 17, 20), units with more rows
+    than one pass holds (E = 4, k = 2: about T / 2 rows per unit), 32-token passes in w2 above 32 tokens."""
+    print(f"case decode_long_reduction T={T}", flush=True)
+    layer = Int4Layer(H=2304, I=2176, E=4, I_sh=2560, seed=8)
+    check_layer(layer, T, 2, 0, cuda)
+
+
+@pytest.mark.parametrize("T", [1, 4, 16, 32, 64])
 def test_decode_layer_deepseek_shape(cuda, T):
     print(f"case decode_deepseek T={T}", flush=True)
     # DeepSeek-MoE-16B layer shape; 16 experts instead of 64 keeps host-side quantisation short

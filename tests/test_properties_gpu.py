@@ -18,7 +18,7 @@ def _images(kind, n, H, I, dev, gen):
 def _experts(kind, x, d, table, shared, H, I, I_sh):
     from promoe_amd import ops, _lib as L
     fmt = {"int4": L.FMT_INT4_G128, "q4k": L.FMT_Q4K, "bf16": L.FMT_BF16}[kind]
-    if kind == "bf16" or x.shape[0] > 16:
+    if kind == "bf16" or x.shape[0] > ops.gemv_max_tokens(fmt):
         return ops.experts_prefill(x, d, table, shared, H, I, I_sh, fmt)[:3]
     if kind == "q4k":
         return ops.experts_decode_q4k(x, d, table, shared, H, I, I_sh)[:3]
@@ -30,6 +30,8 @@ def _experts(kind, x, d, table, shared, H, I, I_sh):
     ("deepseek prefill", "int4", 2048, 2048, 64, 1408, 6, 2816),
     ("qwen1.5 prefill", "bf16", 2048, 2048, 60, 1408, 4, 5632),
     ("mixtral decode", "int4", 1, 4096, 8, 14336, 2, 0),
+    ("mixtral decode 64 tokens", "int4", 64, 4096, 8, 14336, 2, 0),
+    ("deepseek decode 64 tokens", "int4", 64, 2048, 64, 1408, 6, 2816),
     ("mixtral prefill", "int4", 4096, 4096, 8, 14336, 2, 0),
     ("qwen2 decode", "q4k", 3, 3584, 64, 2560, 8, 0),
     ("qwen2 prefill", "q4k", 512, 3584, 64, 2560, 8, 0),
