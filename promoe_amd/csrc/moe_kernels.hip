@@ -1451,27 +1451,34 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 // ---------------------------------------------------------------------------
 // k3, matrix-core form for long reductions and for up to 32 rows per pass.  Same tiles, same
 // products and the same scale/zero correction as k_gemv_int4_mfma, different work split:
-//   * a wave owns one block pair (gate/up blocks, or two row blocks) over the whole reduction, so
-//     there is no cross-wave reduction; a workgroup = four adjacent pairs of one unit;
+//   * KS waves own one block pair (gate/up blocks, or two row blocks) over the whole reduction; a
+//     workgroup = 4 / KS adjacent pairs of one unit.  KS = 1: no cross-wave reduction at all; KS = 2, 4
+//     (launches with few block pairs): the waves of a pair take 1 / KS of every chunk's groups and their
+//     sums meet in LDS once, at the end, in a fixed order;
 //   * the activations are staged CG groups (CG x 128 columns) at a time, double-buffered, one
 //     barrier per chunk, so the LDS footprint does not grow with K (two workgroups per CU at any K);
-//   * the weight tiles of the next four groups and the activations and scales of the next chunk
+//   * the weight tiles of the wave's next step and the activations and scales of the next chunk
 //     are in flight while the current ones are worked on;
 //   * NT = 2: two 16-token column blocks per pass share every dequantised weight tile.
 // ---------------------------------------------------------------------------
-template <bool SWIGLU, bool DEVUNITS, int NT, int CG>
+template <bool SWIGLU, bool DEVUNITS, int NT, int CG, int KS>
 __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
-  constexpr int NB = 2, WS = 4;        // 16-row blocks per wave, groups per weight step
+  constexpr int NB = 2;                // 16-row blocks per wave
+  constexpr int GW = CG / KS;          // groups per wave and chunk
+  constexpr int WS = GW < 4 ? GW : 4;  // groups per weight step
+  constexpr int SPC = GW / WS;         // weight steps per wave and chunk
   constexpr int TBK = 16 * NT;         // token rows per pass
   constexpr int XSC = CG * 256 + 16;   // padded row stride of a staged chunk (bytes)
   constexpr int XV = CG * 16;          // 16-byte vectors per row and chunk
   constexpr int NPC = TBK * XV / 256;  // vectors per thread and chunk
-  constexpr int NSD = NB * CG * 8 / 64;  // scale dwords (two rows each) per lane and chunk
-  constexpr int SPC = CG / WS;         // weight steps per chunk
-  static_assert(CG % WS == 0 && (SPC == 1 || SPC == 2) && NPC >= 1 && NSD >= 1, "chunk shape");
+  constexpr int NSE = NB * GW * 8;     // scale dwords (two rows each) per wave and chunk
+  constexpr int NSD = (NSE + 63) / 64;
+  static_assert(CG % KS == 0 && GW >= 1 && GW == SPC * WS && (SPC == 1 || SPC == 2) && NPC >= 1, "chunk shape");
+  static_assert(4 * NB * NT * 4 * 64 * 4 <= 2 * TBK * XSC, "the partial sums reuse the activation buffers");
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
+  const int kh = w % KS;  // which part of every chunk this wave takes
 
   const GemvWork wk = gemv_resolve<DEVUNITS>(a);
   const GemvClass &c = wk.c;
@@ -1485,16 +1492,18 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   const int K = c.K, G = c.G;
   unsigned char *xs = smem;                                   // [2][TBK][XSC]
   float *xsum = (float *)(smem + (size_t)2 * TBK * XSC);      // [2][TBK][CG]
-  float *sfw = xsum + 2 * TBK * CG + w * (NB * CG * 32);      // this wave's [NB][CG][16 rows][2]
+  float *sfw = xsum + 2 * TBK * CG + w * (NB * CG * 32);      // this wave's [NB][GW][16 rows][2]
 
-  const int b = wk.b * 4 + w;  // the wave's block pair
+  const int b = wk.b * (4 / KS) + w / KS;  // the wave's block pair
   const int rbA = 2 * b;
   const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
   const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
   const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
   const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
   const int NCH = (G + CG - 1) / CG;  // activation chunks
-  const int NS = (G + WS - 1) / WS;   // weight steps
+  // first group of this wave's weight step i (steps past the end of the reduction are empty;
+  // the non-empty ones are a prefix)
+  auto step_group = [&](const int i) { return (i / SPC) * CG + kh * GW + (i % SPC) * WS; };
 
   for (int t0 = 0; t0 < m; t0 += TBK) {
     const int mc = (m - t0) < TBK ? (m - t0) : TBK;
@@ -1510,8 +1519,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
     }
     uint4 xr[NPC];
     u32 scr[NSD], zr[NSD];
-    // loads of one chunk: activations, scale dwords and the zero dwords that hold their nibbles
-    // (groups past the end of the reduction: zero activations, zero scales)
+    // loads of one chunk: activations, this wave's scale dwords and the zero dwords that hold their
+    // nibbles (groups past the end of the reduction: zero activations, zero scales)
     auto load_chunk = [&](const int ch) {
 #pragma unroll
       for (int i = 0; i < NPC; ++i) {
@@ -1523,16 +1532,17 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
 #pragma unroll
       for (int i = 0; i < NSD; ++i) {
         const int e = lane + 64 * i;
-        const int n = e / (CG * 8), g = ch * CG + ((e % (CG * 8)) >> 3), j = e & 7;
-        const bool ok = g < G;
+        const int n = e / (GW * 8), g = ch * CG + kh * GW + ((e % (GW * 8)) >> 3), j = e & 7;
+        const bool ok = e < NSE && g < G;
         scr[i] = bload4(rs, ok ? ((n * G + g) * 8 + j) * 4 : 0x7ffffff0, 0);
         zr[i] = bload4(rz, ok ? (n * G + g) * 8 + (j >> 2) * 4 : 0x7ffffff0, 0);
       }
     };
-    auto load_w = [&](const int s, uint4 (&wt_)[WS][NB]) {
+    auto load_w = [&](const int i, uint4 (&wt_)[WS][NB]) {
+      const int g0 = step_group(i);
 #pragma unroll
       for (int j = 0; j < WS; ++j) {
-        const int g = s * WS + j < G ? s * WS + j : G - 1;
+        const int g = g0 + j < G ? g0 + j : G - 1;
 #pragma unroll
         for (int n = 0; n < NB; ++n) wt_[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
       }
@@ -1562,19 +1572,22 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
 #pragma unroll
       for (int i = 0; i < NSD; ++i) {
         const int e = lane + 64 * i;
-        ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
+        if (e < NSE) ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
       }
       __syncthreads();
       if (ch + 1 < NCH) load_chunk(ch + 1);
     };
-    // weight step s (four groups) on the tiles in cur; the next step's tiles go to nxt first
-    auto step = [&](const int s, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
-      if (s + 1 < NS) load_w(s + 1, nxt);
-      const int cb = (s / SPC) & 1;
+    // this wave's weight step i on the tiles in cur; the next step's tiles go to nxt first
+    auto step = [&](const int i, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
+      const int g0 = step_group(i);
+      if (g0 >= G) return;
+      if (step_group(i + 1) < G) load_w(i + 1, nxt);
+      const int cb = (i / SPC) & 1;
 #pragma unroll
       for (int j = 0; j < WS; ++j) {
-        if (s * WS + j < G) {  // uniform
-          const int gq = (s % SPC) * WS + j;
+        if (g0 + j < G) {  // uniform
+          const int gl = (i % SPC) * WS + j;  // group within this wave's part of the chunk
+          const int gq = kh * GW + gl;        // and within the chunk
           bf16x8_t xv[NT][4];
           float xg[NT];
 #pragma unroll
@@ -1589,7 +1602,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
             const bf16x8_t w0 = deq8_bf16(cur[j][n].x), w1 = deq8_bf16(cur[j][n].y);
             const bf16x8_t w2 = deq8_bf16(cur[j][n].z), w3 = deq8_bf16(cur[j][n].w);
             // (s, -s (128 + z)) of the 4 rows this lane owns in D: rows 4qd..4qd+3
-            const float4 *sf = (const float4 *)(sfw + ((n * CG + gq) * 16 + 4 * qd) * 2);
+            const float4 *sf = (const float4 *)(sfw + ((n * GW + gl) * 16 + 4 * qd) * 2);
             const float4 f0 = sf[0], f1 = sf[1];
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -1610,12 +1623,12 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
 
     uint4 wA[WS][NB], wB[WS][NB];
     load_chunk(0);
-    load_w(0, wA);
+    if (step_group(0) < G) load_w(0, wA);
     if constexpr (SPC == 2) {
       for (int ch = 0; ch < NCH; ++ch) {
         chunk_begin(ch);
         step(2 * ch, wA, wB);
-        if (2 * ch + 1 < NS) step(2 * ch + 1, wB, wA);
+        step(2 * ch + 1, wB, wA);
       }
     } else {
       for (int ch = 0; ch < NCH; ch += 2) {
@@ -1627,26 +1640,52 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
         }
       }
     }
-    // every lane holds 4 consecutive rows of both blocks for one token per column block
+    if constexpr (KS > 1) {
+      // the sums of a pair's waves meet in the activation buffers (free once every wave is done with them)
+      __syncthreads();
+      float *red = (float *)smem;  // [4 waves][NB][NT][4][64 lanes]
+      if (kh != 0) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      if (16 * t + r < mc) {
-        const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
-        if (SWIGLU) {
-          u32 h[2];
+        for (int n = 0; n < NB; ++n)
 #pragma unroll
-          for (int i = 0; i < 2; ++i) {
-            const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
-            const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
-            const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
-            h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
-          }
-          *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
-        } else {
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((w * NB + n) * NT + t) * 256 + i * 64 + lane] = acc[n][t][i];
+      }
+      __syncthreads();
+      if (kh == 0) {
+#pragma unroll
+        for (int q = 1; q < KS; ++q)
 #pragma unroll
           for (int n = 0; n < NB; ++n)
-            *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
-                make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) acc[n][t][i] += red[(((w + q) * NB + n) * NT + t) * 256 + i * 64 + lane];
+      }
+    }
+    // every lane holds 4 consecutive rows of both blocks for one token per column block
+    if (kh == 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (16 * t + r < mc) {
+          const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
+          if (SWIGLU) {
+            u32 h[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+              const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
+              const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
+              const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
+              h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
+            }
+            *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
+          } else {
+#pragma unroll
+            for (int n = 0; n < NB; ++n)
+              *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
+                  make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
+          }
         }
       }
     }
@@ -1917,26 +1956,27 @@ static size_t gemv_mfma_kc_lds(int nt, int cg) {
   return (size_t)2 * 16 * nt * (cg * 256 + 16) + (size_t)2 * 16 * nt * cg * 4 + (size_t)4 * 2 * cg * 32 * 4;
 }
 
-// chunked-K form: a workgroup takes four block pairs of a unit (both classes' pair counts are
+// chunked-K form: a workgroup takes 4 / KS block pairs of a unit (both classes' pair counts are
 // multiples of four: I and H are multiples of 128)
-template <bool SW, int NT, int CG>
-static int launch_gemv_mfma_kc(const GemvArgs &a_in, int grid_in, hipStream_t s) {
+template <bool SW, int NT, int CG, int KS>
+static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t s) {
+  constexpr int PW = 4 / KS;
   GemvArgs a = a_in;
   const int units = a.cls[1].nblk > 0 ? (grid_in - a.n_sh_blocks) / a.cls[1].nblk : 0;
   if ((a.n_sh_blocks > 0 && a.cls[0].nblk % 4) || (units > 0 && a.cls[1].nblk % 4)) {
     moe_set_error("k_gemv_int4_mfma_kc: block pairs per unit not a multiple of 4");
     return MOE_EINVAL;
   }
-  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= 4; a.n_sh_blocks /= 4; }
-  a.cls[1].nblk /= 4;
+  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
+  a.cls[1].nblk /= PW;
   const int grid = a.n_sh_blocks + units * a.cls[1].nblk;
   const size_t lds = gemv_mfma_kc_lds(NT, CG);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NT, CG>,
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NT, CG, KS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NT, CG>,
+      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NT, CG, KS>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
@@ -1945,10 +1985,18 @@ static int launch_gemv_mfma_kc(const GemvArgs &a_in, int grid_in, hipStream_t s)
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NT, CG>), dim3(grid), dim3(256), lds, s, a);
-  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NT, CG>), dim3(grid), dim3(256), lds, s, a);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NT, CG, KS>), dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NT, CG, KS>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4_mfma_kc");
+}
+
+// Waves per block pair: one if the launch would give every CU its two workgroups with all units in use
+// (the unit list is made on the device, the host only knows its capacity), else two.  Four never paid.
+template <bool SW, int NT, int CG>
+static int launch_gemv_mfma_kc(const GemvArgs &a, int grid, hipStream_t s) {
+  if (grid / 4 >= 512) return launch_gemv_mfma_kc_ks<SW, NT, CG, 1>(a, grid, s);
+  return launch_gemv_mfma_kc_ks<SW, NT, CG, 2>(a, grid, s);
 }
 
 // 0: dot2 GEMV for T == 1, matrix-core form otherwise (default); 1: always dot2; 2: always MFMA
@@ -1970,10 +2018,14 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
   if (ch < 1) ch = 1;
   const int mode = gemv_mode();
   if (mode == 2 || (mode == 0 && T > 1)) {
-    // chunked-K form: reductions too long for two workgroups per CU with the whole rows staged, and
-    // batches of more than 16 tokens (measured on the 4096 x 14336 and 2048 x 1408 shapes: the w2 pass
-    // gains from 32-token passes above 32 tokens, the w13 pass does not)
-    if (Kmax > 2048 || T > 16) {
+    // token rows the whole-row form would stage, and whether two of its workgroups then share a CU
+    int tb_full = 1;
+    while (tb_full < T && tb_full < 16) tb_full <<= 1;
+    const bool whole_rows_fit = gemv_mfma_lds(tb_full, Kmax, 2) <= 80 * 1024;
+    // chunked-K form: 16 tokens and more, and reductions too long for the whole-row form (measured on
+    // the 2048 x 1408 (+ 2816 shared) and 4096 x 14336 shapes; the w2 pass gains from 32-token passes
+    // above 32 tokens, the w13 pass does not)
+    if (T >= 16 || !whole_rows_fit) {
       if (!SW && T > 32) return launch_gemv_mfma_kc<SW, 2, 4>(a, grid, s);
       return launch_gemv_mfma_kc<SW, 1, 8>(a, grid, s);
     }
