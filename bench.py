@@ -40,7 +40,8 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (matrix-core) legs")
     ap.add_argument("--only", default="", help="profiling aid: run only these prefill legs (comma list of "
-                    "qwen, deepseek, mixtral) and print their results, without the decode benchmark")
+                    "qwen, deepseek, mixtral; other = the decode legs of the other configurations) and print their "
+                    "results, without the decode benchmark")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: also run a plain 256 MiB read + 256 MiB write elementwise kernel three "
                          "times, the known-size reference for FETCH_SIZE / WRITE_SIZE counters")
@@ -194,9 +195,19 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
     ws = None
     nact = []
 
+    # one token, int4: the path moe_forward takes (routing inside the w13 kernel, w2 + combine in one launch)
+    token_path = T == 1 and not q4k
+    unit_ws = torch.zeros(32 * k, dtype=torch.uint8, device=dev)
+    ws_tok = None
+
     def step(i, phases=3, route=True):
-        nonlocal ws
+        nonlocal ws, ws_tok
         l, x = i % layers, xs[i % len(xs)]
+        if token_path and phases == 3:
+            ops.gate_logits(x, gws[l], biases[l], out=logits)
+            ws_tok = ops.decode_token_int4(x, logits, E, k, mode, tables[l], shs[l], H, I, I_sh, ws=ws_tok, phases=5,
+                                           unit_ws=unit_ws, sg_logit=logits[:, E] if gated else None, y=y)
+            return
         if route:
             ops.gate_logits(x, gws[l], biases[l], out=logits)
             idx, w = ops.topk(logits, k, mode, E=E)
@@ -220,7 +231,14 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
 
     for i in range(4 * layers):
         step(i)
-        nact.append(int(d.n_active.cpu()[0]))
+        nact.append(int((ws_tok[2] if token_path else d).n_active.cpu()[0]))
+    if token_path:   # the one-token path against the separate kernels on the same input
+        y_tok = y.float().clone()
+        token_path = False
+        step(4 * layers - 1)
+        token_path = True
+        assert int(ws_tok[5].cpu()[0]) == 0
+        assert float((y_tok - y.float()).abs().max()) <= 1e-2 * float(y.float().abs().max())
     assert int(ws[2].cpu()[0]) == 0
     t_layer = timed(step, steps)
     # the w13 + SwiGLU GEMV alone, back to back, with the routing of the last full step kept
@@ -279,8 +297,11 @@ def main():
                              2048, 2048, 64, 1408, 6, 2816, L.FMT_INT4_G128, False, 0, 20),
                 "mixtral": ("Mixtral-8x7B-shaped layer, int4-g128 experts, prefill T=4096, all resident",
                             4096, 4096, 8, 14336, 2, 0, L.FMT_INT4_G128, False, 2, 5)}
-        res = [prefill_leg(torch, *legs[n][:-1], steps=legs[n][-1]) for n in a.only.split(",")]
-        print(json.dumps({"prefill": res}))
+        names = a.only.split(",")
+        res = {"prefill": [prefill_leg(torch, *legs[n][:-1], steps=legs[n][-1]) for n in names if n != "other"]}
+        if "other" in names:
+            res["other_decode_configs"] = other_configs(torch)
+        print(json.dumps(res))
         return
 
     global xs_out

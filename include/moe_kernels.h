@@ -120,7 +120,7 @@ int moe_route_decode(const void *x_bf16, const void *wg_bf16, const float *bias,
                      moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
                      unsigned *counter, void *stream);
 
-/* k1b + k2 in one launch (one workgroup) for decode batches: T <= 16, E <= 256, T*k <= 512; same
+/* k1b + k2 in one launch (one workgroup) for decode batches: T <= 64, E <= 256, T*k <= 512; same
  * results, bit for bit, as moe_topk + moe_dispatch.  units_host_out / n_active_host_out /
  * seq_host_out (optional, pinned HOST memory): the kernel also stores the unit list and its length
  * there and then, once those stores have completed, seq_value into *seq_host_out. */
@@ -135,7 +135,8 @@ int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mod
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL
  *   h_r [P, I] bf16, h_s [T, I_sh] bf16, part_r [P, H] fp32, part_s [T, H] fp32: workspaces
  * Rows of the routed buffers follow the sorted pair order of moe_dispatch.
- * Covers tokens-per-expert of any size by chunks of <=16 rows; meant for T <= 16.
+ * Covers tokens-per-expert of any size by passes of 16 rows (32 in the w2 pass above 32 tokens);
+ * meant for T <= 64.
  * units_host / expert_ptr_host (HOST copies of the unit list and of the slot table row,
  * both optional): when given and max_units <= 64 the units travel in the kernel arguments
  * and the kernels read neither `units` nor `expert_ptr`.

@@ -2287,7 +2287,7 @@ extern "C" int moe_route_decode(const void *x, const void *wg, const float *bias
                                 int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
                                 int64_t *active_ids, int max_units, unsigned *counter, void *stream) {
   if (!x || !wg || !logits || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair ||
-      !sorted_tok || !units || !n_active || !active_ids || !counter || T <= 0 || T > ROUTE_MAXT || H <= 0 || H % 8 ||
+      !sorted_tok || !units || !n_active || !active_ids || !counter || T <= 0 || T > 16 || H <= 0 || H % 8 ||
       E <= 0 || E > 256 || E_rows < E || E_rows > E + 1 || ldl < E_rows || k <= 0 || k > 32 || k > E ||
       T * k > ROUTE_MAXP || mode < 0 || mode > 2 || max_units < 0) {
     moe_set_error("moe_route_decode: bad argument (T=%d H=%d E=%d k=%d)", T, H, E, k);

@@ -74,7 +74,7 @@ def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispa
 
 
 def topk_dispatch(logits: torch.Tensor, k: int, E: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
-    """Top-k and dispatch in one launch for T <= 16.  Returns (idx, w, Dispatch)."""
+    """Top-k and dispatch in one launch for T <= 64.  Returns (idx, w, Dispatch)."""
     T = logits.shape[0]
     idx = torch.empty(T, k, dtype=torch.int32, device=logits.device)
     w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
@@ -90,7 +90,7 @@ _route_counter = {}
 
 
 def route_decode(x, wg, bias, E: int, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK):
-    """Fused gate logits + top-k + dispatch for T <= 16.  wg may carry one extra row (shared gate)."""
+    """Fused gate logits + top-k + dispatch for T <= 64.  wg may carry one extra row (shared gate)."""
     if x.device not in _route_counter:   # the launch counter of the fused kernel: zero between calls
         _route_counter[x.device] = torch.zeros(1, dtype=torch.int32, device=x.device)
     T, H = x.shape

@@ -295,7 +295,7 @@ def test_token_decode_w2_and_combine_in_one_launch(cuda, H, I, E, k, mode, I_sh,
 
 
 @pytest.mark.parametrize("T,E,k,mode", [(1, 64, 6, 0), (4, 64, 6, 0), (16, 64, 6, 1), (16, 60, 4, 2), (7, 200, 8, 0),
-                                        (16, 8, 2, 2), (3, 256, 32, 0)])
+                                        (16, 8, 2, 2), (3, 256, 32, 0), (32, 64, 6, 0), (64, 64, 8, 1), (33, 60, 4, 2)])
 def test_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode):
     from promoe_amd import ops
     print(f"case topk_dispatch T={T} E={E} k={k} mode={mode}", flush=True)
