@@ -1525,9 +1525,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
 #pragma unroll
       for (int i = 0; i < NPC; ++i) {
         const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
-        const bool in = kv * 8 < K;
-        const uint4 v = bload16(rx, xoff[i] + (in ? kv * 16 : 0), 0);
-        xr[i] = in ? v : make_uint4(0u, 0u, 0u, 0u);
+        // columns past K: any valid address; chunk_begin zeroes them (a select here would wait for the load)
+        xr[i] = bload16(rx, xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
       }
 #pragma unroll
       for (int i = 0; i < NSD; ++i) {
@@ -1563,10 +1562,11 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
       for (int i = 0; i < NPC; ++i) {
         const int p = tid + 256 * i;
         const int row = p / XV, v = p & (XV - 1);
-        float ps = sum8_bf16(xr[i]);
+        const uint4 xq = (ch * XV + v) * 8 < K ? xr[i] : make_uint4(0u, 0u, 0u, 0u);
+        float ps = sum8_bf16(xq);
         ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
         ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
-        *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xr[i];
+        *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xq;
         if ((tid & 15) == 0) xsum[(cb * TBK + row) * CG + (v >> 4)] = ps;
       }
 #pragma unroll
