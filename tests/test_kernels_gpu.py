@@ -148,7 +148,7 @@ def test_decode_layer_small_variants(cuda):
     check_layer(Int4Layer(H=384, I=640, E=4, I_sh=128, seed=6), 3, 2, 0, cuda)
 
 
-@pytest.mark.parametrize("T", [3, 16, 20, 40, 64])
+@pytest.mark.parametrize("T", [3, 16, 20, 40, 64, 70])
 def test_decode_layer_long_reduction(cuda, T):
     """Reductions longer than 2048 and batches of more than 16 tokens take the chunked-K GEMV: group counts
     that leave a partial last chunk and an odd number of weight steps (G = 18, 17, 20), units with more rows
