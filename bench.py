@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2700)
     ap.add_argument("--warmup", type=int, default=270)
-    ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch): 1, 4 or 16")
+    ap.add_argument("--tokens", type=int, default=1, help="tokens per step (decode batch): 1 to 64 stay on the GEMV kernels")
     ap.add_argument("--layers", type=int, default=27)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-cache-run", action="store_true")
