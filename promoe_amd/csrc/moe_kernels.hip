@@ -1991,11 +1991,13 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   return moe_check_launch("k_gemv_int4_mfma_kc");
 }
 
-// Waves per block pair: one if the launch would give every CU its two workgroups with all units in use
-// (the unit list is made on the device, the host only knows its capacity), else two.  Four never paid.
+// Waves per block pair: two for launches of few block pairs (under 384 workgroups of four pairs with every
+// unit slot in use; the unit list is made on the device, the host only knows its capacity), else one.
+// Measured: 256 workgroups (4096 x 14336 w2, 8 units) 101 us with one wave per pair, 77 us with two; 484
+// workgroups (2048 x 1408 w13, 20 units) 19.5 us against 25.7 us.  Four never paid.
 template <bool SW, int NT, int CG>
 static int launch_gemv_mfma_kc(const GemvArgs &a, int grid, hipStream_t s) {
-  if (grid / 4 >= 512) return launch_gemv_mfma_kc_ks<SW, NT, CG, 1>(a, grid, s);
+  if (grid / 4 >= 384) return launch_gemv_mfma_kc_ks<SW, NT, CG, 1>(a, grid, s);
   return launch_gemv_mfma_kc_ks<SW, NT, CG, 2>(a, grid, s);
 }
 
