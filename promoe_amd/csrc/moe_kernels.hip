@@ -1575,13 +1575,15 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
         if (e < NSE) ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
       }
       __syncthreads();
-      if (ch + 1 < NCH) load_chunk(ch + 1);
+      // unconditional (past the end: clamped addresses, zero scales), so that every iteration issues the
+      // same number of loads and the waits for the prefetched registers can be exact
+      load_chunk(ch + 1);
     };
     // this wave's weight step i on the tiles in cur; the next step's tiles go to nxt first
     auto step = [&](const int i, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
       const int g0 = step_group(i);
+      load_w(i + 1, nxt);  // unconditional, clamped: see chunk_begin
       if (g0 >= G) return;
-      if (step_group(i + 1) < G) load_w(i + 1, nxt);
       const int cb = (i / SPC) & 1;
 #pragma unroll
       for (int j = 0; j < WS; ++j) {
@@ -1623,7 +1625,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
 
     uint4 wA[WS][NB], wB[WS][NB];
     load_chunk(0);
-    if (step_group(0) < G) load_w(0, wA);
+    load_w(0, wA);
     if constexpr (SPC == 2) {
       for (int ch = 0; ch < NCH; ++ch) {
         chunk_begin(ch);
