@@ -77,10 +77,12 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[4][2], uint16
   const int kc = tid & 7, r0 = tid >> 3;  // staging: row r0 + 64 i (block 2i + g), 16-byte chunk kc
   const int fr = lane & 31, q = lane >> 5;
   u32x4_t ra[4], bufA[2][4], bufB[2][4];
+  // (block 2i + g is live iff i < NBW: a compile-time condition, so every iteration issues the same
+  // number of loads and the compiler's waits for the prefetched registers can be exact)
   auto gloadA = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (2 * i + g < nb) ra[i] = *(g_uint4 *)(a_ptr[i] + kt * PF_BK);
+      if (i < NBW) ra[i] = *(g_uint4 *)(a_ptr[i] + kt * PF_BK);
   };
   auto gloadB = [&](u32x4_t(&b)[2][4], int kt) {
     int k0 = kt + rot0, k1 = kt + rot1;  // slab position inside the 128-row group's storage
@@ -95,7 +97,7 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[4][2], uint16
     uint16_t *A_ = As + st * PF_BM * PF_LDK;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (2 * i + g < nb) *(u32x4_t *)(A_ + (r0 + 64 * i) * PF_LDK + kc * 8) = ra[i];
+      if (i < NBW) *(u32x4_t *)(A_ + (r0 + 64 * i) * PF_LDK + kc * 8) = ra[i];
   };
   auto compute = [&](int st, const u32x4_t(&b)[2][4]) {
     const uint16_t *A_ = As + st * PF_BM * PF_LDK + (32 * g + fr) * PF_LDK + 32 * q;
@@ -114,10 +116,11 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[4][2], uint16
   // one K slab: the weight fragments of slab kt are in `cur`; slab kt+1's are requested into
   // `nxt`, and its activations go through registers into the other LDS stage
   auto step = [&](int kt, const u32x4_t(&cur)[2][4], u32x4_t(&nxt)[2][4]) {
-    if (kt + 1 < nk) {
-      gloadA(kt + 1);
-      if (NBW > 0) gloadB(nxt, kt + 1);
-    }
+    // unconditional: the last slab requests itself once more instead of branching around the loads
+    const int kn = kt + 1 < nk ? kt + 1 : kt;
+    gloadA(kn);
+    if (NBW > 0) gloadB(nxt, kn);
+    __builtin_amdgcn_sched_barrier(0);  // the requests go out before the products, not after them
     compute(kt & 1, cur);
     if (kt + 1 < nk) {
       sstore((kt + 1) & 1);
@@ -302,8 +305,8 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   // the same three staging registers
   auto gloadA = [&](int gi, int half) {
 #pragma unroll
-    for (int i = 0; i < 3; ++i)
-      if (3 * half + i < nb) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[3 * half + i], gi * 256, 0);
+    for (int i = 0; i < 3; ++i)  // unconditional (blocks past the tile's end re-read its first rows): the same
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[3 * half + i], gi * 256, 0);  // number of loads in every iteration
   };
   auto sstore = [&](int st, int half) {
     uint16_t *A_ = As + st * PI_BM * PI_LDK;
@@ -364,15 +367,16 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   };
   auto step = [&](int gi, const u32x4_t(&cur)[4], const PiMeta &mc, u32x4_t(&nxt)[4], PiMeta &mn) {
     const bool more = gi + 1 < G;
-    if (more) {
-      gloadA(gi + 1, 0);
-      if (NBW > 0) gloadW(nxt, mn, gi + 1);
-    }
+    // unconditional requests (the last group asks for itself once more), pinned in front of the products: with
+    // loads under conditions the compiler's waits for the current tiles also wait for the ones just requested
+    const int gn = more ? gi + 1 : gi;
+    gloadA(gn, 0);
+    if (NBW > 0) gloadW(nxt, mn, gn);
+    __builtin_amdgcn_sched_barrier(0);
     if (NBW > 0) compute2(gi & 1, cur, mc, 0);
-    if (more) {
-      sstore((gi + 1) & 1, 0);
-      if (nb > 3) gloadA(gi + 1, 1);
-    }
+    if (more) sstore((gi + 1) & 1, 0);
+    gloadA(gn, 1);
+    __builtin_amdgcn_sched_barrier(0);
     if (NBW > 0) compute2(gi & 1, cur, mc, 2);
     if (more) {
       if (nb > 3) sstore((gi + 1) & 1, 1);
