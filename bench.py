@@ -315,7 +315,7 @@ def main():
           (L_, E, stack.expert_bytes * L_ * E / 1e9, time.perf_counter() - t_setup), file=sys.stderr, flush=True)
 
     # ---- steady-state hits: every expert resident -------------------------------------
-    pm = stack.engine(max(16, T), cache_rate=1.0, cache_policy="lru")
+    pm = stack.engine(max(64, T), cache_rate=1.0, cache_policy="lru")
     import numpy as np
     for l in range(L_):                      # bring every expert into its slot
         pm.acquire_layer(l, np.arange(E, dtype=np.int64))
@@ -412,7 +412,7 @@ def main():
 
     sweep = {}
     if not a.no_sweep:
-        for Tn in (1, 4, 16):
+        for Tn in (1, 4, 16, 64):
             if Tn == T:
                 sweep[str(Tn)] = value
                 continue
