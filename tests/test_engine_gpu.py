@@ -118,7 +118,8 @@ def test_forward_all_resident_has_no_misses_after_warmup(cuda):
     pm.release_layer(0)
     c0 = pm.counters()
     n_act = 0
-    for T in (1, 5, 16, 2):
+    # 24, 32: routing tail in one launch above 16 tokens; 40, 64: separate routing kernels, still the GEMV kernels
+    for T in (1, 5, 16, 2, 24, 32, 40, 64):
         x = O.synth_acts(T, 256, seed=50 + T)
         y = pm.forward(0, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
         torch.cuda.synchronize()
