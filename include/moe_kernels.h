@@ -135,7 +135,7 @@ int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mod
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL
  *   h_r [P, I] bf16, h_s [T, I_sh] bf16, part_r [P, H] fp32, part_s [T, H] fp32: workspaces
  * Rows of the routed buffers follow the sorted pair order of moe_dispatch.
- * Covers tokens-per-expert of any size by passes of 16 rows (32 in the w2 pass above 32 tokens);
+ * Covers tokens-per-expert of any size by passes of 16 rows (32 in the w2 pass above 48 tokens);
  * meant for T <= 64.
  * units_host / expert_ptr_host (HOST copies of the unit list and of the slot table row,
  * both optional): when given and max_units <= 64 the units travel in the kernel arguments

@@ -2032,9 +2032,10 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
     const bool whole_rows_fit = gemv_mfma_lds(tb_full, Kmax, 2) <= 80 * 1024;
     // chunked-K form: 16 tokens and more, and reductions too long for the whole-row form (measured on
     // the 2048 x 1408 (+ 2816 shared) and 4096 x 14336 shapes; the w2 pass gains from 32-token passes
-    // above 32 tokens, the w13 pass does not)
+    // above 48 tokens - at 40 and 48 they tie on the first shape and lose 128 to 85 us on the second -,
+    // the w13 pass only under skewed routing)
     if (T >= 16 || !whole_rows_fit) {
-      if (!SW && T > 32) return launch_gemv_mfma_kc<SW, 2, 4>(a, grid, s);
+      if (!SW && T > 48) return launch_gemv_mfma_kc<SW, 2, 4>(a, grid, s);
       return launch_gemv_mfma_kc<SW, 1, 8>(a, grid, s);
     }
     int tb = 1;

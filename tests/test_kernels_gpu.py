@@ -152,7 +152,7 @@ def test_decode_layer_small_variants(cuda):
 def test_decode_layer_long_reduction(cuda, T):
     """Reductions longer than 2048 and batches of more than 16 tokens take the chunked-K GEMV: group counts
     that leave a partial last chunk and an odd number of weight steps (G = 18, 17, 20), units with more rows
-    than one pass holds (E = 4, k = 2: about T / 2 rows per unit), 32-token passes in w2 above 32 tokens."""
+    than one pass holds (E = 4, k = 2: about T / 2 rows per unit), 32-token passes in w2 above 48 tokens."""
     print(f"case decode_long_reduction T={T}", flush=True)
     layer = Int4Layer(H=2304, I=2176, E=4, I_sh=2560, seed=8)
     check_layer(layer, T, 2, 0, cuda)
