@@ -211,6 +211,10 @@ int moe_forward_prepare(moe_engine *eng, int max_tokens);
 int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y);
 /* routing of the last moe_forward call of this layer (device pointers; valid until the next call) */
 int moe_last_routing(moe_engine *eng, const int **idx, const float **w, const int **sorted_pair);
+/* the same routing copied to the host once the compute stream has drained: idx_host [T*k] int32 and/or
+ * w_host [T*k] fp32 (either may be NULL).  A checking aid with no reference counterpart (the reference's
+ * module keeps its routing in torch tensors of its own). */
+int moe_last_routing_host(moe_engine *eng, int T, int k, int *idx_host, float *w_host);
 
 #ifdef __cplusplus
 }

@@ -143,3 +143,4 @@ _sig("moe_set_layer", [vp, i32, C.POINTER(LayerDesc)])
 _sig("moe_forward_prepare", [vp, i32])
 _sig("moe_forward", [vp, i32, vp, i32, vp])
 _sig("moe_last_routing", [vp, pp, pp, pp])
+_sig("moe_last_routing_host", [vp, i32, i32, vp, vp])

@@ -607,6 +607,8 @@ moe_engine::~moe_engine() {
   moe_predictor_free(this);
   if (fetch_thread.joinable()) fetch_thread.join();
   if (fw) { moe_forward_free(fw); fw = nullptr; }
+  for (LayerState *old : fw_retired) moe_forward_free(old);
+  fw_retired.clear();
 }
 
 extern "C" int moe_engine_create(const moe_cfg *cfg, int backend, void *compute_stream, moe_engine **out) {
@@ -1060,9 +1062,10 @@ int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int6
   for (int64_t i = 0; i < n; ++i)
     if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
   // run-ahead budget (worker.cpp:41-53)
-  while (eng->budget <= 0) {
+  if (eng->exiting) return MOE_ESTATE;  // a producer that arrives after shutdown began must not sleep on the budget
+  if (eng->budget <= 0) {
     if (!blocking) return 1;
-    eng->cv_sem.wait(lk);
+    eng->cv_sem.wait(lk, [&] { return eng->budget > 0 || eng->exiting; });
     if (eng->exiting) return MOE_ESTATE;
   }
   eng->budget--;
@@ -1184,7 +1187,18 @@ extern "C" int moe_drain(moe_engine *eng) {
     return true;
   });
   if (!eng->fatal.empty()) { moe_set_error("engine failed: %s", eng->fatal.c_str()); return MOE_ESTATE; }
-  return MOE_OK;
+  lk.unlock();
+  return moe_forward_check_kernels(eng);
+}
+
+void engine_drop_seq_releases(moe_engine *eng) {
+  std::lock_guard<std::mutex> lk(eng->mu);
+  for (auto &x : eng->experts)
+    if (x->seq_ptr) {
+      x->seq_ptr = nullptr;
+      if (x->status.load() == kUsing) x->status = kReady;
+    }
+  eng->cv_state.notify_all();
 }
 
 extern "C" int moe_streams(moe_engine *eng, void **compute, void **copy) {

@@ -17,7 +17,7 @@ struct LayerState {
   int E = 0, H = 0, I = 0, I_sh = 0;
   float *logits = nullptr, *topk_w = nullptr, *part_r = nullptr, *part_s = nullptr;
   int *idx = nullptr, *counts = nullptr, *offsets = nullptr, *sorted_pair = nullptr, *pos_of_pair = nullptr,
-      *sorted_tok = nullptr, *n_active = nullptr, *err = nullptr;
+      *sorted_tok = nullptr, *n_active = nullptr;
   unsigned *route_counter = nullptr;
   unsigned char *unit_ws = nullptr;  // resolved units of the one-token path (16 bytes each)
   moe_unit *units = nullptr, *units_sub = nullptr;
@@ -25,8 +25,12 @@ struct LayerState {
   void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
   // pinned host mirrors
   moe_unit *units_host = nullptr, *units_sub_host = nullptr;
-  int *n_active_host = nullptr, *err_host = nullptr, *opt_seq = nullptr;
-  int *err_opt = nullptr;  // error word of launches that are allowed to meet non-resident experts
+  int *n_active_host = nullptr, *opt_seq = nullptr;
+  // error words the kernels raise when a selected expert has no slot, in pinned host memory so that the host
+  // sees them without a copy: one per layer for launches in which that must not happen (checked at the next
+  // call and when the engine drains), one for launches that are allowed to meet non-resident experts
+  int *err_host = nullptr, *err_loose = nullptr;
+  int num_layer = 0;
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
   int sub_cursor = 0;
@@ -113,7 +117,18 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
     H = std::max(H, d.H); I = std::max(I, d.I); I_sh = std::max(I_sh, d.I_sh); k = std::max(k, d.top_k);
   }
   if (H == 0) { moe_set_error("moe_forward_prepare: no layer described (moe_set_layer)"); return MOE_ESTATE; }
-  if (eng->fw) { moe_forward_free(eng->fw); eng->fw = nullptr; }
+  if (eng->fw) {
+    // a second prepare: account the routings still pending, let the stream drain, and take every expert off
+    // the sequence words of the old workspace (their launches are over) before that memory goes away
+    if (int rc = moe_forward_harvest(eng, true)) return rc;
+    HIPC(hipStreamSynchronize((hipStream_t)eng->be->compute_stream()));
+    if (int rc = moe_forward_check_kernels(eng)) return rc;
+    engine_drop_seq_releases(eng);
+    // the fetch thread may still be polling one of the old sequence words (it reads them without the
+    // lock): the old workspace is only freed with the engine, after that thread has been joined
+    eng->fw_retired.push_back(eng->fw);
+    eng->fw = nullptr;
+  }
   LayerState *s = new LayerState();
   eng->fw = s;
   const int E = eng->cfg.num_expert, T = max_tokens;
@@ -130,7 +145,6 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->pos_of_pair, P);
   rc |= dalloc(s, &s->sorted_tok, P);
   rc |= dalloc(s, &s->n_active, 1);
-  rc |= dalloc(s, &s->err, 1);
   rc |= dalloc(s, &s->route_counter, 1);
   rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
   rc |= dalloc(s, &s->units, s->max_units);
@@ -144,9 +158,10 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= halloc(s, &s->units_host, s->max_units);
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
   rc |= halloc(s, &s->n_active_host, 1);
-  rc |= halloc(s, &s->err_host, 1);
+  s->num_layer = eng->cfg.num_layer;
+  rc |= halloc(s, &s->err_host, eng->cfg.num_layer);
+  rc |= halloc(s, &s->err_loose, 1);
   rc |= halloc(s, &s->opt_seq, 1);
-  rc |= dalloc(s, &s->err_opt, 1);
   for (auto &p : s->pend) {
     rc |= halloc(s, &p.units, s->max_units);
     rc |= halloc(s, &p.n_active, 1);
@@ -155,11 +170,22 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
     if (hipEventCreateWithFlags(&p.ev, hipEventDisableTiming) != hipSuccess) rc = 1;
   }
   if (rc) return MOE_EHIP;
-  HIPC(hipMemset(s->err, 0, sizeof(int)));
+  memset(s->err_host, 0, sizeof(int) * eng->cfg.num_layer);
+  *s->err_loose = 0;
   HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
-  HIPC(hipMemset(s->err_opt, 0, sizeof(int)));
   *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
+  return MOE_OK;
+}
+
+// A strict error word is up: some launch of that layer skipped a selected expert, so what it combined is
+// wrong.  The engine fails (every later call reports it), as the reference would abort on a broken invariant.
+int moe_forward_check_kernels(moe_engine *eng) {
+  LayerState *s = eng->fw;
+  if (!s) return MOE_OK;
+  for (int l = 0; l < s->num_layer; ++l)
+    if (((volatile int *)s->err_host)[l])
+      return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", l);
   return MOE_OK;
 }
 
@@ -204,16 +230,16 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
   if (use_prefill(d, T))
     return moe_experts_prefill(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
                                s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
-                               s->part_s, s->tiles_ws, s->err, 3, st);
+                               s->part_s, s->tiles_ws, s->err_host + layer, 3, st);
   if (d.fmt == MOE_FMT_Q4K)
     return moe_experts_decode_q4k(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                   s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
-                                  s->part_r, s->part_s, s->err, 3, st);
+                                  s->part_r, s->part_s, s->err_host + layer, 3, st);
   // the host knows the units and the slot addresses: they travel in the kernel arguments
   const uint64_t *table_host = units_host ? eng->h_table + (size_t)layer * eng->cfg.num_expert : nullptr;
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
-                                 s->part_r, s->part_s, s->err, units_host, table_host, 3, st);
+                                 s->part_r, s->part_s, s->err_host + layer, units_host, table_host, 3, st);
 }
 
 // the one-token w2 + combine kernel stages the h vectors of all units in LDS
@@ -238,6 +264,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   int rc;
   // hook order of the reference (utils/hooks.py:216-223)
   // the layer hook's pre_forward: this block's input (decode: what the built-in predictor reads)
+  if ((rc = moe_forward_check_kernels(eng))) return rc;  // of earlier calls: the words arrive without a copy
   if ((rc = moe_report_layer_logits(eng, layer, x, 1, T, d.H))) return rc;
   const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
   if ((rc = moe_forward_harvest(eng, false))) return rc;
@@ -253,7 +280,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   }
   static const bool token_route = !(getenv("MOE_TOKEN_ROUTE") && atoi(getenv("MOE_TOKEN_ROUTE")) == 0);
   static const bool token_w2c = !(getenv("MOE_TOKEN_W2C") && atoi(getenv("MOE_TOKEN_W2C")) == 0);
-  if (all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
+  if (all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
     // one token: gate logits, then the w13 kernel routes by itself (no top-k / dispatch launches)
     if (!d.gate_bias) {
       if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
@@ -276,7 +303,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err, s->unit_ws, p.units, p.seq, seq,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws, p.units, p.seq, seq,
                                     w2c ? 5 : 3, sg0, y, st)))
       return rc;
     *p.n_active = k;
@@ -293,7 +320,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // reference's order (hits were computed already, misses are fetched and computed one by one) while the GPU
   // works.  From the table snapshot until the hooks have marked the hits, the layer's slot group is guarded:
   // prefetch and demand traffic may evict, but no copy into one of its slots starts.
-  const bool optimistic = !all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 &&
+  const bool optimistic = !all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 &&
                           eng->cfg.early_preempt && eng->cfg.reorder_experts && (size_t)d.H * 2 + 8192 <= 60 * 1024;
   if (optimistic) {
     if (!d.gate_bias) {
@@ -318,7 +345,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
                                     nullptr, nullptr, st)))
       return rc;
     {  // the routing arrives a few microseconds after the kernel starts
@@ -364,8 +391,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_opt, s->unit_ws, nullptr, nullptr, 0,
-                                    w2c ? 4 : 2, sgo, y, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, w2c ? s->err_host + layer : s->err_loose, s->unit_ws,
+                                    nullptr, nullptr, 0, w2c ? 4 : 2, sgo, y, st)))
       return rc;
     // no event in the stream (one costs the step about 4 us of GPU time): the experts count as in use until
     // the routing word of a LATER one-token step arrives, whose kernel starts behind everything queued here
@@ -392,7 +419,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
   bool routed_by_tail = false;
   int tail_seq = 0;
-  if (all_resident && fused_route && T <= 32 && E <= 256 && T * k <= 512) {
+  if (all_resident && fused_route && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory
     if (!d.gate_bias) {
@@ -411,7 +438,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                 max_units, pn.units, pn.n_active, pn.seq, tail_seq, st)))
       return rc;
     routed_by_tail = true;
-  } else if (fused_route && T <= 2 && E <= 256 && T * k <= 512) {
+  } else if (fused_route && T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
     // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
     // single workgroup behind a device-scope counter, which beats two more launches only
     // while that tail is short (measured: +5 % tokens/s at T=1, -2 % at T=4, -25 % at T=16)
@@ -522,5 +549,16 @@ extern "C" int moe_last_routing(moe_engine *eng, const int **idx, const float **
   if (idx) *idx = eng->fw->idx;
   if (w) *w = eng->fw->topk_w;
   if (sorted_pair) *sorted_pair = eng->fw->sorted_pair;
+  return MOE_OK;
+}
+
+extern "C" int moe_last_routing_host(moe_engine *eng, int T, int k, int *idx_host, float *w_host) {
+  if (!eng || !eng->fw) { moe_set_error("moe_last_routing_host: no forward workspace"); return MOE_ESTATE; }
+  LayerState *s = eng->fw;
+  if (T <= 0 || k <= 0 || T > s->max_tokens || k > s->max_k) { moe_set_error("moe_last_routing_host: T=%d k=%d outside the workspace", T, k); return MOE_EINVAL; }
+  HIPC(hipStreamSynchronize((hipStream_t)eng->be->compute_stream()));
+  const size_t n = (size_t)T * k;
+  if (idx_host) HIPC(hipMemcpy(idx_host, s->idx, n * sizeof(int), hipMemcpyDeviceToHost));
+  if (w_host) HIPC(hipMemcpy(w_host, s->topk_w, n * sizeof(float), hipMemcpyDeviceToHost));
   return MOE_OK;
 }

@@ -216,6 +216,7 @@ struct moe_engine {
   // fused forward
   std::vector<moe_layer_desc> layer_desc;
   LayerState *fw = nullptr;
+  std::vector<LayerState *> fw_retired;  // workspaces of earlier moe_forward_prepare calls, freed with the engine
   PredictorState *pred = nullptr;
 
   ~moe_engine();
@@ -231,6 +232,10 @@ int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int 
 int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resident_out);
 void moe_guard_release(moe_engine *eng, int layer);
 int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking, bool over_copy);
+// every expert that waits for a sequence word becomes ready (the caller has drained the compute stream)
+void engine_drop_seq_releases(moe_engine *eng);
+// fails the engine when a kernel raised a strict error word of the forward workspace
+int moe_forward_check_kernels(moe_engine *eng);
 int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need);
 // account demand hits of experts that were launched without a host round trip
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n);

@@ -885,7 +885,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
-    if (tid == 0) atomicOr(a.err, 1);
+    if (tid == 0) moe_raise_err(a.err);
     return;
   }
   const int K = c.K, G = c.G, KS = K >> 5;
@@ -1151,7 +1151,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
         ++gj;  // next item
         if (uj < k && gj >= G) { gj -= G; ++uj; }
       }
-      if (any_missing && lane == 0) atomicOr(a.err, 1);  // a selected expert that is not resident
+      if (any_missing && lane == 0) moe_raise_err(a.err);  // a selected expert that is not resident
       const bool shd = lu >= k;
       const int Gu = shd ? G_sh : G;
       wgt[c] = lw;
@@ -1266,7 +1266,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
-    if (tid == 0) atomicOr(a.err, 1);
+    if (tid == 0) moe_raise_err(a.err);
     return;
   }
   const int K = c.K, G = c.G;
@@ -1486,7 +1486,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
-    if (tid == 0) atomicOr(a.err, 1);
+    if (tid == 0) moe_raise_err(a.err);
     return;
   }
   const int K = c.K, G = c.G;

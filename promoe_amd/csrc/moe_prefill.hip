@@ -546,7 +546,7 @@ __global__ __launch_bounds__(1024) void k_prefill_tiles(const moe_unit *__restri
       if (un.m > 0 && un.expert >= 0) {
         wb = expert_ptr[un.expert];
         if (wb) { m = un.m; row0 = un.row0; }
-        else atomicOr(err, 1);
+        else moe_raise_err(err);
       }
     }
     const int nt = (m + cap - 1) / cap;

@@ -318,6 +318,13 @@ class PrefetchMngr:
         return a.value, b.value, c.value
 
 
+    def last_routing_idx(self, T: int, k: int) -> np.ndarray:
+        """Expert indices [T, k] of the last forward, copied back after the stream has drained (a checking aid)."""
+        out = np.empty((T, k), np.int32)
+        check(lib.moe_last_routing_host(self._h, T, k, out.ctypes.data, None), "last_routing_idx")
+        return out
+
+
 def slot_distribution(num_buffers: int, n_groups: int) -> list[int]:
     out = (C.c_int64 * n_groups)()
     check(lib.moe_slot_distribution(num_buffers, n_groups, out), "slot_distribution")

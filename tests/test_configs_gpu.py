@@ -1,0 +1,229 @@
+"""The benchmark configurations at their real widths, through the C ABI, against the CPU oracle.
+
+  C1  DeepSeek-MoE-16B layer, 64 experts, T = 128, every expert resident
+  C2  the same layer stack as configured for decode: cache rate 0.375 (24 of 64 experts per layer),
+      LRU, T in {1, 4, 16}: outputs against the oracle, residency and counters against the restated
+      reference cache logic (prefetcher.cpp:188-202, cache.cpp:248-312)
+  C4  Mixtral-8x7B layers (4096 x 14336, 8 experts, top-2 then softmax), cache rate 0.5, T = 1 and 64
+  C5  Qwen2-57B-A14B layer in q4_K with its sigmoid-gated shared expert of width 20480: three
+      single-token sequences (T = 3) at kernel level and the 3 + 512 mixed batch through moe_forward
+
+Expert weights are quantised once per module; the fp32 side of a check dequantises only the experts
+the batch activates.  Tolerance of the path: max |y - ref| <= 2e-2 max |ref|; routing bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from oracle import cache_oracle as CO
+from promoe_amd import layout as LY
+from tests.synth import LazyInt4Layer, Q4KLayer
+from tests.test_engine_gpu import build_engine
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def ref_forward_lazy(layer, x, k, mode):
+    lg = O.gate_logits_ordered(x, layer.wg)
+    if layer.bias is not None:
+        lg = (lg + layer.bias[None, :]).astype(np.float32)
+    idx, _ = O.topk_route(lg, k, mode)
+    experts = layer.experts_for(idx) if hasattr(layer, "experts_for") else layer.experts_fp32
+    return O.moe_forward(x, layer.wg, experts, k, mode, shared=layer.shared_fp32,
+                         shared_gate=getattr(layer, "shared_gate", None), logits=lg)
+
+
+def rel_err(y, ref):
+    return float(np.abs(y.float().cpu().numpy() - ref).max() / np.abs(ref).max())
+
+
+@pytest.fixture(scope="module")
+def deepseek_layers():
+    torch.set_num_threads(max(torch.get_num_threads(), 8))
+    return [LazyInt4Layer(H=2048, I=1408, E=64, I_sh=2816, seed=70 + l, zipf=1.2) for l in range(2)]
+
+
+def run_through_cache(pm, sim, layers, k, mode, schedule, cuda, H, seed0, check_counters=("hit", "miss", "evictions", "activated")):
+    Lyr, E = len(layers), layers[0].E
+    worst = 0.0
+    for step, T in enumerate(schedule):
+        for l in range(Lyr):
+            x = O.synth_acts(T, H, seed=seed0 + step * Lyr + l)
+            print(f"  step {step} layer {l} T={T}", flush=True)
+            y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            ref = ref_forward_lazy(layers[l], x, k, mode)
+            got_idx = pm.last_routing_idx(T, k)
+            assert np.array_equal(got_idx, ref["idx"]), (step, l, T)      # routing bit-exact
+            err = rel_err(y, ref["out"])
+            worst = max(worst, err)
+            assert err <= TOL, (step, l, T, err)
+            ids = sim.report_one_layer(l, np.unique(ref["idx"]))
+            for e in ids:
+                sim.wait_expert(l, e); sim.expert_launched(l, e)
+            sim.drain()
+            pm.drain()
+            assert [e for e in range(E) if pm.is_in_cache(l, e)] == sim.resident(l), (step, l)
+        for layer in layers:
+            layer.drop_cache()
+    c = pm.counters()
+    print(f"  worst max-rel-err {worst:.3e}; counters {c}", flush=True)
+    for key in check_counters:
+        assert c[key] == sim.ctr[key], (key, c[key], sim.ctr[key])
+    return worst, c
+
+
+def test_c2_decode_as_configured(cuda, deepseek_layers):
+    """cache rate 0.375, LRU, 64 experts of 2048 x 1408 per layer, T in {1, 4, 16}: the one-token path that
+    launches before the host knows the routing, the slot-group guard and the sequence-word release run at the
+    real expert count, top-k and width."""
+    print("case C2 decode as configured", flush=True)
+    layers, k = deepseek_layers, 6
+    Lyr, E = len(layers), 64
+    cfg = dict(cache_rate=0.375, cache_policy="lru", num_predict_expert_per_layer=0, reorder_experts=True,
+               early_preempt=True)
+    pm = build_engine(layers, k, cuda, max_tokens=16, **cfg)
+    assert pm.slot_info()[0] == CO.cache_len(0.375, Lyr, E) == 48
+    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy="lru", num_predict=0, reorder=True, early_preempt=True)
+    schedule = [1, 1, 4, 1, 16, 1, 1, 4, 16, 1, 1, 1]
+    worst, c = run_through_cache(pm, sim, layers, k, 0, schedule, cuda, 2048, 1000)
+    assert c["miss"] > 0 and c["hit"] > 0 and c["evictions"] > 0
+    assert c["h2d_bytes"] == c["miss"] * LY.int4_layout(2048, 1408)["total_bytes"]
+    pm.close()
+
+
+def test_c1_deepseek_layer_T128_all_resident(cuda, deepseek_layers):
+    """64 experts resident, 128 tokens (the reference's CPU-runnable configuration, here on the GPU kernels):
+    the token group takes the matrix-core tile kernels; also 64 tokens (the largest GEMV batch)."""
+    print("case C1 T=128 all resident", flush=True)
+    layer, k = deepseek_layers[0], 6
+    pm = build_engine([layer], k, cuda, max_tokens=128, cache_rate=1.0, cache_policy="lru")
+    pm.acquire_layer(0, np.arange(64, dtype=np.int64))
+    pm.release_layer(0)
+    c0 = pm.counters()
+    n_act = 0
+    for T in (128, 64, 128):
+        x = O.synth_acts(T, 2048, seed=1200 + T)
+        y = pm.forward(0, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+        torch.cuda.synchronize()
+        ref = ref_forward_lazy(layer, x, k, 0)
+        assert np.array_equal(pm.last_routing_idx(T, k), ref["idx"])
+        err = rel_err(y, ref["out"])
+        print(f"  T={T} max-rel-err {err:.3e}", flush=True)
+        assert err <= TOL
+        n_act += len(np.unique(ref["idx"]))
+    pm.drain()
+    c1 = pm.counters()
+    assert c1["miss"] == c0["miss"] and c1["hit"] - c0["hit"] == n_act
+    layer.drop_cache()
+    pm.close()
+
+
+def test_c4_mixtral_layers_through_cache(cuda):
+    """Two Mixtral-shaped layers (the second one holds the first one's experts in another order), cache rate
+    0.5 = 4 of 8 experts per layer in 91.5 MB slots, top-2 then softmax; T = 1 and 64."""
+    print("case C4 mixtral through cache", flush=True)
+    torch.set_num_threads(max(torch.get_num_threads(), 8))
+    H, I, E, k = 4096, 14336, 8, 2
+    l0 = LazyInt4Layer(H=H, I=I, E=E, seed=80)
+    l1 = LazyInt4Layer(H=H, I=I, E=E, seed=81, alias_of=l0, perm=[3, 5, 0, 7, 1, 6, 2, 4])
+    layers = [l0, l1]
+    cfg = dict(cache_rate=0.5, cache_policy="lru", num_predict_expert_per_layer=0, reorder_experts=True,
+               early_preempt=True)
+    pm = build_engine(layers, k, cuda, mode=2, max_tokens=64, **cfg)
+    assert pm.slot_info()[0] == CO.cache_len(0.5, 2, E) == 8
+    sim = CO.CacheSim(2, E, 6, k, cache_rate=0.5, policy="lru", num_predict=0, reorder=True, early_preempt=True)
+    worst, c = run_through_cache(pm, sim, layers, k, 2, [1, 1, 64, 1, 1, 64, 1], cuda, H, 1300)
+    assert c["miss"] > 0 and c["hit"] > 0 and c["evictions"] > 0
+    assert c["h2d_bytes"] == c["miss"] * LY.int4_layout(H, I)["total_bytes"]
+    pm.close()
+
+
+@pytest.fixture(scope="module")
+def qwen2_q4k_layer():
+    # the layer's real widths; 16 experts instead of 64 keep the host-side quantisation short
+    return Q4KLayer(H=3584, I=2560, E=16, I_sh=20480, seed=1, shared_gate=True, zipf=1.1)
+
+
+def test_c5_q4k_decode_three_sequences(cuda, qwen2_q4k_layer):
+    """T = 1 and T = 3 at kernel level: the shared expert's 20480-column w2 reduction leaves room for one
+    token row per pass in LDS, a path of its own in the q4_K GEMV."""
+    from tests.test_kernels_gpu import check_layer
+    print("case C5 q4_K decode, shared expert 20480 wide", flush=True)
+    for T in (1, 3):
+        check_layer(qwen2_q4k_layer, T, 8, 0, cuda, seed=40 + T)
+
+
+def test_c5_q4k_mixed_batch_through_forward(cuda, qwen2_q4k_layer):
+    """The configuration's 3 + 512 token batch through moe_forward behind the cache (half of the experts
+    resident: every expert is needed, so the call cycles the slots while it runs), then three tokens."""
+    print("case C5 q4_K 3+512 tokens through moe_forward", flush=True)
+    layer, k = qwen2_q4k_layer, 8
+    pm = build_engine([layer], k, cuda, max_tokens=515, cache_rate=0.5, cache_policy="lru")
+    sim = CO.CacheSim(1, 16, 1, k, cache_rate=0.5, policy="lru")
+    for step, T in enumerate((515, 3, 1)):
+        x = O.synth_acts(T, 3584, seed=1400 + step)
+        y = pm.forward(0, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+        torch.cuda.synchronize()
+        ref = ref_forward_lazy(layer, x, k, 0)
+        assert np.array_equal(pm.last_routing_idx(T, k), ref["idx"])
+        err = rel_err(y, ref["out"])
+        print(f"  T={T} max-rel-err {err:.3e}", flush=True)
+        assert err <= TOL, (T, err)
+        ids = sim.report_one_layer(0, np.unique(ref["idx"]))
+        for e in ids:
+            sim.wait_expert(0, e); sim.expert_launched(0, e)
+        sim.drain()
+        pm.drain()
+        assert [e for e in range(16) if pm.is_in_cache(0, e)] == sim.resident(0), step
+    c = pm.counters()
+    for key in ("hit", "miss", "evictions"):
+        assert c[key] == sim.ctr[key], key
+    assert c["miss"] > 0
+    pm.close()
+
+
+@pytest.mark.parametrize("policy", ["nn", "min", "static-1"])
+def test_other_policies_on_the_hip_backend(cuda, policy):
+    """NN, MIN and Static-1 victim selection with real copies underneath: residency and counters against the
+    restated reference policies (cache.hpp:81-126, cache.cpp:340-381, 490-583), outputs against the oracle."""
+    from tests.synth import Int4Layer
+    from tests.test_engine_gpu import ref_forward
+    print(f"case policy {policy} on the HIP backend", flush=True)
+    Lyr, E, k, H = 2, 16, 4, 256
+    layers = [Int4Layer(H=H, I=128, E=E, I_sh=128, seed=90 + l, zipf=1.2) for l in range(Lyr)]
+    n_steps = 14
+    # Belady's policy needs the recorded future: decode steps only, k experts per layer and step
+    tokens = (lambda s: 1) if policy == "min" else (lambda s: 1 if s % 4 else 5)
+    xs = [[O.synth_acts(tokens(s), H, seed=1500 + s * Lyr + l) for l in range(Lyr)] for s in range(n_steps)]
+    refs = [[ref_forward(layers[l], xs[s][l], k, 0) for l in range(Lyr)] for s in range(n_steps)]
+    cfg = dict(cache_rate=0.375, cache_policy=policy, num_predict_expert_per_layer=0)
+    pm = build_engine(layers, k, cuda, **cfg)
+    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy=policy, num_predict=0)
+    if policy == "min":
+        dec = np.array([[np.unique(refs[s][l]["idx"]) for l in range(Lyr)] for s in range(n_steps)], np.int32)
+        em = np.stack([np.zeros(n_steps, np.int64), np.arange(n_steps)], 1)
+        plen = np.zeros((1, Lyr), np.int32); psel = np.zeros((1, Lyr, 1), np.int32)
+        pm.load_oracle(em, plen, psel, dec)
+        sim.oracles = CO.load_oracle(Lyr, E, em, plen, psel, dec)
+        pm.set_cur_seq(0); sim.set_cur_seq(0)
+    for s in range(n_steps):
+        for l in range(Lyr):
+            y = pm.forward(l, torch.from_numpy(xs[s][l]).to(torch.bfloat16).to(cuda))
+            torch.cuda.synchronize()
+            assert rel_err(y, refs[s][l]["out"]) <= TOL, (s, l)
+            ids = sim.report_one_layer(l, np.unique(refs[s][l]["idx"]))
+            for e in ids:
+                sim.wait_expert(l, e); sim.expert_launched(l, e)
+            sim.layer_done(l)
+            sim.drain()
+            pm.drain()
+            assert [e for e in range(E) if pm.is_in_cache(l, e)] == sim.resident(l), (s, l)
+    c = pm.counters()
+    print(f"  counters {c}", flush=True)
+    for key in ("hit", "miss", "evictions"):
+        assert c[key] == sim.ctr[key], key
+    assert c["miss"] > 0 and c["evictions"] > 0
+    pm.close()
