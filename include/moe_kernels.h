@@ -171,6 +171,21 @@ int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k,
                           void *y_bf16, void *stream);
 
 
+/* moe_decode_token_int4 with phases = 5 (routing + w13 + SwiGLU, then w2 + combine into y_bf16 [H]) that
+ * allocates nothing and takes no workspace: the routing arrays, the h vectors and the resolved units live in
+ * a device array of moe_noalloc_scratch_bytes() (under 160 KiB) that is part of the library image; each GPU
+ * the library runs on holds its copy until the process ends.  No counterpart in the reference: it is for
+ * callers that cannot allocate or hand over workspaces (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  Inputs and outputs are the caller's: x, logits (E fp32), the slot table,
+ * the shared expert, y, and the error word err (device or pinned host memory, cleared by the caller; set to 1
+ * when a selected expert is not resident).  Limits: E <= 256, k <= 32, k*I + I_sh <= 71680 (what the
+ * fused w2 + combine kernel stages in LDS), H <= 16384; beyond them MOE_EINVAL.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered. */
+int64_t moe_noalloc_scratch_bytes(void);
+int moe_decode_token_int4_noalloc(const void *x_bf16, const float *logits, int E, int k, int mode, int H, int I,
+                                  int I_sh, const uint64_t *expert_ptr, const void *shared_ptr,
+                                  const float *shared_gate_logit, void *y_bf16, int *err, void *stream);
+
 /* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only. */
 int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, int k,
                            const moe_unit *units, int max_units, const int *sorted_tok,

@@ -2233,6 +2233,68 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   return launch_gemv_t<false>(a, grid, 1, I_sh > I ? I_sh : I, I / 128, s);
 }
 
+// ---------------------------------------------------------------------------
+// One token without any allocation: moe_decode_token_int4 with phases = 5 whose workspaces (routing
+// arrays, h vectors, resolved units) live in a file-scope device array instead of caller buffers.
+// Every GPU holds its own copy of the array at its own address until the process ends.
+// ---------------------------------------------------------------------------
+#define NOALLOC_MAX_E 256
+#define NOALLOC_MAX_K 32
+#define NOALLOC_MAX_H_ELEMS 71680   /* k*I + I_sh bf16 values: what the fused w2 + combine kernel can stage in LDS */
+struct NoAllocScratch {
+  int idx[NOALLOC_MAX_K];
+  float w[NOALLOC_MAX_K];
+  int counts[NOALLOC_MAX_E];
+  int offsets[NOALLOC_MAX_E + 1];
+  int sorted_pair[NOALLOC_MAX_K], pos_of_pair[NOALLOC_MAX_K], sorted_tok[NOALLOC_MAX_K];
+  int n_active, pad_[2];
+  moe_unit units[NOALLOC_MAX_K];
+  long long active_ids[NOALLOC_MAX_K];
+  unsigned char unit_ws[32 * NOALLOC_MAX_K];
+  uint16_t h[NOALLOC_MAX_H_ELEMS];   // h_r [k][I], then h_s [I_sh] at the next 16-byte boundary
+};
+static __device__ __align__(256) unsigned char scratch[sizeof(NoAllocScratch)];
+static_assert(sizeof(NoAllocScratch) <= 160 * 1024, "scratch array grew past its stated maximum");
+
+#define NOALLOC_MAX_DEVICES 64
+static NoAllocScratch *g_scratch_dev[NOALLOC_MAX_DEVICES];  // device address of `scratch` per GPU, set once
+
+extern "C" int64_t moe_noalloc_scratch_bytes(void) { return (int64_t)sizeof(NoAllocScratch); }
+
+extern "C" int moe_decode_token_int4_noalloc(const void *x, const float *logits, int E, int k, int mode, int H,
+                                             int I, int I_sh, const uint64_t *expert_ptr, const void *shared_ptr,
+                                             const float *shared_gate_logit, void *y_bf16, int *err, void *stream) {
+  if (!err || !y_bf16) { moe_set_error("moe_decode_token_int4_noalloc: y and err are required"); return MOE_EINVAL; }
+  if (E <= 0 || E > NOALLOC_MAX_E || k <= 0 || k > NOALLOC_MAX_K || I <= 0 || I_sh < 0 || I % 128 || I_sh % 128 ||
+      (size_t)k * I + (shared_ptr ? I_sh : 0) > NOALLOC_MAX_H_ELEMS) {
+    moe_set_error("moe_decode_token_int4_noalloc: shape beyond the static scratch (E=%d <= %d, k=%d <= %d, "
+                  "k*I + I_sh = %zu <= %d)", E, NOALLOC_MAX_E, k, NOALLOC_MAX_K,
+                  (size_t)k * I + (shared_ptr ? I_sh : 0), NOALLOC_MAX_H_ELEMS);
+    return MOE_EINVAL;
+  }
+  int dev = -1;
+  if (int rc = moe_check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) { moe_set_error("moe_decode_token_int4_noalloc: device %d not supported", dev); return MOE_EINVAL; }
+  NoAllocScratch *ws = __atomic_load_n(&g_scratch_dev[dev], __ATOMIC_ACQUIRE);
+  if (!ws) {
+    // the array's name is a host-side stand-in: ask the runtime where this device keeps it
+    void *p = nullptr;
+    if (int rc = moe_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+    if (!p) { moe_set_error("moe_decode_token_int4_noalloc: no device address for the scratch array"); return MOE_EHIP; }
+    ws = (NoAllocScratch *)p;
+    __atomic_store_n(&g_scratch_dev[dev], ws, __ATOMIC_RELEASE);
+  }
+  uint16_t *h_r = ws->h;
+  uint16_t *h_s = ws->h + (((size_t)k * I + 7) & ~(size_t)7);
+  // phases 5 never touches the partial-row buffers; the entry point it shares wants them non-null
+  float *unused_part = (float *)ws->h;
+  return moe_decode_token_int4(x, logits, E, k, mode, H, I, I_sh, expert_ptr, shared_ptr, ws->idx, ws->w, ws->counts,
+                               ws->offsets, ws->sorted_pair, ws->pos_of_pair, ws->sorted_tok, ws->units, &ws->n_active,
+                               (int64_t *)ws->active_ids, h_r, shared_ptr ? h_s : nullptr, unused_part,
+                               shared_ptr ? unused_part : nullptr, err, ws->unit_ws, nullptr, nullptr, 0, 5,
+                               shared_gate_logit, y_bf16, stream);
+}
+
 extern "C" int moe_q4k_layout_make(int H, int I, moe_int4_layout *out) {
   if (!out || H <= 0 || I <= 0 || H % 256 || I % 256) {
     moe_set_error("moe_q4k_layout_make: H and I must be positive multiples of 256 (H=%d I=%d)", H, I);

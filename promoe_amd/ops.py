@@ -160,6 +160,17 @@ def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, 
     return idx, w, d, part_r, part_s, err, h_r, h_s
 
 
+def decode_token_int4_noalloc(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int,
+                              y, err, sg_logit=None):
+    """One token, routing to y in two launches, with every workspace in the library's static device array:
+    nothing is allocated here or in the library (x, logits, y and err are the caller's)."""
+    check(lib.moe_decode_token_int4_noalloc(ptr(_dev(x)), ptr(logits), E, k, mode, H, I,
+                                            I_sh if shared is not None else 0, ptr(expert_ptr), ptr(shared),
+                                            ptr(sg_logit), ptr(y), ptr(err), cur_stream()),
+          "moe_decode_token_int4_noalloc")
+    return y
+
+
 def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
                        H: int, I: int, I_sh: int, phases: int = 3, ws=None):
     """q4_K flavour of experts_decode_int4 (device-side unit list)."""
