@@ -346,6 +346,45 @@ def quantize_q4k(w: np.ndarray) -> np.ndarray:
 
 
 # --------------------------------------------------------------------------
+# q6_K (ggml block_q6_K): 256 weights per block, 210 bytes: ql[128] (low 4 bits), qh[64] (high 2 bits),
+# int8 scales[16] (one per 16 weights), fp16 d.   w = d * scale * (q - 32), q in 0..63.
+# Not in the reference tree (it names the q4_k_m file type, README.md:29-34, whose ffn_down tensors
+# llama.cpp stores as Q6_K); restated from ggml's published dequantize_row_q6_K, loop for loop.
+Q6K_BYTES = 210
+
+
+def dequant_q6k_block(blk: np.ndarray) -> np.ndarray:
+    """One 210-byte block -> 256 fp32 weights (plain loops on purpose)."""
+    blk = np.asarray(blk, np.uint8)
+    ql, qh = blk[0:128].astype(np.int32), blk[128:192].astype(np.int32)
+    sc = blk[192:208].view(np.int8).astype(np.int32)
+    d = np.float32(blk[208:210].view(np.float16)[0])
+    y = np.zeros(256, np.float32)
+    for half in range(2):                       # 128 weights per half
+        qlh, qhh, sch, yo = ql[64 * half:], qh[32 * half:], sc[8 * half:], 128 * half
+        for l in range(32):
+            i_s = l // 16
+            q1 = ((qlh[l] & 0xF) | (((qhh[l] >> 0) & 3) << 4)) - 32
+            q2 = ((qlh[l + 32] & 0xF) | (((qhh[l] >> 2) & 3) << 4)) - 32
+            q3 = ((qlh[l] >> 4) | (((qhh[l] >> 4) & 3) << 4)) - 32
+            q4 = ((qlh[l + 32] >> 4) | (((qhh[l] >> 6) & 3) << 4)) - 32
+            y[yo + l] = d * np.float32(sch[i_s + 0]) * np.float32(q1)
+            y[yo + l + 32] = d * np.float32(sch[i_s + 2]) * np.float32(q2)
+            y[yo + l + 64] = d * np.float32(sch[i_s + 4]) * np.float32(q3)
+            y[yo + l + 96] = d * np.float32(sch[i_s + 6]) * np.float32(q4)
+    return y
+
+
+def dequant_q6k(blocks: np.ndarray, N: int, K: int) -> np.ndarray:
+    blocks = np.asarray(blocks, np.uint8).reshape(N, K // QK_K, Q6K_BYTES)
+    out = np.zeros((N, K), np.float32)
+    for n in range(N):
+        for b in range(K // QK_K):
+            out[n, b * QK_K:(b + 1) * QK_K] = dequant_q6k_block(blocks[n, b])
+    return out
+
+
+# --------------------------------------------------------------------------
 # k3/k4 expert product, k5 combine, whole-layer forward (HF structure)
 # --------------------------------------------------------------------------
 

@@ -1,0 +1,98 @@
+// Device-side helpers shared by the kernel sources (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "moe_kernels.h"
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int u32;
+
+// ---------------------------------------------------------------------------
+// small device helpers
+// ---------------------------------------------------------------------------
+static __device__ __forceinline__ float bf16lo(u32 v) { return __uint_as_float(v << 16); }
+static __device__ __forceinline__ float bf16hi(u32 v) { return __uint_as_float(v & 0xffff0000u); }
+static __device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even
+  u32 u = __float_as_uint(f);
+  u32 r = ((u >> 16) & 1u) + 0x7fffu;
+  return (uint16_t)((u + r) >> 16);
+}
+static __device__ __forceinline__ float dot2bf(u32 a, u32 b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a),
+                                         __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
+static __device__ __forceinline__ rsrc_t make_rsrc(const void *p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
+}
+// A unit list for the host: stores with both scope bits set go past the caches straight to the pinned
+// host buffer; once they have completed (host_stores_done) the sequence word the host polls may follow.
+// No cache write-back or invalidate is involved, unlike a system-scope fence.
+static __device__ __forceinline__ void host_store_unit(moe_unit *dst, int i, int expert, int m, int row0) {
+  const u32x4_t v = {(u32)expert, (u32)m, (u32)row0, 0u};
+  __builtin_amdgcn_raw_buffer_store_b128(v, make_rsrc(dst, 0x7fffffffu), i * 16, 0, 17 /* sc0 | sc1 */);
+}
+static __device__ __forceinline__ void host_store_i32(int *dst, int v) {
+  __builtin_amdgcn_raw_buffer_store_b32((u32)v, make_rsrc(dst, 0x7fffffffu), 0, 0, 17);
+}
+static __device__ __forceinline__ void host_stores_done() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);  // every outstanding memory operation of this wave has completed
+}
+static __device__ __forceinline__ float half_bits_to_f32(uint16_t h) {
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+// 8 int4 weights (interleaved nibble order) x 8 bf16 activations; the weights
+// enter as the exact bf16 values 128+q (0x4300 | q), the caller removes 128*sum(x).
+static __device__ __forceinline__ float dot8_q4(u32 w, const uint4 &x, float acc) {
+  const u32 M = 0x000f000fu, C = 0x43004300u;
+  acc = dot2bf((w & M) | C, x.x, acc);
+  acc = dot2bf(((w >> 4) & M) | C, x.y, acc);
+  acc = dot2bf(((w >> 8) & M) | C, x.z, acc);
+  acc = dot2bf(((w >> 12) & M) | C, x.w, acc);
+  return acc;
+}
+
+// maximum over the 64 lanes of a wave, built from DPP row shifts and broadcasts (no LDS traffic)
+static __device__ __forceinline__ float wave_max_f32(float x) {
+  // inclusive max-scan inside each row of 16 lanes, then rows 0->1, 2->3, then 1->3: lane 63 holds the result
+#define WMAX_STEP(ctrl, rmask)                                                                          \
+  {                                                                                                     \
+    const int xi = __builtin_bit_cast(int, x);                                                          \
+    x = fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, ctrl, rmask, 0xf, false))); \
+  }
+  WMAX_STEP(0x111, 0xf)  // row_shr:1
+  WMAX_STEP(0x112, 0xf)  // row_shr:2
+  WMAX_STEP(0x114, 0xf)  // row_shr:4
+  WMAX_STEP(0x118, 0xf)  // row_shr:8
+  WMAX_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+  WMAX_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef WMAX_STEP
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
+// global-address-space loads (pointers that come out of the slot table are generic
+// to the compiler and would otherwise become flat_load)
+typedef __attribute__((address_space(1))) const u32x4_t g_uint4;
+typedef __attribute__((address_space(1))) const unsigned int g_u32;
+static __device__ __forceinline__ uint4 ldg_u4(const void *p) {
+  const u32x4_t v = *(g_uint4 *)(unsigned long long)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+static __device__ __forceinline__ u32 ldg_u32(const void *p) { return *(g_u32 *)(unsigned long long)p; }
+static __device__ __forceinline__ float sum8_bf16(const uint4 &v) {
+  return bf16lo(v.x) + bf16hi(v.x) + bf16lo(v.y) + bf16hi(v.y) + bf16lo(v.z) + bf16hi(v.z) + bf16lo(v.w) +
+         bf16hi(v.w);
+}
+
+static __device__ __forceinline__ uint4 bload16(rsrc_t r, int voff, int soff) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+static __device__ __forceinline__ u32 bload4(rsrc_t r, int voff, int soff) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+

@@ -270,6 +270,34 @@ class GGUFFile:
         shape = tuple(reversed(ne[1:])) + (ne[0] // 256, 144)
         return self.raw(name).reshape(shape)
 
+    def q6k_blocks(self, name) -> np.ndarray:
+        """uint8 view [..., ne1, ne0/256, 210] (outermost dimension first) of a Q6_K tensor."""
+        ne, typ, _ = self.tensors[name]
+        if typ != GGML_Q6_K:
+            raise NotImplementedError("%s is stored as %s, not Q6_K" % (name, _GGML_NAME.get(typ, str(typ))))
+        if ne[0] % 256:
+            raise ValueError("%s: row length %d is not a multiple of 256" % (name, ne[0]))
+        shape = tuple(reversed(ne[1:])) + (ne[0] // 256, 210)
+        return self.raw(name).reshape(shape)
+
+    def expert_q4k_blocks(self, name) -> np.ndarray:
+        """An expert tensor as q4_K blocks [..., rows, cols/256, 144].  Q4_K tensors are handed out as they
+        are.  Q6_K tensors (the ffn_down tensors of a q4_k_m file) are dequantised and quantised again to
+        q4_K, the one block format the expert kernels read: a lossy step (a weight moves by at most half a
+        q4_K step of its 32-wide sub-block), so the result is not what llama.cpp computes from the file."""
+        typ = self.tensors[name][1]
+        if typ == GGML_Q4_K:
+            return self.q4k_blocks(name)
+        if typ == GGML_Q6_K:
+            from .quant import dequant_q6k, quantize_q4k
+            b6 = self.q6k_blocks(name)
+            w = dequant_q6k(b6)                               # [..., rows, cols]
+            lead = w.shape[:-2]
+            q = quantize_q4k(w.reshape(-1, w.shape[-1]))
+            return q.reshape(lead + (w.shape[-2], w.shape[-1] // 256, 144))
+        raise NotImplementedError("%s is stored as %s; expert tensors must be Q4_K or Q6_K"
+                                  % (name, _GGML_NAME.get(typ, str(typ))))
+
     def dense(self, name) -> np.ndarray:
         """fp32 array (outermost dimension first) of an F32 / F16 / BF16 tensor."""
         ne, typ, _ = self.tensors[name]
@@ -296,7 +324,7 @@ def gguf_layer_images(g: GGUFFile, layer: int):
     p = "blk.%d." % layer
     gate = g.q4k_blocks(p + "ffn_gate_exps.weight")      # [E, I, H/256, 144]
     up = g.q4k_blocks(p + "ffn_up_exps.weight")
-    down = g.q4k_blocks(p + "ffn_down_exps.weight")      # [E, H, I/256, 144]
+    down = g.expert_q4k_blocks(p + "ffn_down_exps.weight")   # [E, H, I/256, 144]; Q6_K in a q4_k_m file
     E, I, H = gate.shape[0], gate.shape[1], gate.shape[2] * 256
     if up.shape != gate.shape or down.shape != (E, H, I // 256, 144):
         raise ValueError("expert tensors of block %d disagree in shape" % layer)
@@ -306,7 +334,7 @@ def gguf_layer_images(g: GGUFFile, layer: int):
     if (p + "ffn_gate_shexp.weight") in g.tensors:
         sg = g.q4k_blocks(p + "ffn_gate_shexp.weight")   # [I_sh, H/256, 144]
         su = g.q4k_blocks(p + "ffn_up_shexp.weight")
-        sd = g.q4k_blocks(p + "ffn_down_shexp.weight")
+        sd = g.expert_q4k_blocks(p + "ffn_down_shexp.weight")
         out["I_sh"] = sg.shape[0]
         out["shared"] = LY.pack_expert_q4k(sg, su, sd, H, sg.shape[0])
         if (p + "ffn_gate_inp_shexp.weight") in g.tensors:

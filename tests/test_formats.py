@@ -202,3 +202,85 @@ def test_gguf_rejects_bad_files(tmp_path):
     p.write_bytes(b"GGUF" + struct.pack("<IQQ", 3, 1, 0) + struct.pack("<Q", 1000))
     with pytest.raises(ValueError, match="truncated"):
         F.GGUFFile(str(p))
+
+
+# ---- Q6_K (the ffn_down tensors of a q4_k_m file) ---------------------------------------------
+
+def _random_q6k_blocks(rng, shape):
+    b = rng.integers(0, 256, shape + (210,), dtype=np.uint8)
+    b[..., 192:208] = rng.integers(-60, 61, shape + (16,), dtype=np.int8).view(np.uint8)
+    d = (rng.random(shape) * 2e-5 + 1e-5).astype(np.float16)
+    b[..., 208:210] = d[..., None].view(np.uint8).reshape(shape + (2,))
+    return b
+
+
+def test_oracle_q6k_known_answers():
+    """The loop restatement against the closed form of the layout: weight i of a block has scale i // 16,
+    low nibble in ql[64 h + 32 (j & 1) + l] (high nibble for j >= 2) and its two high bits at bit 2 j of
+    qh[32 h + l], with h = i // 128, j = (i % 128) // 32, l = i % 32; w = d * scale * (q - 32)."""
+    blk = np.zeros(210, np.uint8)
+    blk[192:208] = np.ones(16, np.int8).view(np.uint8)
+    blk[208:210] = np.array([1.0], np.float16).view(np.uint8)
+    assert np.array_equal(O.dequant_q6k_block(blk), np.full(256, -32.0, np.float32))     # q = 0 everywhere
+    one = blk.copy(); one[0] = 0x0F; one[128] = 0x03                                       # weight 0: q = 63
+    y = O.dequant_q6k_block(one)
+    assert y[0] == 31.0 and np.all(np.delete(y, 0) == -32.0)
+    hi = blk.copy(); hi[64 + 32 + 5] = 0x70; hi[128 + 32 + 5] = 0x80                       # h=1, j=3, l=5: q = 7 | 2<<4
+    y = O.dequant_q6k_block(hi)
+    assert y[128 + 96 + 5] == float((7 | (2 << 4)) - 32) and np.sum(y != -32.0) == 1
+    rng = np.random.default_rng(11)
+    for _ in range(4):
+        b = _random_q6k_blocks(rng, ())
+        ql, qh = b[0:128].astype(int), b[128:192].astype(int)
+        sc = b[192:208].view(np.int8).astype(np.float32)
+        d = np.float32(b[208:210].view(np.float16)[0])
+        want = np.zeros(256, np.float32)
+        for i in range(256):
+            h, j, l = i // 128, (i % 128) // 32, i % 32
+            byte = ql[64 * h + 32 * (j & 1) + l]
+            q = ((byte >> 4) if j >= 2 else (byte & 0xF)) | (((qh[32 * h + l] >> (2 * j)) & 3) << 4)
+            want[i] = d * sc[i // 16] * np.float32(q - 32)
+        assert np.array_equal(O.dequant_q6k_block(b), want)
+
+
+def test_product_q6k_and_q4k_quantiser_match_the_oracle():
+    from promoe_amd import quant as Q
+    rng = np.random.default_rng(12)
+    b = _random_q6k_blocks(rng, (3, 5, 2))                      # [E, rows, blocks per row]
+    got = Q.dequant_q6k(b)
+    assert got.shape == (3, 5, 512)
+    for e in range(3):
+        assert np.array_equal(got[e], O.dequant_q6k(b[e], 5, 512))
+    w = rng.normal(0, 0.02, (16, 512)).astype(np.float32)
+    w[3, 32:64] = 0.0
+    assert np.array_equal(Q.quantize_q4k(w), O.quantize_q4k(w))
+
+
+def test_gguf_q6k_down_tensors_are_requantised(tmp_path):
+    """A q4_k_m-style layer: gate / up in Q4_K, down in Q6_K.  The down tensors reach the slot image as q4_K
+    blocks made from their exact Q6_K values; the step is lossy and its size is checked."""
+    rng = np.random.default_rng(13)
+    H, I, E = 256, 512, 2
+    gate = np.stack([O.quantize_q4k(rng.normal(0, 0.02, (I, H)).astype(np.float32)) for _ in range(E)])
+    up = np.stack([O.quantize_q4k(rng.normal(0, 0.02, (I, H)).astype(np.float32)) for _ in range(E)])
+    down6 = _random_q6k_blocks(rng, (E, H, I // 256))
+    wg = rng.normal(0, 0.02, (E, H)).astype(np.float32)
+    tensors = [("blk.0.ffn_gate_inp.weight", (H, E), F.GGML_F32, wg.tobytes()),
+               ("blk.0.ffn_gate_exps.weight", (H, I, E), F.GGML_Q4_K, gate.tobytes()),
+               ("blk.0.ffn_up_exps.weight", (H, I, E), F.GGML_Q4_K, up.tobytes()),
+               ("blk.0.ffn_down_exps.weight", (I, H, E), F.GGML_Q6_K, down6.tobytes())]
+    path = str(tmp_path / "q4km.gguf")
+    _write_gguf(path, {"general.architecture": (8, "qwen2moe")}, tensors)
+    g = F.GGUFFile(path)
+    lay = F.gguf_layer_images(g, 0)
+    for e in range(E):
+        exact = O.dequant_q6k(down6[e], H, I)                    # what the file says
+        q4 = O.quantize_q4k(exact)
+        assert np.array_equal(lay["routed"][e], LY.pack_expert_q4k(gate[e], up[e], q4, H, I))
+        back = O.dequant_q4k(q4, H, I)
+        rms = float(np.sqrt(np.mean((back - exact) ** 2)) / np.sqrt(np.mean(exact ** 2)))
+        assert rms < 0.12, rms
+    with pytest.raises(NotImplementedError, match="Q4_K or Q6_K"):
+        bad = str(tmp_path / "bad.gguf")
+        _write_gguf(bad, {}, [("blk.0.ffn_down_exps.weight", (256, 4, 1), 8, bytes(34 * 32))])
+        F.GGUFFile(bad).expert_q4k_blocks("blk.0.ffn_down_exps.weight")
