@@ -10,8 +10,13 @@ and the experts' weights live in pinned host memory as slot images instead of mo
 
 Works on the stock `transformers` sparse blocks that keep their experts in fused tensors
 (`experts.gate_up_proj [E, 2I, H]`, `experts.down_proj [E, H, I]`, `gate.weight [E, H]`):
-Qwen2-MoE (softmax -> top-k, optional renormalisation, sigmoid-gated shared expert) and Mixtral
-(softmax -> top-k -> renormalise, which is the softmax over the selected logits).
+Qwen2-MoE (softmax -> top-k, optional renormalisation, sigmoid-gated shared expert), Mixtral
+(softmax -> top-k -> renormalise, which is the softmax over the selected logits) and the DeepSeek
+family (DeepSeek-MoE / DeepSeek-V2-Lite: softmax -> greedy top-k without renormalisation, a plain
+shared expert `shared_experts` of n_shared_experts * I columns; the reference's metas for it are
+utils/common_metas.py:17-41 and 69-94).  In the DeepSeek models the first decoder layers are dense:
+MoE layers are numbered from 0 in model order, so decoder layer i is engine layer
+i - first_k_dense_replace (the reference subtracts the same 1, common_metas.py:19-23).
 """
 from __future__ import annotations
 
@@ -40,9 +45,19 @@ def find_moe_blocks(model):
 
 def _route_mode(block) -> int:
     gate = block.gate
+    if hasattr(gate, "topk_method"):                         # DeepSeek router
+        if gate.topk_method != "greedy":
+            raise NotImplementedError("DeepSeek routing method %r (only 'greedy' top-k is supported)" % gate.topk_method)
+        return L.ROUTE_SOFTMAX_TOPK
     if hasattr(gate, "norm_topk_prob"):                      # Qwen2-MoE router
         return L.ROUTE_SOFTMAX_TOPK_RENORM if gate.norm_topk_prob else L.ROUTE_SOFTMAX_TOPK
     return L.ROUTE_TOPK_SOFTMAX                              # Mixtral: renormalised top-k of the softmax
+
+
+def _shared_expert(block):
+    """The block's always-on expert: Qwen2-MoE calls it shared_expert, the DeepSeek family shared_experts."""
+    sh = getattr(block, "shared_expert", None)
+    return sh if sh is not None else getattr(block, "shared_experts", None)
 
 
 def _bf16_bits(t: torch.Tensor) -> np.ndarray:
@@ -76,7 +91,7 @@ def inject_model(model, device="cuda:0", fmt: str = "bf16", max_tokens: int = 40
     E, two_i, H = b0.experts.gate_up_proj.shape
     I = two_i // 2
     top_k = int(getattr(b0.gate, "top_k", getattr(b0, "top_k", 0)))
-    sh0 = getattr(b0, "shared_expert", None)
+    sh0 = _shared_expert(b0)
     I_sh = sh0.gate_proj.weight.shape[0] if sh0 is not None else 0
     total = LY.bf16_expert_bytes(H, I) if fmt == "bf16" else LY.int4_layout(H, I)["total_bytes"]
     chunks = [("w", 0, total)] if fmt == "bf16" else LY.split_chunks_int4(H, I)
@@ -94,11 +109,13 @@ def inject_model(model, device="cuda:0", fmt: str = "bf16", max_tokens: int = 40
         gu, dn = blk.experts.gate_up_proj, blk.experts.down_proj
         if tuple(gu.shape) != (E, 2 * I, H) or tuple(dn.shape) != (E, H, I):
             raise ValueError("block %s differs in shape from the first block" % name)
+        # DeepSeek scales the routed experts' sum by a constant; it goes into their down projections
+        scale = float(getattr(blk.gate, "routed_scaling_factor", 1.0) or 1.0)
         for e in range(E):
-            img = _expert_image(gu[e, :I], gu[e, I:], dn[e], H, I, fmt)
+            img = _expert_image(gu[e, :I], gu[e, I:], dn[e] if scale == 1.0 else dn[e] * scale, H, I, fmt)
             base = (l * E + e) * total
             stage.array[base: base + total] = img
-        sh = getattr(blk, "shared_expert", None)
+        sh = _shared_expert(blk)
         shared_imgs.append(None if sh is None else
                            _expert_image(sh.gate_proj.weight, sh.up_proj.weight, sh.down_proj.weight, H, I_sh, fmt))
         if drop_expert_params:      # the experts no longer live in the module (nor, later, on the device)

@@ -102,10 +102,26 @@ def oracle_tensors(trace: dict, n_layer: int, top_k: int, max_new_tokens: int | 
     return em, plen, psel, ds
 
 
+def expert_pattern(layer: int, expert: int, n_expert: int, nbytes: int) -> np.ndarray:
+    """The bytes the replay gives expert (layer, expert) on the HIP backend: distinct per expert, never zero."""
+    rng = np.random.default_rng(1000003 * layer + expert)
+    return rng.integers(1, 256, nbytes, dtype=np.uint8)
+
+
 def replay(trace: dict, n_layer: int, n_expert: int, top_k: int, max_new_tokens: int | None = None,
-           skip_first_prompts: int = 0, **cfg) -> dict:
+           skip_first_prompts: int = 0, backend: int = L.BACKEND_HOST, expert_bytes: int = 64, on_expert=None,
+           **cfg) -> dict:
     """One configuration: every sequence of the trace through a fresh engine; returns the engine's
-    report (per-stage hit / ready / prefetch-hit counts and rates) plus its raw counters."""
+    report (per-stage hit / ready / prefetch-hit counts and rates) plus its raw counters.
+
+    backend L.BACKEND_HOST (default): no GPU, copies are memcpy's, the experts carry no weights (the
+    reference's stand-in model, whose experts do nothing).  L.BACKEND_HIP: the same hook sequence with
+    real slots in HBM and real copies from pinned host memory on the copy stream; every expert holds
+    expert_pattern(...) of expert_bytes bytes.  on_expert(pm, layer, expert) is called between
+    report_one_expert and one_expert_done, when the expert's slot must hold its bytes."""
+    if backend == L.BACKEND_HIP:
+        return _replay_hip(trace, n_layer, n_expert, top_k, max_new_tokens, skip_first_prompts, expert_bytes,
+                           on_expert, cfg)
     m = ModuleMeta(n_layer, n_expert)
     m.init_param_list(["w"])
     d = {"num_expert_per_token": str(top_k)}
@@ -123,22 +139,54 @@ def replay(trace: dict, n_layer: int, n_expert: int, top_k: int, max_new_tokens:
     pm.init_gpu_mem_buffer()
     pm.launch_thread()
     try:
-        if str(cfg.get("cache_policy", "")).lower() == "min":
-            pm.load_oracle(*oracle_tensors(trace, n_layer, top_k, max_new_tokens))
-        for si, s in enumerate(sorted(trace, key=int)):
-            pm.set_cur_seq(si)
-            for seq_len, layers in sequence_forwards(trace[s], n_layer, max_new_tokens):
-                pm.report_moe_layer_logits(0, None, seq_len=seq_len)
-                for l, ids in enumerate(layers):
-                    order = pm.report_one_layer(l, np.asarray(ids, np.int64))
-                    for e in order:
-                        pm.report_one_expert(l, int(e))
-                        pm.one_expert_done(l, int(e))
-                    pm.one_moe_layer_done(l)
-        pm.drain()
-        out = pm.report(skip_first_prompts)
-        out.update({"counter_" + k: v for k, v in pm.counters().items()})
-        return out
+        return _drive(pm, trace, n_layer, top_k, max_new_tokens, skip_first_prompts, on_expert, cfg)
+    finally:
+        pm.close()
+
+
+def _drive(pm, trace, n_layer, top_k, max_new_tokens, skip_first_prompts, on_expert, cfg) -> dict:
+    """The hook sequence of the reference's stand-in model, forward by forward
+    (transformers-deepseek-moe.py:36-49 inside :66-88)."""
+    if str(cfg.get("cache_policy", "")).lower() == "min":
+        pm.load_oracle(*oracle_tensors(trace, n_layer, top_k, max_new_tokens))
+    for si, s in enumerate(sorted(trace, key=int)):
+        pm.set_cur_seq(si)
+        for seq_len, layers in sequence_forwards(trace[s], n_layer, max_new_tokens):
+            pm.report_moe_layer_logits(0, None, seq_len=seq_len)
+            for l, ids in enumerate(layers):
+                order = pm.report_one_layer(l, np.asarray(ids, np.int64))
+                for e in order:
+                    pm.report_one_expert(l, int(e))
+                    if on_expert is not None:
+                        on_expert(pm, l, int(e))
+                    pm.one_expert_done(l, int(e))
+                pm.one_moe_layer_done(l)
+    pm.drain()
+    out = pm.report(skip_first_prompts)
+    out.update({"counter_" + k: v for k, v in pm.counters().items()})
+    return out
+
+
+def _replay_hip(trace, n_layer, n_expert, top_k, max_new_tokens, skip_first_prompts, expert_bytes, on_expert, cfg):
+    from .engine import PinnedBuffer
+    m = ModuleMeta(n_layer, n_expert)
+    m.init_param_list(["w"])
+    d = {"num_expert_per_token": str(top_k)}
+    d.update({a: str(b) for a, b in cfg.items()})
+    m.init_from_map(d)
+    m.handle_uninited_configs()
+    pm = PrefetchMngr(m, backend=L.BACKEND_HIP, compute_stream=0)   # the engine makes its own compute stream
+    stage = PinnedBuffer(expert_bytes * n_layer * n_expert)
+    pm._keep.append(stage)
+    for l in range(n_layer):
+        for e in range(n_expert):
+            base = (l * n_expert + e) * expert_bytes
+            stage.array[base: base + expert_bytes] = expert_pattern(l, e, n_expert, expert_bytes)
+            pm.add_one_expert_param(stage.array[base: base + expert_bytes], l, e, "w")
+    pm.init_gpu_mem_buffer()
+    pm.launch_thread()
+    try:
+        return _drive(pm, trace, n_layer, top_k, max_new_tokens, skip_first_prompts, on_expert, cfg)
     finally:
         pm.close()
 
