@@ -68,7 +68,38 @@ def kernel_times(lib):
     return out
 
 
-def cpu_baseline(T, H, I, E, I_sh, k, threads):
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "hbm_traffic_decode_T1_and_prefill_qwen.md")
+KERNEL_SOURCES = ["promoe_amd/csrc/moe_kernels.hip", "promoe_amd/csrc/moe_device.h"]
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    root = os.path.dirname(os.path.abspath(__file__))
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(root, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic():
+    """HBM bytes per launch of the T=1 w13 kernel as recorded in the committed counter summary (lines
+    `decode_w13_traffic_bytes_per_launch: N` and `decode_kernel_source_sha256_16: H`); None when the summary
+    is missing or was measured on other kernel sources than the ones in the tree."""
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    import re
+    m = re.search(r"decode_w13_traffic_bytes_per_launch:\s*(\d+)", text)
+    hsh = re.search(r"decode_kernel_source_sha256_16:\s*([0-9a-f]{16})", text)
+    if not m or not hsh or hsh.group(1) != kernel_source_hash():
+        return None
+    return int(m.group(1))
+
+
+def cpu_baseline(T, H, I, E, I_sh, k, threads, budget_s=12.0):
     """The oracle's fp32 forward in the reference's structure (per-expert loop), on host cores."""
     import numpy as np
     import torch
@@ -84,14 +115,14 @@ def cpu_baseline(T, H, I, E, I_sh, k, threads):
     times = []
     t_begin = time.perf_counter()
     rep = 0
-    while rep < 7 or (time.perf_counter() - t_begin < 12.0 and rep < 5000):
+    while rep < 5 or (time.perf_counter() - t_begin < budget_s and rep < 5000):
         x = O.synth_acts(T, H, seed=rep + 1)
         t0 = time.perf_counter()
         lg = (O.gate_logits(x, wg) + bias[None, :]).astype(np.float32)
         O.moe_forward(x, wg, experts, k, 0, shared=shared, logits=lg)
         times.append(time.perf_counter() - t0)
         rep += 1
-    steady = times[2:]
+    steady = times[2:] if len(times) > 4 else times[1:]
     return T * len(steady) / sum(steady), statistics.median(steady), len(steady)
 
 
@@ -330,10 +361,21 @@ def main():
         timed_steps(pm, xs, L_, warmup, torch)
         return timed_steps(pm, xs, L_, steps, torch)
 
-    dt = run(T, a.steps, a.warmup)
+    # `value`: median over repeats of a timed region of at least --steps steps and at least 0.2 s (a 20-step
+    # region is 0.4 ms of wall clock: one scheduler hiccup on the host moves it by 10 %)
+    dt_probe = run(T, a.steps, a.warmup)
+    n_timed = max(a.steps, int(0.2 / max(dt_probe / a.steps, 1e-7)) + 1)
+    n_timed = (n_timed + L_ - 1) // L_ * L_                 # whole passes over the layer stack
+    xs_v = stack.acts(T, 8, seed=1)
+    xs_out = torch.empty_like(xs_v[0])
+    reps = sorted(timed_steps(pm, xs_v, L_, n_timed, torch) for _ in range(5))
+    dt = reps[len(reps) // 2] * a.steps / n_timed           # per --steps steps, from the median repeat
     c1 = pm.counters()
     assert c1["miss"] == base_ctr["miss"], "steady-state run took cache misses"
     value = T * a.steps / dt
+    timing = {"timed_steps_per_repeat": n_timed, "repeats": len(reps), "statistic": "median",
+              "ms_per_step_min": reps[0] / n_timed * 1e3, "ms_per_step_max": reps[-1] / n_timed * 1e3,
+              "first_region_of_exactly_steps_ms_per_step": dt_probe / a.steps * 1e3}
 
     # per-kernel durations (HIP event pairs around every launch), separate short pass; an
     # event pair adds about 2-3 us to a launch, so these are upper bounds
@@ -400,8 +442,9 @@ def main():
                 "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this kernel at this
-                # workload (T=1, 27 layers), scaled by a copy kernel of known size; not measurable in-process
-                "traffic": 24245555 if (T == 1 and L_ == 27) else None,
+                # workload (T=1, 27 layers), scaled by a copy kernel of known size; not measurable in-process:
+                # read from the committed counter summary, null when the kernel sources changed since
+                "traffic": recorded_traffic() if (T == 1 and L_ == 27) else None,
                 "algorithmic_bytes_per_launch": w13_bytes_k, "avg_launch_us": w13_us,
                 "distinct_routed_experts_per_launch": D_k,
                 "method": "%d back-to-back launches between one HIP event pair" % n_k}
@@ -422,46 +465,70 @@ def main():
 
     # ---- the configured cache rate: 24 of 64 experts per layer resident, LRU ------------
     cache_run = None
+    as_configured = None
     if not a.no_cache_run:
-        def cache_leg(predict):
+        def cache_leg(Tn, predict=None):
+            """predict: None (demand fetching only), "exact" (every layer of a token sees one hidden state, so the
+            gate-as-predictor is always right: what prefetching can hide at best) or "drifting" (the hidden state
+            of a token drifts from layer to layer, x_l+1 = x_l + 0.5 noise: predictions made from an earlier
+            layer's input are sometimes wrong, as with a real model)."""
             cfg = dict(cache_rate=0.375, cache_policy="lru", reorder_experts=True, early_preempt=True,
                        num_predict_expert_per_layer=k if predict else 0)
             if predict:
                 cfg.update(layer_predict_interval=1, layer_predict_max_window=10, limit_layer_0_window=10)
             pm2 = stack.engine(16, **cfg)
             if predict:
-                # the built-in predictor with the destination layer's gate as the model of every pair; this
-                # bench feeds ONE hidden state to all layers of a token, so these predictions are exact: what
-                # prefetching can hide when the predictor is right
+                # the built-in predictor with the destination layer's gate as the model of every pair
                 for src, (f0, f1) in enumerate(pm2.predictor_windows()):
                     for dst in range(f0, f1):
                         pm2.set_predictor_model(src, dst, stack.gate_w[dst], stack.gate_bias[dst])
                 pm2.start_predictor()
-            xs2 = stack.acts(T, 64, seed=3)
-            out2 = torch.empty_like(xs2[0])
+            n_tok = 64
+            base = stack.acts(Tn, n_tok, seed=3)
+            if predict == "drifting":
+                gen = torch.Generator(device=dev).manual_seed(11)
+                xs2 = []
+                for t in range(n_tok):
+                    x = base[t].float()
+                    row = []
+                    for l in range(L_):
+                        row.append(x.to(torch.bfloat16))
+                        x = (x + 0.5 * torch.randn(x.shape, device=dev, generator=gen)) / (1.25 ** 0.5)
+                    xs2.append(row)
+                act = lambda step, l: xs2[step % n_tok][l]
+            else:
+                act = lambda step, l: base[step % n_tok]
+            out2 = torch.empty_like(base[0])
             n2 = 40 * L_
             for i in range(10 * L_):              # fill the slots along the Zipf popularity
-                pm2.forward(i % L_, xs2[(i // L_) % len(xs2)], out=out2)
+                pm2.forward(i % L_, act(i // L_, i % L_), out=out2)
             torch.cuda.synchronize()
             c0 = pm2.counters()
             t0 = time.perf_counter()
             for i in range(n2):
-                pm2.forward(i % L_, xs2[(10 + i // L_) % len(xs2)], out=out2)
+                pm2.forward(i % L_, act(10 + i // L_, i % L_), out=out2)
             torch.cuda.synchronize()
             d3 = time.perf_counter() - t0
             c2 = pm2.counters()
             pm2.close()
             dl = {kk: c2[kk] - c0[kk] for kk in ("hit", "miss", "prefetch_hit", "prefetch_miss", "ready", "unready",
                                                  "wait_us", "h2d_bytes")}
-            return {"cache_rate": 0.375, "policy": "lru", "tokens_per_s": T * n2 / d3, "ms_per_step": d3 / n2 * 1e3,
+            return {"cache_rate": 0.375, "policy": "lru", "tokens_per_step": Tn, "tokens_per_s": Tn * n2 / d3,
+                    "ms_per_step": d3 / n2 * 1e3,
                     "hit_rate": dl["hit"] / max(dl["hit"] + dl["miss"], 1), "h2d_GB": dl["h2d_bytes"] / 1e9,
                     "h2d_GBps": dl["h2d_bytes"] / d3 / 1e9, "steps": n2, "misses": dl["miss"],
                     "wait_us_per_miss": dl["wait_us"] / max(dl["miss"], 1) if not predict else None,
                     "prefetch_hits": dl["prefetch_hit"], "prefetch_copies": dl["prefetch_miss"],
                     "ready_rate": dl["ready"] / max(dl["ready"] + dl["unready"], 1), "wait_us_total": dl["wait_us"]}
-        cache_run = cache_leg(False)
+        cache_run = cache_leg(T)
         if T == 1:
-            cache_run["with_predictor"] = cache_leg(True)
+            cache_run["with_predictor"] = cache_leg(T, "exact")
+            cache_run["with_predictor_drifting_hidden_state"] = cache_leg(T, "drifting")
+        # the decode configuration as configured (cache rate 0.375, LRU, demand fetching): T = 1, 4, 16
+        as_configured = {}
+        for Tn in (1, 4, 16):
+            r = cache_run if Tn == T else cache_leg(Tn)
+            as_configured[str(Tn)] = {kk: r[kk] for kk in ("tokens_per_s", "ms_per_step", "hit_rate", "h2d_GBps", "misses", "steps")}
 
     prefill = None
     if not a.no_prefill:
@@ -483,13 +550,39 @@ def main():
                                    512, 3584, 64, 2560, 8, 20480, L.FMT_Q4K, True, 0, steps=10))
 
     cpu = None
+    cpu_more = None
     if not a.no_cpu:
         threads = 8   # the reference's own torch.set_num_threads(8) (utils/__init__.py:343)
+        ncpu = os.cpu_count() or threads
+        try:
+            ncpu = min(ncpu, len(os.sched_getaffinity(0)))
+        except AttributeError:
+            pass
         v, med, n_cpu = cpu_baseline(T, H, I, E, I_sh, k, threads)
         cpu = {"value": v, "unit": "tokens/s", "cores": threads, "kind": "port",
                "sample": "the oracle's fp32 per-expert forward (F.linear) of one layer of the same shape, T=%d: %d "
                          "layer steps in about 12 s after 2 warm-ups (median %.1f ms/step); host has %d logical "
-                         "cores" % (T, n_cpu, med * 1e3, os.cpu_count())}
+                         "cores" % (T, n_cpu, med * 1e3, ncpu)}
+        cpu_more = []
+        for Tn, thr in ((T, ncpu), (128, threads), (128, ncpu)):   # all cores, and the reference's CPU-runnable T = 128
+            if (Tn, thr) == (T, threads):
+                continue
+            v2, med2, n2c = cpu_baseline(Tn, H, I, E, I_sh, k, thr, budget_s=5.0)
+            cpu_more.append({"value": v2, "unit": "tokens/s", "cores": thr, "kind": "port", "tokens_per_step": Tn,
+                             "sample": "same forward, T=%d, %d threads: %d layer steps in about 5 s (median %.1f ms/step)"
+                                       % (Tn, thr, n2c, med2 * 1e3)})
+
+    roofline_by_T = None
+    if not a.no_sweep and T == 1:
+        from promoe_amd import _lib as L
+        roofline_by_T = {}
+        for Tn in (4, 16):
+            leg = decode_leg(torch, "DeepSeek-MoE-16B-shaped layer, int4-g128 experts, decode T=%d, all resident, "
+                             "Zipf(1.2)" % Tn, L.FMT_INT4_G128, Tn, H, E, I, k, I_sh, False, 0, 8, 1.2, steps=216)
+            roofline_by_T[str(Tn)] = {"roofline": leg["roofline"], "us_per_layer": leg["us_per_layer"],
+                                      "layer_GBps": leg["layer_GBps"], "layer_frac_of_hbm_peak": leg["layer_GBps"] / HBM_PEAK_GBS,
+                                      "distinct_routed_experts_per_step": leg["distinct_routed_experts_per_step"],
+                                      "algorithmic_bytes_per_step": leg["algorithmic_bytes_per_step"]}
 
     out = {"metric": "moe_layer_decode_tokens_per_s", "value": value, "unit": "tokens/s", "n_gpus": 1,
            "steps": a.steps, "warmup": a.warmup, "ms_per_step": dt / a.steps * 1e3, "higher_is_better": True,
@@ -497,8 +590,11 @@ def main():
            "config": {"workload": "DeepSeek-MoE-16B-shaped MoE layer, int4-g128 experts, decode T=%d, "
                                   "steady-state hits (all routed experts resident), %d-layer stack" % (T, L_),
                       "hidden": H, "experts": E, "intermediate": I, "shared_intermediate": I_sh, "top_k": k,
-                      "tokens_per_step": T, "layers": L_, "zipf": 1.2},
-           "roofline": roofline, "cpu_baseline": cpu, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
+                      "tokens_per_step": T, "layers": L_, "zipf": 1.2,
+                      "weights": "random int4-g128 images (uniform nibbles and zero points, fp16 scales 0.005 to 0.009): "
+                                 "the kernels' time does not depend on the values"},
+           "timing": timing, "c2_as_configured_tokens_per_s": as_configured,
+           "roofline": roofline, "roofline_by_T": roofline_by_T, "cpu_baseline": cpu, "cpu_baseline_more": cpu_more, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
            "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run, "prefill": prefill, "other_decode_configs": others}
     print(json.dumps(out))
 
