@@ -40,7 +40,8 @@ def parse():
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill (matrix-core) legs")
     ap.add_argument("--only", default="", help="profiling aid: run only these prefill legs (comma list of "
-                    "qwen, deepseek, mixtral; other = the decode legs of the other configurations) and print their "
+                    "qwen, deepseek, mixtral, qwen2q4k; other = the decode legs of the other configurations; tN = the "
+                    "DeepSeek-shaped decode layer at N tokens per step) and print their "
                     "results, without the decode benchmark")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: also run a plain 256 MiB read + 256 MiB write elementwise kernel three "
@@ -328,10 +329,18 @@ def main():
                              2048, 2048, 64, 1408, 6, 2816, L.FMT_INT4_G128, False, 0, 20),
                 "mixtral": ("Mixtral-8x7B-shaped layer, int4-g128 experts, prefill T=4096, all resident",
                             4096, 4096, 8, 14336, 2, 0, L.FMT_INT4_G128, False, 2, 5)}
+        legs["qwen2q4k"] = ("Qwen2-57B-A14B-shaped layer, q4_K experts, prefill T=512, all resident",
+                            512, 3584, 64, 2560, 8, 20480, L.FMT_Q4K, True, 0, 10)
         names = a.only.split(",")
-        res = {"prefill": [prefill_leg(torch, *legs[n][:-1], steps=legs[n][-1]) for n in names if n != "other"]}
+        res = {"prefill": [prefill_leg(torch, *legs[n][:-1], steps=legs[n][-1]) for n in names if n in legs]}
         if "other" in names:
             res["other_decode_configs"] = other_configs(torch)
+        # t4, t16, t64, ...: the decode kernels of the DeepSeek-shaped layer at that many tokens per step
+        tn = [int(n[1:]) for n in names if n[:1] == "t" and n[1:].isdigit()]
+        if tn:
+            res["decode_by_T"] = [decode_leg(torch, "DeepSeek-MoE-16B-shaped layer, int4-g128 experts, decode T=%d, all "
+                                             "resident, Zipf(1.2)" % t, L.FMT_INT4_G128, t, 2048, 64, 1408, 6, 2816, False, 0,
+                                             8, 1.2, steps=108) for t in tn]
         print(json.dumps(res))
         return
 

@@ -278,9 +278,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
                    eng->layer_complete[layer] == E && !eng->predictor_attached;
   }
-  static const bool token_route = !(getenv("MOE_TOKEN_ROUTE") && atoi(getenv("MOE_TOKEN_ROUTE")) == 0);
-  static const bool token_w2c = !(getenv("MOE_TOKEN_W2C") && atoi(getenv("MOE_TOKEN_W2C")) == 0);
-  if (all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
+  if (all_resident && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
     // one token: gate logits, then the w13 kernel routes by itself (no top-k / dispatch launches)
     if (!d.gate_bias) {
       if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
@@ -299,7 +297,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     // the kernel stores the unit list into the pending slot's pinned memory and then the sequence word
     const int seq = ++s->seq_counter;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
-    const bool w2c = token_w2c && w2c_fits(d, k);  // w2 and the combine in one launch
+    const bool w2c = w2c_fits(d, k);  // w2 and the combine in one launch
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
@@ -320,7 +318,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // reference's order (hits were computed already, misses are fetched and computed one by one) while the GPU
   // works.  From the table snapshot until the hooks have marked the hits, the layer's slot group is guarded:
   // prefetch and demand traffic may evict, but no copy into one of its slots starts.
-  const bool optimistic = !all_resident && token_route && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 &&
+  const bool optimistic = !all_resident && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 &&
                           eng->cfg.early_preempt && eng->cfg.reorder_experts && (size_t)d.H * 2 + 8192 <= 60 * 1024;
   if (optimistic) {
     if (!d.gate_bias) {
@@ -387,7 +385,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     // every selected expert resident it also combines, otherwise it leaves partial rows for the
     // experts computed below and the combine after them
     const float *sgo = d.shared_gated ? s->logits + E : nullptr;
-    const bool w2c = later.empty() && token_w2c && w2c_fits(d, k);
+    const bool w2c = later.empty() && w2c_fits(d, k);
     if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
@@ -416,10 +414,9 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
-  static const bool fused_route = !(getenv("MOE_FUSED_ROUTE") && atoi(getenv("MOE_FUSED_ROUTE")) == 0);
   bool routed_by_tail = false;
   int tail_seq = 0;
-  if (all_resident && fused_route && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
+  if (all_resident && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory
     if (!d.gate_bias) {
@@ -438,7 +435,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                 max_units, pn.units, pn.n_active, pn.seq, tail_seq, st)))
       return rc;
     routed_by_tail = true;
-  } else if (fused_route && T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
+  } else if (T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
     // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
     // single workgroup behind a device-scope counter, which beats two more launches only
     // while that tail is short (measured: +5 % tokens/s at T=1, -2 % at T=4, -25 % at T=16)

@@ -1920,16 +1920,6 @@ static int launch_gemv_mfma_kc(const GemvArgs &a, int grid, hipStream_t s) {
   return launch_gemv_mfma_kc_ks<SW, NT, CG, 2>(a, grid, s);
 }
 
-// 0: dot2 GEMV for T == 1, matrix-core form otherwise (default); 1: always dot2; 2: always MFMA
-static int gemv_mode() {
-  static int mode = -1;
-  if (mode < 0) {
-    const char *e = getenv("MOE_DECODE_GEMV");
-    mode = e ? atoi(e) : 0;
-  }
-  return mode;
-}
-
 template <bool SW>
 static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_routed, hipStream_t s) {
   // tiles in flight per wave and block: the routed class's groups per wave, at most 4
@@ -1937,8 +1927,7 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
   const int gpw = (G_routed + 3) / 4;
   int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
   if (ch < 1) ch = 1;
-  const int mode = gemv_mode();
-  if (mode == 2 || (mode == 0 && T > 1)) {
+  if (T > 1) {  // matrix-core forms; one token takes the dot2 GEMV below
     // token rows the whole-row form would stage, and whether two of its workgroups then share a CU
     int tb_full = 1;
     while (tb_full < T && tb_full < 16) tb_full <<= 1;
@@ -2119,20 +2108,18 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
       moe_set_error("moe_decode_token_int4: fused w2 + combine does not fit LDS (k=%d I=%d)", k, I);
       return MOE_EINVAL;
     }
-    static const int ni_env = getenv("MOE_W2C_SPLIT") ? atoi(getenv("MOE_W2C_SPLIT")) : 0;
-    const int ni = ni_env == 1 || ni_env == 2 || ni_env == 4 ? ni_env : 2;
+    // two workgroups per 16-row tile (8 rows each): 256 workgroups at H = 2048, one per compute unit; one
+    // workgroup per tile took 10.0 us where two take 6.8 us, four no less
     static bool attr_set = false;
     if (lds > 64 * 1024 && !attr_set) {
-      for (const void *f : {(const void *)k_w2_combine_token<1>, (const void *)k_w2_combine_token<2>, (const void *)k_w2_combine_token<4>})
-        if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                   "hipFuncSetAttribute(k_w2_combine_token)"))
-          return rc;
+      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_w2_combine_token<2>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                 "hipFuncSetAttribute(k_w2_combine_token)"))
+        return rc;
       attr_set = true;
     }
     moe_ktimer_begin(MOE_K_W2, s);
-    if (ni == 1) hipLaunchKernelGGL(k_w2_combine_token<1>, dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
-    else if (ni == 2) hipLaunchKernelGGL(k_w2_combine_token<2>, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
-    else hipLaunchKernelGGL(k_w2_combine_token<4>, dim3(H / 4), dim3(64 * W2C_WAVES), lds, s, c);
+    hipLaunchKernelGGL(k_w2_combine_token<2>, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
     moe_ktimer_end(MOE_K_W2, s);
     return moe_check_launch("k_w2_combine_token");
   }
