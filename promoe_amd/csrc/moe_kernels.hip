@@ -173,19 +173,17 @@ __global__ __launch_bounds__(256) void k_topk(const float *__restrict__ logits, 
   float sel_v = 0.f;  // lane j keeps the j-th selected logit
   float sum_sel = 0.f;
   for (int j = 0; j < k; ++j) {
-    // local best, ties to the lower index
-    float bv = v[0];
-    int bi = lane;
+    // the maximum (DPP row shifts and broadcasts: no LDS round trips), then the lowest expert id that holds
+    // it: lowest 64-wide column first, then lowest lane
+    const float bv = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+    int wr = -1, wl = 0;
 #pragma unroll
-    for (int r = 1; r < 4; ++r) {
-      if (v[r] > bv) { bv = v[r]; bi = lane + 64 * r; }
+    for (int r = 0; r < 4; ++r) {
+      const unsigned long long mr = __ballot(v[r] == bv);
+      if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) {
-      const float ov = __shfl_xor(bv, m, 64);
-      const int oi = __shfl_xor(bi, m, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
+    const int bi = wl + 64 * wr;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       if (bi == lane + 64 * r) v[r] = NEG;
@@ -975,11 +973,10 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
 //   item i < k*G : unit i / G, quantisation group i % G;  items k*G .. : the shared expert's groups
 //   A tile holds 16 rows; the workgroup wants 8 of them, so a wave reads the halves of TWO items with
 //   one load: lanes whose tile row is 0..7 take item 2s, the others item 2s + 1, each its row & 7 of
-//   the workgroup's half.  Wave w takes the item pairs s = w, w+16, ...; W2C_CHUNK loads per wave are
+//   the workgroup's half.  Wave w takes the item pairs s = w, w+16, ...; up to six loads per wave are
 //   requested before the activations (the h vectors of all units) are staged in LDS.
 //   H/8 workgroups: twice the compute units of a 16-row split, which is what the load latency wants.
 // ---------------------------------------------------------------------------
-#define W2C_CHUNK 3
 #define W2C_WAVES 16
 struct W2cArgs {
   const KUnit *kunits;   // resolved routed units (slot address; row = position of the unit's h vector)
@@ -993,8 +990,10 @@ struct W2cArgs {
   int *err;
 };
 
-// NI = items a wave reads with one load = 16 / (rows per workgroup)
-template <int NI>
+// NI = items a wave reads with one load = 16 / (rows per workgroup); W2C_CHUNK = loads a wave keeps in flight
+// (3 covers the whole share of a wave at 2048 x 1408 with six units; long reductions such as 4096 x 14336
+// take 6, so that a wave's share is two round trips to memory instead of three or more)
+template <int NI, int W2C_CHUNK>
 __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2cArgs a) {
   extern __shared__ __align__(16) unsigned char wsm[];
   constexpr int RW = 16 / NI;  // rows of this workgroup
@@ -1816,13 +1815,19 @@ static int launch_gemv_q4k_t(const GemvArgs &a, int grid, size_t lds, hipStream_
 
 template <bool SW>
 static int launch_gemv_q4k(const GemvArgs &a, int grid, int T, int Kmax, hipStream_t s) {
-  int tmax = T <= 1 ? 1 : (T <= 4 ? 4 : 16);
-  while (tmax > 1 && gemv_q4k_lds(tmax, Kmax) > 150 * 1024) tmax >>= 2;
+  // rows per pass: the smallest power of two >= T (at most 16) whose activations fit LDS; a unit with more
+  // rows than that streams its weights once per pass (three tokens against a 20480-column reduction: two
+  // rows per pass, two passes)
+  int tmax = 1;
+  while (tmax < T && tmax < 16) tmax <<= 1;
+  while (tmax > 1 && gemv_q4k_lds(tmax, Kmax) > 150 * 1024) tmax >>= 1;
   const size_t lds = gemv_q4k_lds(tmax, Kmax);
   if (lds > 150 * 1024) { moe_set_error("k_gemv_int4<q4k>: K=%d does not fit LDS", Kmax); return MOE_EINVAL; }
   switch (tmax) {
     case 1: return launch_gemv_q4k_t<SW, 1>(a, grid, lds, s);
+    case 2: return launch_gemv_q4k_t<SW, 2>(a, grid, lds, s);
     case 4: return launch_gemv_q4k_t<SW, 4>(a, grid, lds, s);
+    case 8: return launch_gemv_q4k_t<SW, 8>(a, grid, lds, s);
     default: return launch_gemv_q4k_t<SW, 16>(a, grid, lds, s);
   }
 }
@@ -2112,14 +2117,20 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
     // workgroup per tile took 10.0 us where two take 6.8 us, four no less
     static bool attr_set = false;
     if (lds > 64 * 1024 && !attr_set) {
-      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_w2_combine_token<2>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                 "hipFuncSetAttribute(k_w2_combine_token)"))
-        return rc;
+      for (const void *f : {(const void *)k_w2_combine_token<2, 3>, (const void *)k_w2_combine_token<2, 6>,
+                            (const void *)k_w2_combine_token<1, 7>})
+        if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                   "hipFuncSetAttribute(k_w2_combine_token)"))
+          return rc;
       attr_set = true;
     }
     moe_ktimer_begin(MOE_K_W2, s);
-    hipLaunchKernelGGL(k_w2_combine_token<2>, dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+    // loads per wave: the (unit, group) items, two per load, over the 16 waves
+    const int loads_per_wave = ((k * c.G + c.G_sh + 1) / 2 + W2C_WAVES - 1) / W2C_WAVES;
+    if (loads_per_wave <= 3) hipLaunchKernelGGL((k_w2_combine_token<2, 3>), dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+    else if (H / 16 >= 256)  // one workgroup per 16-row tile already gives every compute unit one: whole tiles
+      hipLaunchKernelGGL((k_w2_combine_token<1, 7>), dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
+    else hipLaunchKernelGGL((k_w2_combine_token<2, 6>), dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
     moe_ktimer_end(MOE_K_W2, s);
     return moe_check_launch("k_w2_combine_token");
   }
