@@ -19,6 +19,7 @@ CXX_SOURCES = ["moe_common.cpp", "engine_cfg.cpp", "engine_core.cpp", "engine_fo
 
 # -packed-fp32-ops: keep hipcc from forming v_pk_*_f32 out of scalar float code.
 HIP_FLAGS = [
+    "-Wno-inline-asm",
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

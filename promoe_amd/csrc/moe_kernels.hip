@@ -650,7 +650,13 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
     wk.m = 1; wk.row0 = 0; wk.base = a.shared_base;
     return wk;
   }
-  if (publisher && w != 0) { wk.m = 0; wk.row0 = 0; wk.base = nullptr; return wk; }
+  // One wave of the workgroup derives the routing and hands the unit's slot address to the others through
+  // LDS: four waves doing the same rounds would each take their turn on the SIMDs.  Workgroups b, b + 256, ...
+  // share a compute unit when the grid is resident as a whole; they route on different SIMDs.
+  __shared__ unsigned s_route_base[2];
+  const int rw = publisher ? 0 : (int)((blockIdx.x >> 8) & 3);
+  wk.m = publisher ? 0 : 1; wk.row0 = u;
+  if (w == rw) {
   const float NEG = -__builtin_inff();
   float v[NR], v0[NR];
   unsigned long long ptrs[NR];  // slot addresses of the lane's candidates, fetched alongside the logits
@@ -704,11 +710,9 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
     }
     cum += cnt;
   }
-  wk.m = 1; wk.row0 = u;
-  wk.base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+  if (lane == 0) { s_route_base[0] = lo; s_route_base[1] = hi; }
 
   if (publisher) {  // publish the routing: weights as in k_topk, arrays as in k_dispatch (T = 1)
-    wk.m = 0;       // no weight tiles for this workgroup
     // position of a pair = rank of its expert id among the selected
     int below[NR], cb = 0;
 #pragma unroll
@@ -771,6 +775,9 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
     }
     if (lane == 0) { a.r_offsets[E] = k; *a.r_n_active = k; }
   }
+  }
+  __syncthreads();
+  wk.base = (const unsigned char *)(((unsigned long long)s_route_base[1] << 32) | s_route_base[0]);
   return wk;
 }
 

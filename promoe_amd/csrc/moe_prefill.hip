@@ -4,15 +4,16 @@
 //   w13 pass: h[rows, I]   = silu(A Wg^T) * (A Wu^T)     A = gathered activations
 //   w2  pass: part[rows,H] = h W2^T
 //
-// Workgroup = 512 threads (8 waves) -> a tile of up to 256 rows x (128+128) columns: for
-// w13 the two column halves are the SAME columns of gate and up (SwiGLU fused in the
-// epilogue), for w2 they are adjacent column blocks.  K advances 64 at a time; the
-// activation slab goes global -> registers -> double-buffered LDS, the weight fragments go
-// global -> registers in operand order and feed v_mfma_f32_32x32x16_bf16 directly.
+// bf16 experts: workgroup = 256 threads (4 waves, one per SIMD) -> a tile of up to 256 rows x (128+128)
+// columns: for w13 the two column halves are the SAME columns of gate and up (SwiGLU fused in the epilogue),
+// for w2 they are adjacent column blocks.  K advances 64 at a time; the activation slab goes global -> LDS
+// directly (a ring of four slabs), the weight fragments go global -> registers in operand order and feed
+// v_mfma_f32_32x32x16_bf16.  int4 / q4_K experts: 8 waves, fragments dequantised in registers (below).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string.h>
 #include <stdlib.h>
+#include <type_traits>
 
 #include "moe_common.h"
 #include "moe_kernels.h"
@@ -28,7 +29,6 @@ typedef __attribute__((address_space(1))) const u32x4_t g_uint4;
 #define PF_BM_SHARED_W2 128  // and in its w2 pass, which has few column tiles (H/256) and a long K
 #define PF_BNH 128   // columns per half
 #define PF_BK 64
-#define PF_LDK 72    // LDS row stride in bf16 (64 + 8 pad = 144 bytes: conflict-free b128 reads)
 
 struct PfTile {
   unsigned long long w_base;  // expert image base (device address)
@@ -55,102 +55,166 @@ struct PfArgs {
   int n_blocks_total;  // blocks of c[0] come first
 };
 
-static __device__ __forceinline__ uint16_t pf_f32_to_bf16(float f) {
-  u32 u = __float_as_uint(f);
-  u32 r = ((u >> 16) & 1u) + 0x7fffu;
-  return (uint16_t)((u + r) >> 16);
+// silu(g) * u with the hardware's 2^x and reciprocal (1 ulp each; the result is rounded to bf16 by the caller,
+// round to nearest even in hardware): a tile's epilogue computes 128 of these per lane
+static __device__ __forceinline__ float pf_silu_mul(float g, float u) {
+  return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * -1.44269504088896f)) * u;
 }
 
-// Main loop of one wave.  The workgroup has 8 waves: wave w = 0..3 of group g = 0..1 owns
-// columns 32w..32w+31 of both column halves and the 32-row blocks g, g+2, g+4, g+6 of the
-// tile (NBW of them are live), 128 accumulator registers; the two waves that share a SIMD
-// (same w) fill each other's stalls.  The weight operand never touches LDS: a wave loads its
-// fragments straight from global memory, where they lie in operand order (blocks of 32 rows
-// x 64 k, one contiguous KiB per MFMA step); the second group's loads of the same fragments
-// hit in the CU's vector L1.  Within a 64-wide K slab lane half q = lane/32 takes
-// k = 32q + 8j + 0..7 for MFMA j: both operands use the same permutation of k, which a dot
-// product allows.
-template <int NBW>
-static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[4][2], uint16_t *As, const uint16_t *const (&a_ptr)[4],
-                                                   const uint16_t *b0p, const uint16_t *b1p, int nk, int rot0, int rot1, int nb, int tid) {
-  const int lane = tid & 63, g = tid >> 8;
-  const int kc = tid & 7, r0 = tid >> 3;  // staging: row r0 + 64 i (block 2i + g), 16-byte chunk kc
+// Which class and which block of it a physical workgroup takes: the blocks of class 0 come first, each class
+// padded to a multiple of 8 blocks, so that physical id % 8 is the XCD inside either class.  (Alternating the
+// classes in groups of 8 was measured: no gain in the w13 launch, 19 % slower in the w2 launch.)
+static __device__ __forceinline__ void pf_block_of(const PfArgs &a, int &ci, int &pb) {
+  const int pad0 = (a.c[0].n_blocks + 7) & ~7;
+  ci = (int)blockIdx.x >= pad0;
+  pb = ci ? (int)blockIdx.x - pad0 : (int)blockIdx.x;
+}
+
+// ---- bf16 experts: main loop of one wave ------------------------------------------------------------
+// One wave per SIMD, 512 registers each: wave w owns columns 32w..32w+31 of both column halves and ALL row
+// blocks of the tile (up to 8 x 32 rows: 256 accumulator registers, which the compiler keeps in the
+// accumulation half of the register file), so every weight fragment is fetched by exactly one wave of the
+// workgroup.  The weights lie in HBM in operand order (blocks of 32 rows x 64 k, one contiguous KiB per MFMA
+// step; within a 64-wide K slab lane half q = lane / 32 takes k = 32 q + 8 j + 0..7 for MFMA j: both operands
+// use the same permutation of k, which a dot product allows) and never touch LDS.
+// What a single wave per SIMD needs, since nothing else fills its stalls (each measured on the Qwen1.5 shape
+// and in a stand-alone loop of the same structure):
+//   * weight fragments and activations are requested three slabs ahead (four register sets of fragments,
+//     four activation slabs in LDS);
+//   * the requests are spread between the products, at most one behind each, instead of standing in a block
+//     at the head of a slab where the matrix core runs dry behind them (stand-alone loop, streaming from HBM:
+//     1.29 -> 1.53 PFLOP/s);
+//   * the activation fragment of a product is read from LDS four product groups ahead, and nothing may move
+//     across the pinned order (left to itself the scheduler puts every read right in front of its own
+//     products and waits for it there: an LDS round trip per pair of products);
+//   * no vector instruction computes an address inside the loop (buffer addressing: lane offsets that never
+//     change, slab offsets in scalars; LDS addresses with compile-time ring slots).
+#define PF_ST 4                      // register sets of weight fragments: requested three slabs ahead
+#define PF4_SLAB (PF_BM * PF_BK)     // bf16 elements of one activation slab in LDS (rows of 128 bytes, no padding)
+#define PF4_RING 4                   // slabs in LDS: one being read, three on their way
+#define PF_FD 4                      // LDS reads in flight in front of the products
+typedef __attribute__((address_space(3))) void pf_lds_void;
+typedef __attribute__((address_space(1))) const void pf_g_void;
+// s_waitcnt that waits for all but the N most recent vector-memory operations and for nothing else
+#define PF_VMCNT(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (7 << 4) | (15 << 8) | (((N) >> 4) << 14))
+
+typedef int pf_i32x4_t __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t pf_rsrc_t;
+
+// Activations go global -> LDS directly (no registers, no LDS store instructions): transfer n of wave w
+// brings rows 32 n + 8 w .. + 7 of the slab, 8 lanes per row.  An LDS row is 128 bytes = 8 chunks of 16; the
+// chunk that holds k = 8 c .. 8 c + 7 of row r sits in slot c ^ ((r >> 1) & 7), so the 16 lanes that a
+// ds_read_b128 serves together (16 rows, one chunk index) fall on 16 different bank groups.  The lanes choose
+// their global address accordingly; the LDS side of the transfer is fixed (lane l writes 16 bytes at 16 l).
+// All addresses are buffer addresses (lane offset in a register that never changes, slab offset in a scalar):
+// with one wave per SIMD every vector instruction that is not a product is issue time taken from the products.
+template <int NB>
+static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsigned lds_base, const pf_i32x4_t ra_rsrc,
+                                                    const int (&a_voff)[8], const pf_rsrc_t rb, int b_delta1, int nk, int rot0,
+                                                    int rot1, int tid) {
+  const int lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int fr = lane & 31, q = lane >> 5;
-  u32x4_t ra[4], bufA[2][4], bufB[2][4];
-  // (block 2i + g is live iff i < NBW: a compile-time condition, so every iteration issues the same
-  // number of loads and the compiler's waits for the prefetched registers can be exact)
-  auto gloadA = [&](int kt) {
+  constexpr int NL = NB + 8;   // requests of a step: NB activation transfers, 8 weight fragments
+  constexpr int NS = 4 * NB;   // groups of two products
+  u32x4_t bw[PF_ST][2][4];
+  const int b_voff = lane * 16;
+  // transfer n of slab kt_ into ring slot `slot` (past the end: the last slab again, into a slot nobody reads)
+  auto dma = [&](int n, int kt_, int slot) {
+    const int kt = kt_ < nk ? kt_ : nk - 1;
+    // Written as assembly on purpose: the compiler, told that a load writes LDS, waits for ALL such loads in
+    // front of every barrier and LDS read, which would end the run-ahead; here the waits are placed by hand
+    // (PF_VMCNT below).  Its own counts for the fragment loads then include fewer operations than are in
+    // flight, which only makes its waits for those loads earlier, never later.
+    const unsigned lds_addr = lds_base + (unsigned)(slot * PF4_SLAB + (32 * n + 8 * w) * PF_BK) * 2u;
+    __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(a_voff[n]), "s"(ra_rsrc), "s"(kt * (PF_BK * 2)) : "memory", "m0");
+  };
+  auto bslab = [&](int kt_, int rot) {
+    const int kt = kt_ < nk ? kt_ : nk - 1;  // past the end: the last slab once more (never used)
+    const int k = kt + rot;                  // slab position inside the 128-row group's storage
+    return (k >= nk ? k - nk : k) * 16384;   // bytes
+  };
+  // LDS byte address of the lane's fragment of MFMA step j in row block 0 of slot 0 (chunk 4 q + j of its row)
+  unsigned faddr[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (i < NBW) ra[i] = *(g_uint4 *)(a_ptr[i] + kt * PF_BK);
+  for (int j = 0; j < 4; ++j) faddr[j] = lds_base + (unsigned)(fr * PF_BK + (((4 * q + j) ^ ((fr >> 1) & 7)) * 8)) * 2u;
+  auto lds_frag = [&](int slot, int g) {
+    typedef __attribute__((address_space(3))) const bf16x8_t lds_frag_t;
+    return *(lds_frag_t *)(uintptr_t)(faddr[g / NB] + (unsigned)(slot * PF4_SLAB + 32 * (g % NB) * PF_BK) * 2u);
+  };
+  // slab kt (ring slot S = kt % 4, a compile-time number in the unrolled loop): its weight fragments are in
+  // `cur`.  Requested meanwhile, at most one request behind every product: the activations (into slot
+  // (S + 3) % 4) and the fragments (into `far`) of slab kt + 3.
+  auto step = [&](auto S_, int kt, const u32x4_t(&cur)[2][4], u32x4_t(&far)[2][4]) {
+    constexpr int S = decltype(S_)::value;
+    const int sb0 = bslab(kt + 3, rot0), sb1 = bslab(kt + 3, rot1) + b_delta1;
+    // product group g = MFMA step j = g / NB of row block i = g % NB; its activation fragment is read from LDS
+    // PF_FD groups ahead of its products
+    bf16x8_t fa[PF_FD + 1];
+#pragma unroll
+    for (int g = 0; g < PF_FD && g < NS; ++g) fa[g] = lds_frag(S, g);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < NS; ++g) {
+      acc[g % NB][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[g % (PF_FD + 1)], __builtin_bit_cast(bf16x8_t, cur[0][g / NB]),
+                                                               acc[g % NB][0], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (g + PF_FD < NS) fa[(g + PF_FD) % (PF_FD + 1)] = lds_frag(S, g + PF_FD);
+      __builtin_amdgcn_sched_barrier(0);
+      acc[g % NB][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[g % (PF_FD + 1)], __builtin_bit_cast(bf16x8_t, cur[1][g / NB]),
+                                                               acc[g % NB][1], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int n = 0; n < NL; ++n)
+        if (n * NS / NL == g) {  // request n of this step goes out behind product group g
+          if (n < NB) dma(n, kt + 3, (S + 3) % PF4_RING);
+          else if (n - NB < 4) far[0][n - NB] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB), sb0, 0);
+          else far[1][n - NB - 4] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB - 4), sb1, 0);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // slab kt + 1 must have landed before anybody reads it: its transfers are two steps old, issued before
+    // the 8 fragment loads of their own step and the NB + 8 requests of each of the two steps since
+    PF_VMCNT(2 * NB + 24);
+    __syncthreads();
   };
   auto gloadB = [&](u32x4_t(&b)[2][4], int kt) {
-    int k0 = kt + rot0, k1 = kt + rot1;  // slab position inside the 128-row group's storage
-    k0 = k0 >= nk ? k0 - nk : k0;
-    k1 = k1 >= nk ? k1 - nk : k1;
+    const int sb0 = bslab(kt, rot0), sb1 = bslab(kt, rot1) + b_delta1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[0][j] = *(g_uint4 *)(b0p + (size_t)k0 * 8192 + 512 * j);
+    for (int j = 0; j < 4; ++j) b[0][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb0, 0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[1][j] = *(g_uint4 *)(b1p + (size_t)k1 * 8192 + 512 * j);
+    for (int j = 0; j < 4; ++j) b[1][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb1, 0);
   };
-  auto sstore = [&](int st) {
-    uint16_t *A_ = As + st * PF_BM * PF_LDK;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (i < NBW) *(u32x4_t *)(A_ + (r0 + 64 * i) * PF_LDK + kc * 8) = ra[i];
-  };
-  auto compute = [&](int st, const u32x4_t(&b)[2][4]) {
-    const uint16_t *A_ = As + st * PF_BM * PF_LDK + (32 * g + fr) * PF_LDK + 32 * q;
+  for (int t = 0; t < 3; ++t) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      bf16x8_t fa[NBW > 0 ? NBW : 1];
-#pragma unroll
-      for (int i = 0; i < NBW; ++i) fa[i] = *(const bf16x8_t *)(A_ + 64 * i * PF_LDK + 8 * j);
-#pragma unroll
-      for (int i = 0; i < NBW; ++i)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          acc[i][h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], __builtin_bit_cast(bf16x8_t, b[h][j]), acc[i][h], 0, 0, 0);
-    }
-  };
-  // one K slab: the weight fragments of slab kt are in `cur`; slab kt+1's are requested into
-  // `nxt`, and its activations go through registers into the other LDS stage
-  auto step = [&](int kt, const u32x4_t(&cur)[2][4], u32x4_t(&nxt)[2][4]) {
-    // unconditional: the last slab requests itself once more instead of branching around the loads
-    const int kn = kt + 1 < nk ? kt + 1 : kt;
-    gloadA(kn);
-    if (NBW > 0) gloadB(nxt, kn);
-    __builtin_amdgcn_sched_barrier(0);  // the requests go out before the products, not after them
-    compute(kt & 1, cur);
-    if (kt + 1 < nk) {
-      sstore((kt + 1) & 1);
-      __syncthreads();
-    }
-  };
-  gloadA(0);
-  if (NBW > 0) gloadB(bufA, 0);
-  sstore(0);
+    for (int n = 0; n < NB; ++n) dma(n, t, t);
+    gloadB(bw[t], t);
+  }
+  PF_VMCNT(0);
   __syncthreads();
-  for (int kt = 0; kt < nk; kt += 2) {  // nk is even (K % 128 == 0)
-    step(kt, bufA, bufB);
-    step(kt + 1, bufB, bufA);
+  typedef std::integral_constant<int, 0> S0; typedef std::integral_constant<int, 1> S1;
+  typedef std::integral_constant<int, 2> S2; typedef std::integral_constant<int, 3> S3;
+  for (int kt = 0; kt < nk; kt += 4) {  // nk is even; no separate tail: its register assignment would differ
+    step(S0(), kt, bw[0], bw[3]);      // from the loop's and the compiler would spill around the loop's back edge
+    step(S1(), kt + 1, bw[1], bw[0]);
+    if (kt + 2 < nk) {
+      step(S2(), kt + 2, bw[2], bw[1]);
+      step(S3(), kt + 3, bw[3], bw[2]);
+    }
   }
 }
 
 template <bool SWIGLU>
-__global__ __launch_bounds__(512, 1) void k_prefill_gemm(const PfArgs a) {
-  extern __shared__ __align__(16) uint16_t As[];  // [2][PF_BM][PF_LDK]
-  const int tid = threadIdx.x, lane = tid & 63, w = (tid >> 6) & 3, g = tid >> 8;
-
-  // XCD-aware order: workgroup i runs on XCD i % 8; give every XCD one contiguous range of
-  // the block list, so that blocks that share an operand (n tiles of one m tile for the
-  // routed experts, m tiles of one n tile for the shared expert) meet in one L2.
-  // Each class occupies a multiple of 8 physical blocks, so physical id % 8 is the XCD inside
-  // either class and the heavy and the light class are both spread over all XCDs.
-  const int pad0 = (a.c[0].n_blocks + 7) & ~7;
-  const int ci = (int)blockIdx.x >= pad0;
-  const int pb = ci ? blockIdx.x - pad0 : blockIdx.x;
-  // only the tiles in use are spread over the XCDs; the launch covers an upper bound
+__global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
+  extern __shared__ __align__(16) uint16_t As[];  // [PF4_RING][PF_BM][PF_BK]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  // XCD-aware order: workgroup i runs on XCD i % 8; give every XCD one contiguous range of the block list,
+  // so that blocks that share an operand (n tiles of one m tile for the routed experts, m tiles of one n
+  // tile for the shared expert) meet in one L2.  Only the tiles in use are spread over the XCDs; the launch
+  // covers an upper bound.
+  int ci, pb;
+  pf_block_of(a, ci, pb);
   const int n_mt = *a.c[ci].n_tiles_real;
   const int n_real = n_mt * a.c[ci].n_ntiles;
   const int per_xcd = (n_real + 7) >> 3;
@@ -167,55 +231,67 @@ __global__ __launch_bounds__(512, 1) void k_prefill_gemm(const PfArgs a) {
   const int n0 = nt * c.n_cols_per_tile;
   const uint16_t *W = (const uint16_t *)(tile.w_base + c.w_off);
 
-  const int kc = tid & 7, r0 = tid >> 3;
-  const uint16_t *a_ptr[4];
+  // transfer n of this wave brings rows 32 n + 8 w .. + 7, 8 lanes per row; the lane in slot s of row r
+  // fetches chunk s ^ ((r >> 1) & 7).  Byte offsets from the activation tensor's base (< 2 GiB, checked by the launcher)
+  int a_voff[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int row = r0 + 64 * i;
-    row = row < tile.rows ? row : 0;  // rows past the group's end re-read row 0 (never stored)
+  for (int i = 0; i < 8; ++i) {
+    const int rt = 32 * i + 8 * w + (lane >> 3);
+    const int row = rt < tile.rows ? rt : 0;  // rows past the group's end re-read row 0 (never stored)
     const int grow = tile.row0 + row;
     const int arow = c.gather ? c.gather[grow] : grow;
-    a_ptr[i] = c.act + (size_t)arow * c.act_stride + kc * 8;
+    a_voff[i] = (arow * c.act_stride + (((lane & 7) ^ ((rt >> 1) & 7)) * 8)) * 2;
   }
-  // weight blocks of 32 rows x 64 k (2048 elements); the 4 blocks of a 128-row group are
-  // adjacent for each k slab, so one slab of a column half is 16 KiB of contiguous memory
-  const uint16_t *b0 = W + ((size_t)(n0 / 128) * (K / PF_BK) * 4 + w) * 2048 + lane * 8;
-  const uint16_t *b1 = b0 + (size_t)(c.half_delta / 128) * (K / PF_BK) * 8192;
+  pf_i32x4_t ra_rsrc;
+  {
+    const unsigned long long ab = (unsigned long long)c.act;
+    ra_rsrc.x = __builtin_amdgcn_readfirstlane((int)(unsigned)ab);
+    ra_rsrc.y = __builtin_amdgcn_readfirstlane((int)(unsigned)(ab >> 32));
+    ra_rsrc.z = 0x7fffffff; ra_rsrc.w = 0x00020000;
+  }
+  // weight blocks of 32 rows x 64 k (4 KiB); the 4 blocks of a 128-row group are adjacent for each k slab, so
+  // one slab of a column half is 16 KiB of contiguous memory; wave w reads block w
+  const int nk = K / PF_BK;
+  const unsigned char *wb = (const unsigned char *)W + ((size_t)(n0 / 128) * nk * 4 + w) * 4096;
+  const unsigned long long wbu = (unsigned long long)wb;
+  const pf_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)(((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(wbu >> 32)) << 32) |
+               (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)wbu)), 0, 0x7fffffff, 0x00020000);
+  const int b_delta1 = (int)(c.half_delta / 128) * nk * 16384;
 
-  f32x16_t acc[4][2];
+  f32x16_t acc[8][2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int h = 0; h < 2; ++h)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][h][e] = 0.f;
 
-  const int nk = K / PF_BK;
-  // the slabs of 128-row group G are stored rotated by (G * c.slab_step) % nk, so that groups
-  // read in step (same slab at the same time) stream from different DRAM channels
   const int G0 = n0 / 128, G1 = G0 + (int)(c.half_delta / 128);
   const int rot0 = (int)((unsigned)(G0 * c.slab_step) % (unsigned)nk), rot1 = (int)((unsigned)(G1 * c.slab_step) % (unsigned)nk);
-  const int nb = (tile.rows + 31) >> 5;
-  const int nbw = (nb - g + 1) >> 1;  // live blocks of this wave group (uniform per wave)
-  switch (nbw) {
-    case 0: pf_mainloop<0>(acc, As, a_ptr, b0, b1, nk, rot0, rot1, nb, tid); break;
-    case 1: pf_mainloop<1>(acc, As, a_ptr, b0, b1, nk, rot0, rot1, nb, tid); break;
-    case 2: pf_mainloop<2>(acc, As, a_ptr, b0, b1, nk, rot0, rot1, nb, tid); break;
-    case 3: pf_mainloop<3>(acc, As, a_ptr, b0, b1, nk, rot0, rot1, nb, tid); break;
-    default: pf_mainloop<4>(acc, As, a_ptr, b0, b1, nk, rot0, rot1, nb, tid); break;
+  const int nb = (tile.rows + 31) >> 5;  // live row blocks (uniform for the workgroup)
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)As;
+  switch (nb) {
+    case 1: pf_mainloop<1>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 2: pf_mainloop<2>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 3: pf_mainloop<3>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 4: pf_mainloop<4>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 5: pf_mainloop<5>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 6: pf_mainloop<6>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    case 7: pf_mainloop<7>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+    default: pf_mainloop<8>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
   }
   // epilogue.  acc element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l%32
   const int col = 32 * w + (lane & 31);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int row = 32 * (2 * i + g) + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+      const int row = 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
       if (row < tile.rows) {
         const size_t orow = (size_t)(tile.row0 + row) * c.out_stride;
         if (SWIGLU) {
-          const float gt = acc[i][0][e], up = acc[i][1][e];
-          ((uint16_t *)c.out)[orow + n0 + col] = pf_f32_to_bf16(gt / (1.f + expf(-gt)) * up);
+          ((__bf16 *)c.out)[orow + n0 + col] = (__bf16)pf_silu_mul(acc[i][0][e], acc[i][1][e]);
         } else {
           ((float *)c.out)[orow + n0 + col] = acc[i][0][e];
           ((float *)c.out)[orow + n0 + PF_BNH + col] = acc[i][1][e];
@@ -404,9 +480,8 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   const int r = lane & 15, qd = lane >> 4;
 
   // block order: as in k_prefill_gemm
-  const int pad0 = (a.c[0].n_blocks + 7) & ~7;
-  const int ci = (int)blockIdx.x >= pad0;
-  const int pb = ci ? blockIdx.x - pad0 : blockIdx.x;
+  int ci, pb;
+  pf_block_of(a, ci, pb);
   const int n_mt = *a.c[ci].n_tiles_real;
   const int n_real = n_mt * a.c[ci].n_ntiles;
   const int per_xcd = (n_real + 7) >> 3;
@@ -467,7 +542,7 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
             const float gt = acc[2 * b][tb][i], up = acc[2 * b + 1][tb][i];
-            ((uint16_t *)c.out)[orow + 16 * (rb0 / 2 + b) + r] = pf_f32_to_bf16(gt / (1.f + expf(-gt)) * up);
+            ((__bf16 *)c.out)[orow + 16 * (rb0 / 2 + b) + r] = (__bf16)pf_silu_mul(gt, up);
           }
         } else {
 #pragma unroll
@@ -507,7 +582,7 @@ static int pi_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
 static int pf_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
   if (a.n_blocks_total <= 0) return MOE_OK;
   const int grid = ((a.c[0].n_blocks + 7) & ~7) + ((a.c[1].n_blocks + 7) & ~7);
-  const size_t lds = (size_t)2 * PF_BM * PF_LDK * 2;
+  const size_t lds = (size_t)PF4_RING * PF4_SLAB * 2;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e1 = hipFuncSetAttribute((const void *)k_prefill_gemm<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -516,8 +591,8 @@ static int pf_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
     attr_set = true;
   }
   moe_ktimer_begin(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
-  if (swiglu) hipLaunchKernelGGL(k_prefill_gemm<true>, dim3(grid), dim3(512), lds, s, a);
-  else hipLaunchKernelGGL(k_prefill_gemm<false>, dim3(grid), dim3(512), lds, s, a);
+  if (swiglu) hipLaunchKernelGGL(k_prefill_gemm<true>, dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL(k_prefill_gemm<false>, dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
   return moe_check_launch("k_prefill_gemm");
 }
@@ -616,7 +691,7 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
   }
   {
     const long long widest = I > H ? I : H, rows = (long long)T * (k > 1 ? k : 1);
-    if (int4 && (rows * widest * 2 >= (1ll << 31) || (shared_ptr && (long long)T * (I_sh > H ? I_sh : H) * 2 >= (1ll << 31)))) {
+    if (rows * widest * 2 >= (1ll << 31) || (shared_ptr && (long long)T * (I_sh > H ? I_sh : H) * 2 >= (1ll << 31))) {
       moe_set_error("moe_experts_prefill: activation buffers of 2 GiB or more are not supported (T=%d k=%d)", T, k);
       return MOE_EINVAL;
     }
