@@ -186,7 +186,14 @@ int moe_decode_token_int4_noalloc(const void *x_bf16, const float *logits, int E
                                   int I_sh, const uint64_t *expert_ptr, const void *shared_ptr,
                                   const float *shared_gate_logit, void *y_bf16, int *err, void *stream);
 
-/* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only. */
+/* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only.
+ * Exception: part_s.  With few output rows and a long reduction (H / 32 block pairs, I_sh columns: Qwen2-57B's
+ * shared expert is 112 block pairs over 20480 columns) the w2 pass splits the shared expert's reduction over
+ * moe_decode_shared_splits(MOE_FMT_Q4K, T, H, I_sh) = S workgroups per block pair; split s writes its partial
+ * rows to part_s + s*T*H, so part_s must hold S*T*H floats and the combine must be told
+ * (moe_combine_splits).  S = 1 for every other format.  No reference counterpart (the reference leaves the
+ * arithmetic to llama.cpp's kernels, adapter-llama.cpp:12-46). */
+int moe_decode_shared_splits(int fmt, int T, int H, int I_sh);
 int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, int k,
                            const moe_unit *units, int max_units, const int *sorted_tok,
                            const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
@@ -217,6 +224,11 @@ int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int I_sh, int k
 int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
                 const int *pos_of_pair, const float *shared_gate_logit, int sg_stride, void *y_bf16,
                 int T, int H, int k, void *stream);
+/* the same with a shared expert whose partial rows come in n_shared_splits pieces (piece s at part_s + s*T*H),
+ * added in piece order before the gate is applied; n_shared_splits = 1 is moe_combine */
+int moe_combine_splits(const float *part_r, const float *part_s, const float *topk_w,
+                       const int *pos_of_pair, const float *shared_gate_logit, int sg_stride, void *y_bf16,
+                       int T, int H, int k, int n_shared_splits, void *stream);
 
 /* Per-kernel timing with HIP events recorded on the launch stream around every kernel
  * the launchers below start (no reference counterpart; used by the benchmark to report

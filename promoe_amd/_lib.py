@@ -67,6 +67,8 @@ _sig("moe_experts_prefill", [vp, i32, i32, i32, i32, i32, i32, vp, i32, vp, vp, 
 _sig("moe_kernel_timing", [i32])
 _sig("moe_kernel_timing_read", [i32, C.POINTER(C.c_double), C.POINTER(i32)])
 _sig("moe_combine", [vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, vp])
+_sig("moe_combine_splits", [vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, vp])
+_sig("moe_decode_shared_splits", [i32, i32, i32, i32])
 
 
 def check(rc: int, what: str = ""):

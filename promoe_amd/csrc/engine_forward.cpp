@@ -153,7 +153,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, (uint16_t **)&s->h_r, P * I);
   rc |= dalloc(s, (uint16_t **)&s->h_s, (size_t)T * I_sh);
   rc |= dalloc(s, &s->part_r, P * H);
-  rc |= dalloc(s, &s->part_s, (size_t)T * H);
+  // q4_K decode batches (at most 16 tokens) may leave the shared expert's partial rows in up to 8 pieces
+  rc |= dalloc(s, &s->part_s, (size_t)(T > 128 ? T : 128) * H);
   rc |= dalloc(s, (unsigned char **)&s->tiles_ws, (size_t)moe_prefill_workspace_bytes(T, k, s->max_units));
   rc |= halloc(s, &s->units_host, s->max_units);
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
@@ -240,6 +241,11 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
   return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                  s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
                                  s->part_r, s->part_s, s->err_host + layer, units_host, table_host, 3, st);
+}
+
+// pieces the expert launch of run_units leaves the shared expert's partial rows in
+static int shared_pieces(const moe_layer_desc &d, int T) {
+  return d.I_sh > 0 && d.fmt == MOE_FMT_Q4K && !use_prefill(d, T) ? moe_decode_shared_splits(MOE_FMT_Q4K, T, d.H, d.I_sh) : 1;
 }
 
 // the one-token w2 + combine kernel stages the h vectors of all units in LDS
@@ -476,7 +482,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
     if ((rc = run_units(eng, d, s, x, T, s->units, nullptr, max_units, d.I_sh > 0, layer, table, st))) return rc;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
-    if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k, st)))
+    if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k,
+                                 shared_pieces(d, T), st)))
       return rc;
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
@@ -534,7 +541,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
   }
   const float *sg = d.shared_gated ? s->logits + E : nullptr;
-  if ((rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k, st)))
+  if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k,
+                               shared_pieces(d, T), st)))
     return rc;
   // MoeLayerHook.post_forward (utils/hooks.py:220-223)
   if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;

@@ -539,7 +539,9 @@ struct GemvClass {
   const int *gather;    // row -> activation row (NULL = identity)
   void *out;            // bf16 (SWIGLU) or fp32
   long long off_q, off_s, off_z;
-  int K, G, act_stride, out_stride, nblk, pad;
+  int K, G, act_stride, out_stride, nblk;
+  int ksplit;           // q4_K, shared expert's w2 pass: workgroups per block pair, each over 1/ksplit of the
+                        // reduction, partial rows to out + split * T * out_stride (0 or 1: the whole reduction)
 };
 #define GEMV_MAX_KUNITS 64
 struct KUnit { unsigned long long base; int m, row0; };
@@ -584,7 +586,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
   c.act = sh ? c0.act : c1.act; c.gather = sh ? c0.gather : c1.gather; c.out = sh ? c0.out : c1.out;
   c.off_q = sh ? c0.off_q : c1.off_q; c.off_s = sh ? c0.off_s : c1.off_s; c.off_z = sh ? c0.off_z : c1.off_z;
   c.K = sh ? c0.K : c1.K; c.G = sh ? c0.G : c1.G; c.act_stride = sh ? c0.act_stride : c1.act_stride;
-  c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk; c.pad = 0;
+  c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk; c.ksplit = sh ? c0.ksplit : c1.ksplit;
   const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
   const int u = sh ? 0 : rr / c.nblk;
   wk.b = rr - u * c.nblk;
@@ -796,14 +798,21 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
 
   const GemvWork wk = ROUTE ? gemv_resolve_route(a, lane, w) : gemv_resolve<DEVUNITS>(a);
   const GemvClass &c = wk.c;
-  const int m = wk.m, row0 = wk.row0, b = wk.b;
+  const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
     if (tid == 0) moe_raise_err(a.err);
     return;
   }
-  const int K = c.K, G = c.G, KS = K >> 5;
+  // Gt groups per row block in memory; this workgroup reduces over the window [g0, g0 + G) of them (the whole
+  // row unless the class is split: then `split` of c.ksplit workgroups share a block pair)
+  const int Gt = c.G;
+  const int nsp = (Q4K && c.ksplit > 1) ? c.ksplit : 1;
+  const int split = nsp > 1 ? wk.b % nsp : 0;
+  const int b = nsp > 1 ? wk.b / nsp : wk.b;
+  const int G = Gt / nsp, g0 = split * G;
+  const int K = G * 128, KS = K >> 5;
   // LDS: activations, their 32-wide sums, the scale/zero sections of the two row blocks,
   // and the cross-wave reduction buffer
   uint16_t *xs = (uint16_t *)smem;                                    // [TMAX][K]
@@ -816,10 +825,10 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   const int GPW = (G - w + 3) >> 2;  // groups of this wave: g = w + 4j, j < GPW
   const int rbA = 2 * b;
   // tiles of block A then block B are contiguous: 2*G KiB
-  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, 2u * G * 1024u);
-  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * SCB, 2u * G * SCB);
-  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * ZZB, 2u * G * ZZB);
-  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
+  const rsrc_t rq = make_rsrc(base + c.off_q + ((size_t)rbA * Gt + g0) * 1024, (u32)(Gt + G) * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + ((size_t)rbA * Gt + g0) * SCB, (u32)(Gt + G) * SCB);
+  const rsrc_t rz = make_rsrc(base + c.off_z + ((size_t)rbA * Gt + g0) * ZZB, (u32)(Gt + G) * ZZB);
+  const rsrc_t rx = make_rsrc((const unsigned char *)c.act + (size_t)g0 * 256, 0x7fffffffu);
   const int zsh = (r & 1) * 4;
   const int vec_per_row = K >> 3;
   const int n_sc = 2 * G * SCB / 4;   // dwords of section s
@@ -837,14 +846,18 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
       // threads past the row's end re-read vector 0 (staged nowhere): never past the tensor
       xv[t] = bload16(rx, (tid < vec_per_row ? tid : 0) * 16, arow * c.act_stride * 2);
     }
-    const u32 msc0 = bload4(rs, tid * 4, 0), msc1 = bload4(rs, tid * 4, 1024);
-    const u32 mzz = bload4(rz, tid * 4, 0);
+    // dword i of the LDS copy [2][G] of a section lies at i * 4 in memory, plus the gap between the two blocks'
+    // windows for the second block (no gap when the window is the whole row)
+    const int sc_half = G * SCB / 4, zz_half = G * ZZB / 4, sc_gap = (Gt - G) * SCB, zz_gap = (Gt - G) * ZZB;
+    const u32 msc0 = bload4(rs, tid * 4 + (tid >= sc_half ? sc_gap : 0), 0);
+    const u32 msc1 = bload4(rs, (tid + 256) * 4 + (tid + 256 >= sc_half ? sc_gap : 0), 0);
+    const u32 mzz = bload4(rz, tid * 4 + (tid >= zz_half ? zz_gap : 0), 0);
     uint4 wa[CH], wb[CH];
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       const int g = j < GPW ? w + 4 * j : 0;  // clamped: tile 0 always exists
       wa[j] = bload16(rq, lane * 16, g * 1024);
-      wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+      wb[j] = bload16(rq, lane * 16, (Gt + g) * 1024);
     }
     // ---- stage: x -> LDS (+ 32-wide sums via a quad reduction), scale/zero -> LDS ----------
 #pragma unroll
@@ -873,8 +886,8 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
         if ((tid & 3) == 0) xsum[(t * vec_per_row + v) >> 2] = ps;
       }
     }
-    for (int i = tid + 512; i < n_sc; i += 256) ((u32 *)s_sc)[i] = bload4(rs, i * 4, 0);
-    for (int i = tid + 256; i < n_zz; i += 256) ((u32 *)s_zz)[i] = bload4(rz, i * 4, 0);
+    for (int i = tid + 512; i < n_sc; i += 256) ((u32 *)s_sc)[i] = bload4(rs, i * 4 + (i >= sc_half ? sc_gap : 0), 0);
+    for (int i = tid + 256; i < n_zz; i += 256) ((u32 *)s_zz)[i] = bload4(rz, i * 4 + (i >= zz_half ? zz_gap : 0), 0);
     __syncthreads();
 
     float accA[TMAX], accB[TMAX];
@@ -887,7 +900,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
         for (int j = 0; j < CH; ++j) {
           const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
           wa[j] = bload16(rq, lane * 16, g * 1024);
-          wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+          wb[j] = bload16(rq, lane * 16, (Gt + g) * 1024);
         }
       }
 #pragma unroll
@@ -966,7 +979,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
         float v = 0.f;
 #pragma unroll
         for (int ww = 0; ww < 4; ++ww) v += red[((ww * TMAX + t) * 2 + ab) * 16 + rr2];
-        ((float *)c.out)[(size_t)(row0 + t0 + t) * c.out_stride + (2 * b + ab) * 16 + rr2] = v;
+        ((float *)c.out)[((size_t)split * a.T + (row0 + t0 + t)) * c.out_stride + (2 * b + ab) * 16 + rr2] = v;
       }
     }
     if (t0 + TMAX < m) __syncthreads();
@@ -1623,7 +1636,7 @@ __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_
                                                   const int *__restrict__ pos_of_pair,
                                                   const float *__restrict__ sg_logit,
                                                   int sg_stride, uint16_t *__restrict__ y, int H,
-                                                  int k) {
+                                                  int k, int n_sh_splits) {
   const int t = blockIdx.y;
   const int n = (blockIdx.x * 256 + threadIdx.x) * 4;
   if (n >= H) return;
@@ -1651,7 +1664,12 @@ __global__ __launch_bounds__(256) void k_combine(const float *__restrict__ part_
   }
   if (part_s) {
     const float g = sg_logit ? 1.f / (1.f + expf(-sg_logit[(size_t)t * sg_stride])) : 1.f;
-    const float4 v = *(const float4 *)(part_s + (size_t)t * H + n);
+    float4 v = *(const float4 *)(part_s + (size_t)t * H + n);
+    // a shared expert whose reduction was split over workgroups: its partial rows, added in split order
+    for (int sp = 1; sp < n_sh_splits; ++sp) {
+      const float4 u = *(const float4 *)(part_s + ((size_t)sp * gridDim.y + t) * H + n);
+      v.x += u.x; v.y += u.y; v.z += u.z; v.w += u.w;
+    }
     acc.x = fmaf(g, v.x, acc.x); acc.y = fmaf(g, v.y, acc.y);
     acc.z = fmaf(g, v.z, acc.z); acc.w = fmaf(g, v.w, acc.w);
   }
@@ -2229,6 +2247,21 @@ extern "C" int moe_q4k_layout_make(int H, int I, moe_int4_layout *out) {
   return MOE_OK;
 }
 
+// Workgroups per block pair of the shared expert's w2 pass (q4_K decode): with few output rows (H / 32 block
+// pairs) and a long reduction every block pair is one long workgroup, and a reduction that does not fit the LDS
+// with all token rows costs a pass over the weights per row group.  Splitting the reduction over 2, 4 or 8
+// workgroups gives the launch enough of them and keeps every token row of a decode batch in one pass; each
+// split writes its own partial rows and the combine adds them in split order.
+extern "C" int moe_decode_shared_splits(int fmt, int T, int H, int I_sh) {
+  if (fmt != MOE_FMT_Q4K || T <= 0 || H <= 0 || I_sh <= 0 || I_sh % 256) return 1;
+  const int pairs = H / 32, G = I_sh / 128;
+  int sp = 1;
+  // as long as the launch has under 448 shared workgroups and a split keeps at least 16 groups (a whole number
+  // of 256-wide super-blocks)
+  while (sp < 8 && pairs * sp < 448 && G % (sp * 4) == 0 && G / (sp * 2) >= 16) sp *= 2;
+  return sp;
+}
+
 extern "C" int moe_experts_decode_q4k(const void *x, int T, int H, int I, int I_sh, int k,
                                       const moe_unit *units, int max_units, const int *sorted_tok,
                                       const uint64_t *expert_ptr, const void *shared_ptr,
@@ -2259,14 +2292,15 @@ extern "C" int moe_experts_decode_q4k(const void *x, int T, int H, int I, int I_
   int grid = a.n_sh_blocks + max_units * (I / 16);
   if (grid > 0 && (phases & 1))
     if (int rc = launch_gemv_q4k<true>(a, grid, T, H, s)) return rc;
+  const int sp = sh ? moe_decode_shared_splits(MOE_FMT_Q4K, T, H, I_sh) : 1;
   a.cls[0] = GemvClass{(const uint16_t *)h_s, nullptr, part_s, ls.off2_q, ls.off2_s, ls.off2_z,
-                       I_sh, I_sh / 128, I_sh, H, H / 32, 0};
+                       I_sh, I_sh / 128, I_sh, H, (H / 32) * sp, sp};
   a.cls[1] = GemvClass{(const uint16_t *)h_r, nullptr, part_r, lr.off2_q, lr.off2_s, lr.off2_z,
                        I, I / 128, I, H, H / 32, 0};
-  a.n_sh_blocks = sh ? H / 32 : 0;
+  a.n_sh_blocks = sh ? (H / 32) * sp : 0;
   grid = a.n_sh_blocks + max_units * (H / 32);
   if (grid > 0 && (phases & 2))
-    if (int rc = launch_gemv_q4k<false>(a, grid, T, I_sh > I ? I_sh : I, s)) return rc;
+    if (int rc = launch_gemv_q4k<false>(a, grid, T, I_sh / sp > I ? I_sh / sp : I, s)) return rc;
   return MOE_OK;
 }
 
@@ -2325,19 +2359,25 @@ extern "C" int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int
   return moe_check_launch("k_topk_dispatch");
 }
 
-extern "C" int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
-                           const int *pos_of_pair, const float *sg_logit, int sg_stride, void *y,
-                           int T, int H, int k, void *stream) {
+extern "C" int moe_combine_splits(const float *part_r, const float *part_s, const float *topk_w,
+                                  const int *pos_of_pair, const float *sg_logit, int sg_stride, void *y,
+                                  int T, int H, int k, int n_shared_splits, void *stream) {
   if (!y || T < 0 || H <= 0 || H % 4 || k < 0 || (k > 0 && (!part_r || !topk_w || !pos_of_pair)) ||
-      T > 65535) {
-    moe_set_error("moe_combine: bad argument (T=%d H=%d k=%d)", T, H, k);
+      T > 65535 || n_shared_splits < 1 || n_shared_splits > 8) {
+    moe_set_error("moe_combine: bad argument (T=%d H=%d k=%d splits=%d)", T, H, k, n_shared_splits);
     return MOE_EINVAL;
   }
   if (T == 0) return MOE_OK;
   dim3 grid((H / 4 + 255) / 256, T);
   moe_ktimer_begin(MOE_K_COMBINE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_combine, grid, dim3(256), 0, (hipStream_t)stream, part_r, part_s, topk_w,
-                     pos_of_pair, sg_logit, sg_stride, (uint16_t *)y, H, k);
+                     pos_of_pair, sg_logit, sg_stride, (uint16_t *)y, H, k, n_shared_splits);
   moe_ktimer_end(MOE_K_COMBINE, (hipStream_t)stream);
   return moe_check_launch("k_combine");
+}
+
+extern "C" int moe_combine(const float *part_r, const float *part_s, const float *topk_w,
+                           const int *pos_of_pair, const float *sg_logit, int sg_stride, void *y,
+                           int T, int H, int k, void *stream) {
+  return moe_combine_splits(part_r, part_s, topk_w, pos_of_pair, sg_logit, sg_stride, y, T, H, k, 1, stream);
 }

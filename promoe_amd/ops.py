@@ -185,7 +185,8 @@ def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.T
         h_s = part_s = None
         if shared is not None:
             h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
-            part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+            # the w2 pass may split the shared expert's reduction: one set of partial rows per split
+            part_s = torch.empty(shared_splits(L.FMT_Q4K, T, H, I_sh) * T, H, dtype=torch.float32, device=dev)
         err = torch.zeros(1, dtype=torch.int32, device=dev)
     check(lib.moe_experts_decode_q4k(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
                                      ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
@@ -218,12 +219,20 @@ def experts_prefill(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tens
     return part_r, part_s, err, h_r, h_s, tiles
 
 
+def shared_splits(fmt: int, T: int, H: int, I_sh: int) -> int:
+    """Pieces the decode w2 pass leaves the shared expert's partial rows in (1 unless q4_K with a long reduction)."""
+    return int(lib.moe_decode_shared_splits(fmt, T, H, I_sh)) if I_sh else 1
+
+
 def combine(part_r, part_s, topk_w, pos_of_pair, shared_gate_logit, T: int, H: int, k: int,
             out: torch.Tensor | None = None):
+    """part_s [S*T, H]: S > 1 when the shared expert's reduction was split (piece s = rows s*T .. s*T+T-1)."""
     dev = (part_r if part_r is not None else part_s).device
     if out is None:
         out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
     sg_stride = shared_gate_logit.stride(0) if shared_gate_logit is not None else 0
-    check(lib.moe_combine(ptr(part_r), ptr(part_s), ptr(topk_w), ptr(pos_of_pair),
-                          ptr(shared_gate_logit), sg_stride, ptr(out), T, H, k, cur_stream()), "moe_combine")
+    n_splits = 1 if part_s is None else max(1, part_s.shape[0] // max(T, 1))
+    check(lib.moe_combine_splits(ptr(part_r), ptr(part_s), ptr(topk_w), ptr(pos_of_pair),
+                                 ptr(shared_gate_logit), sg_stride, ptr(out), T, H, k, n_splits, cur_stream()),
+          "moe_combine")
     return out
