@@ -30,6 +30,11 @@ struct LayerState {
   // sees them without a copy: one per layer for launches in which that must not happen (checked at the next
   // call and when the engine drains), one for launches that are allowed to meet non-resident experts
   int *err_host = nullptr, *err_loose = nullptr;
+  // error words of the w2 + combine launches that go out before the host knows the routing (one per layer), and
+  // what the host expects of each once it does: 1 = must stay zero (every selected expert was resident at
+  // launch), 2 = may be set (an expert was missing; that launch's output is recomputed), 0 = none outstanding
+  int *err_spec = nullptr;
+  std::vector<char> spec_state;
   int num_layer = 0;
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
@@ -162,6 +167,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   s->num_layer = eng->cfg.num_layer;
   rc |= halloc(s, &s->err_host, eng->cfg.num_layer);
   rc |= halloc(s, &s->err_loose, 1);
+  rc |= halloc(s, &s->err_spec, eng->cfg.num_layer);
   rc |= halloc(s, &s->opt_seq, 1);
   for (auto &p : s->pend) {
     rc |= halloc(s, &p.units, s->max_units);
@@ -173,6 +179,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   if (rc) return MOE_EHIP;
   memset(s->err_host, 0, sizeof(int) * eng->cfg.num_layer);
   *s->err_loose = 0;
+  memset(s->err_spec, 0, sizeof(int) * eng->cfg.num_layer);
+  s->spec_state.assign(eng->cfg.num_layer, 0);
   HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
   *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
@@ -185,7 +193,7 @@ int moe_forward_check_kernels(moe_engine *eng) {
   LayerState *s = eng->fw;
   if (!s) return MOE_OK;
   for (int l = 0; l < s->num_layer; ++l)
-    if (((volatile int *)s->err_host)[l])
+    if (((volatile int *)s->err_host)[l] || (s->spec_state[l] == 1 && ((volatile int *)s->err_spec)[l]))
       return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", l);
   return MOE_OK;
 }
@@ -352,6 +360,24 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                     s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
                                     nullptr, nullptr, st)))
       return rc;
+    // The w2 pass with the combine goes out at once as well, as if nothing were missing: in most steps nothing
+    // is, and then the GPU has this layer's kernels queued while the host runs the hooks and is never waited
+    // for.  When an expert turns out to be missing, its output is recomputed below (the kernel skips the
+    // missing expert and raises its own error word, which the host then knows to expect).
+    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
+    const bool spec_w2c = w2c_fits(d, k);
+    if (spec_w2c) {
+      if (s->spec_state[layer] == 1 && ((volatile int *)s->err_spec)[layer])   // the launch of this layer's last turn
+        return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", layer);
+      s->spec_state[layer] = 0;
+      s->err_spec[layer] = 0;
+      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                      d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                      s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                      s->h_r, s->h_s, s->part_r, s->part_s, s->err_spec + layer, s->unit_ws,
+                                      nullptr, nullptr, 0, 4, sgo, y, st)))
+        return rc;
+    }
     {  // the routing arrives a few microseconds after the kernel starts
       volatile int *sq = s->opt_seq;
       const auto t0 = std::chrono::steady_clock::now();
@@ -387,16 +413,17 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       eng->ctr.ready += (uint64_t)now_ids.size();
     }
     guard.release();
-    // the w2 pass goes out now that the routing is known (the w13 kernel is still running): with
-    // every selected expert resident it also combines, otherwise it leaves partial rows for the
-    // experts computed below and the combine after them
-    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
-    const bool w2c = later.empty() && w2c_fits(d, k);
-    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+    // with every selected expert resident the launch above was the whole layer; otherwise the w2 pass goes out
+    // again without the combine (the w13 kernel is still running) and leaves partial rows for the experts
+    // computed below and the combine after them
+    const bool w2c = later.empty() && spec_w2c;
+    if (spec_w2c) s->spec_state[layer] = later.empty() ? 1 : 2;
+    if (!w2c &&
+        (rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, w2c ? s->err_host + layer : s->err_loose, s->unit_ws,
-                                    nullptr, nullptr, 0, w2c ? 4 : 2, sgo, y, st)))
+                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws,
+                                    nullptr, nullptr, 0, 2, sgo, y, st)))
       return rc;
     // no event in the stream (one costs the step about 4 us of GPU time): the experts count as in use until
     // the routing word of a LATER one-token step arrives, whose kernel starts behind everything queued here

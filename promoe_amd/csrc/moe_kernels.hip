@@ -802,7 +802,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   const unsigned char *base = wk.base;
   if (m <= 0) return;
   if (base == nullptr) {
-    if (tid == 0) moe_raise_err(a.err);
+    if (tid == 0 && wk.b == 0) moe_raise_err(a.err);  // one store per missing unit (the word may be host memory)
     return;
   }
   // Gt groups per row block in memory; this workgroup reduces over the window [g0, g0 + G) of them (the whole
@@ -1052,6 +1052,13 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
     uw = a.sg_logit ? 1.f / (1.f + expf(-a.sg_logit[0])) : 1.f;
   }
 
+  // a selected expert that is not resident (slot address 0) is skipped below and reported here, by one wave of
+  // the launch: the word may live in pinned host memory, where a store per wave would be thousands of
+  // transactions over the host link
+  if (blockIdx.x == 0 && w == 0) {
+    const bool miss = (lane < k || (lane == k && I_sh > 0)) && ub_lo == 0 && ub_hi == 0;
+    if (__ballot(miss) != 0ull && lane == 0) moe_raise_err(a.err);
+  }
   float acc = 0.f;
   // cursor of the wave's current group of NI items: first item = unit u (k = the shared expert), group g
   int u = 0, g = NI * w;
@@ -1067,7 +1074,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
     for (int c = 0; c < W2C_CHUNK; ++c) {
       // the group's items are consecutive; pick the lane's own while walking them (all uniform but the selects)
       int uj = u, gj = g;
-      bool on = false, any_missing = false;
+      bool on = false;
       int lu = 0, lg = 0;
       unsigned long long base = 0ull;
       float lw = 0.f;
@@ -1078,12 +1085,10 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
         const u32 lo = __builtin_amdgcn_readlane(ub_lo, ul), hi = __builtin_amdgcn_readlane(ub_hi, ul);
         const float wj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul));
         const unsigned long long bj = ((unsigned long long)hi << 32) | lo;
-        any_missing = any_missing || (onj && bj == 0ull);
         if (mine == j) { on = onj && bj != 0ull; lu = uj; lg = gj; base = bj; lw = wj; }
         ++gj;  // next item
         if (uj < k && gj >= G) { gj -= G; ++uj; }
       }
-      if (any_missing && lane == 0) moe_raise_err(a.err);  // a selected expert that is not resident
       const bool shd = lu >= k;
       const int Gu = shd ? G_sh : G;
       wgt[c] = lw;
