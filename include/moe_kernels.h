@@ -109,6 +109,17 @@ int moe_dispatch(const int *idx, int T, int k, int E, int *counts, int *offsets,
                  int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
                  int64_t *active_ids, int max_units, void *stream);
 
+/* k2 with a workspace, for prefill batches: the same arrays, bit for bit, from one workgroup per 1024 pairs when
+ * P = T*k >= 2048 and E <= 256 (otherwise, or with ws NULL or smaller than moe_dispatch_workspace_bytes, this is
+ * moe_dispatch).  ws: device memory whose first 64 bytes are zero before the first call (the kernel leaves them
+ * zero); calls that share a workspace must not overlap.  err: word that a workgroup raises when the others'
+ * counts do not arrive within a second (device memory or pinned host memory).
+ * moe_dispatch_workspace_bytes returns 0 where the workspace would not be used. */
+int64_t moe_dispatch_workspace_bytes(int T, int k, int E);
+int moe_dispatch_ws(const int *idx, int T, int k, int E, int *counts, int *offsets, int *sorted_pair,
+                    int *pos_of_pair, int *sorted_tok, moe_unit *units, int *n_active,
+                    int64_t *active_ids, int max_units, void *ws, int64_t ws_bytes, int *err, void *stream);
+
 /* k1a+k1b+k2 in one launch for decode batches (T <= 16, E <= 256, T*k <= 512): same results,
  * bit for bit, as moe_gate_logits + moe_topk + moe_dispatch.  E_rows = E, or E+1 when row E of
  * wg is the shared expert's gate vector (its logit lands in logits[t*ldl + E], no bias).

@@ -48,6 +48,8 @@ _sig("moe_int4_layout_make", [i32, i32, C.POINTER(Int4Layout)])
 _sig("moe_gate_logits", [vp, vp, vp, vp, i32, i32, i32, i32, vp])
 _sig("moe_topk", [vp, i32, i32, i32, i32, i32, vp, vp, vp])
 _sig("moe_dispatch", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
+_sig("moe_dispatch_workspace_bytes", [i32, i32, i32], C.c_int64)
+_sig("moe_dispatch_ws", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, i64, vp, vp])
 _sig("moe_route_decode", [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp])
 _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_topk_dispatch", [vp, i32, i32, i32, i32, i32] + [vp] * 10 + [i32, vp, vp, vp, i32, vp])

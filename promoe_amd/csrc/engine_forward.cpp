@@ -23,6 +23,8 @@ struct LayerState {
   moe_unit *units = nullptr, *units_sub = nullptr;
   int64_t *active_ids = nullptr;
   void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
+  unsigned char *disp_ws = nullptr;  // workspace of the prefill batches' dispatch (starts with its zeroed barrier words)
+  int64_t disp_ws_bytes = 0;
   // pinned host mirrors
   moe_unit *units_host = nullptr, *units_sub_host = nullptr;
   int *n_active_host = nullptr, *opt_seq = nullptr;
@@ -161,6 +163,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   // q4_K decode batches (at most 16 tokens) may leave the shared expert's partial rows in up to 8 pieces
   rc |= dalloc(s, &s->part_s, (size_t)(T > 128 ? T : 128) * H);
   rc |= dalloc(s, (unsigned char **)&s->tiles_ws, (size_t)moe_prefill_workspace_bytes(T, k, s->max_units));
+  s->disp_ws_bytes = moe_dispatch_workspace_bytes(T, k, E);
+  if (s->disp_ws_bytes) rc |= dalloc(s, &s->disp_ws, (size_t)s->disp_ws_bytes);
   rc |= halloc(s, &s->units_host, s->max_units);
   rc |= halloc(s, &s->units_sub_host, (size_t)s->max_units * 2);
   rc |= halloc(s, &s->n_active_host, 1);
@@ -182,6 +186,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   memset(s->err_spec, 0, sizeof(int) * eng->cfg.num_layer);
   s->spec_state.assign(eng->cfg.num_layer, 0);
   HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
+  if (s->disp_ws) HIPC(hipMemset(s->disp_ws, 0, 64));
   *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
   return MOE_OK;
@@ -487,8 +492,10 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
         return rc;
     }
     if ((rc = moe_topk(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, st))) return rc;
-    if ((rc = moe_dispatch(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
-                           s->units, s->n_active, s->active_ids, max_units, st)))
+    // (the workspace is sized for max_tokens: a smaller batch needs no more of it)
+    if ((rc = moe_dispatch_ws(s->idx, T, k, E, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
+                              s->units, s->n_active, s->active_ids, max_units, s->disp_ws, s->disp_ws_bytes,
+                              s->err_host + layer, st)))
       return rc;
   }
   if (all_resident) {

@@ -71,75 +71,96 @@ __global__ __launch_bounds__(256) void k_gate_logits(const uint16_t *__restrict_
   if (lane == 0) logits[(size_t)t * ldl + e] = bias ? acc + bias[e] : acc;
 }
 
-// Large T: a workgroup stages 16 token rows in LDS and every wave walks its gate rows over all
-// 16 tokens, so a gate row is fetched once per 16 tokens instead of once per token.  Each
-// (token, row) sum is formed in exactly the order of k_gate_logits (lane partials over
-// k = c*512 + 8*lane + i with one fma chain, then the xor butterfly 32..1): same bits.
-#define GATE_TT 16
-__global__ __launch_bounds__(256) void k_gate_logits_tile(const uint16_t *__restrict__ x,
-                                                           const uint16_t *__restrict__ wg,
-                                                           const float *__restrict__ bias,
-                                                           float *__restrict__ logits, int T, int H,
-                                                           int E, int ldl, int rows_per_block) {
-  extern __shared__ uint4 gxs[];  // [GATE_TT][H/8]
+// Large T: a workgroup takes 16 tokens (8 waves x 2) and a group of gate rows.  The rows are staged in LDS once
+// per workgroup; a wave keeps the activations of its two tokens in registers as fp32 (the lane's columns
+// 512 c + 8 lane + j) and walks the rows, so a gate row is fetched once per 16 tokens, converted once per two,
+// and the inner loop is one LDS read per eight fma's of each token.  Each (token, row) sum is formed in exactly
+// the order of k_gate_logits (lane partials over k = 512 c + 8 lane + j with one fma chain, then the xor
+// butterfly 32..1): same bits.
+#define GATE_WAVES 8
+#define GATE_TW 2                        // tokens per wave
+#define GATE_TT (GATE_WAVES * GATE_TW)  // tokens per workgroup
+template <int NCH>  // 512-column chunks of a row (H <= 512 NCH)
+__global__ __launch_bounds__(64 * GATE_WAVES) void k_gate_logits_rows(const uint16_t *__restrict__ x,
+                                                                      const uint16_t *__restrict__ wg,
+                                                                      const float *__restrict__ bias,
+                                                                      float *__restrict__ logits, int T, int H,
+                                                                      int E, int ldl, int rows_per_block) {
+  extern __shared__ uint4 gws[];  // [rows of this workgroup][H/8]
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int t0 = blockIdx.x * GATE_TT;
-  const int nt = (T - t0) < GATE_TT ? (T - t0) : GATE_TT;
   const int vpr = H >> 3;
-  const uint4 *xsrc = (const uint4 *)(x + (size_t)t0 * H);
-  for (int i = tid; i < nt * vpr; i += 256) gxs[i] = xsrc[i];
-  for (int i = nt * vpr + tid; i < GATE_TT * vpr; i += 256) gxs[i] = make_uint4(0, 0, 0, 0);
+  const int e0 = blockIdx.y * rows_per_block;
+  const int nrow = (E - e0) < rows_per_block ? (E - e0) : rows_per_block;
+  const uint4 *wsrc = (const uint4 *)(wg + (size_t)e0 * H);
+  for (int i = tid; i < nrow * vpr; i += 64 * GATE_WAVES) gws[i] = wsrc[i];
+  const int t0 = blockIdx.x * GATE_TT + w * GATE_TW;
+  float xf[GATE_TW][NCH][8];
+#pragma unroll
+  for (int t = 0; t < GATE_TW; ++t) {
+    const int tt = (t0 + t) < T ? (t0 + t) : T - 1;  // a token past the end repeats the last one (not stored)
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int k = c * 512 + 8 * lane;
+      const uint4 v = k < H ? *(const uint4 *)(x + (size_t)tt * H + k) : make_uint4(0, 0, 0, 0);
+      xf[t][c][0] = bf16lo(v.x); xf[t][c][1] = bf16hi(v.x); xf[t][c][2] = bf16lo(v.y); xf[t][c][3] = bf16hi(v.y);
+      xf[t][c][4] = bf16lo(v.z); xf[t][c][5] = bf16hi(v.z); xf[t][c][6] = bf16lo(v.w); xf[t][c][7] = bf16hi(v.w);
+    }
+  }
   __syncthreads();
-  const int e_end = min(E, (int)(blockIdx.y + 1) * rows_per_block);
-  const int nch = (H + 511) >> 9;  // <= 8 (checked by the launcher)
-  const int kl = 8 * lane;
-  uint4 wv[8], wn[8];
-  auto load_row = [&](uint4(&dst)[8], int e) {
-    const uint16_t *wr = wg + (size_t)(e < e_end ? e : blockIdx.y * rows_per_block) * H;
+  // four rows per trip (rows past the end are clamped and not stored): eight independent chains.  Their eight
+  // butterflies run as one: at the steps 32, 16 and 8 a lane keeps one half of its values and sends the other, so
+  // every sum has the operands the plain butterfly gives it (own + partner's, and a + b = b + a), with 10
+  // exchanges instead of 48.  Lane L then holds the sum of chain 4 (L>>3 & 1) + 2 (L>>4 & 1) + (L>>5 & 1).
+  constexpr int GR = 4;
+  const bool h32 = lane & 32, h16 = lane & 16, h8 = lane & 8;
+  const int mine = 4 * ((lane >> 3) & 1) + 2 * ((lane >> 4) & 1) + ((lane >> 5) & 1);  // chain = 2 * row + token
+  for (int r = 0; r < nrow; r += GR) {
+    float acc[GR * GATE_TW];
 #pragma unroll
-    for (int c = 0; c < 8; ++c)
-      if (c < nch) {
-        const int k = c * 512 + kl;
-        dst[c] = *(const uint4 *)(wr + (k < H ? k : 0));
-      }
-  };
-  int e = blockIdx.y * rows_per_block + w;
-  if (e < e_end) load_row(wv, e);
-  for (; e < e_end; e += 4) {
-    load_row(wn, e + 4);  // next row of this wave in flight while this one is used
-    float acc[GATE_TT];
+    for (int i = 0; i < GR * GATE_TW; ++i) acc[i] = 0.f;
 #pragma unroll
-    for (int t = 0; t < GATE_TT; ++t) acc[t] = 0.f;
+    for (int c = 0; c < NCH; ++c) {
+      const int k = c * 512 + 8 * lane;
+      if (k < H) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int k = c * 512 + kl;
-      if (c < nch && k < H) {
+        for (int q = 0; q < GR; ++q) {
+          const int rq = r + q < nrow ? r + q : nrow - 1;
+          const uint4 wv = gws[rq * vpr + (k >> 3)];
+          const float wf[8] = {bf16lo(wv.x), bf16hi(wv.x), bf16lo(wv.y), bf16hi(wv.y),
+                               bf16lo(wv.z), bf16hi(wv.z), bf16lo(wv.w), bf16hi(wv.w)};
 #pragma unroll
-        for (int t = 0; t < GATE_TT; ++t) {
-          const uint4 xv = gxs[t * vpr + (k >> 3)];
-          float a = acc[t];
-          a = fmaf(bf16lo(xv.x), bf16lo(wv[c].x), a);
-          a = fmaf(bf16hi(xv.x), bf16hi(wv[c].x), a);
-          a = fmaf(bf16lo(xv.y), bf16lo(wv[c].y), a);
-          a = fmaf(bf16hi(xv.y), bf16hi(wv[c].y), a);
-          a = fmaf(bf16lo(xv.z), bf16lo(wv[c].z), a);
-          a = fmaf(bf16hi(xv.z), bf16hi(wv[c].z), a);
-          a = fmaf(bf16lo(xv.w), bf16lo(wv[c].w), a);
-          a = fmaf(bf16hi(xv.w), bf16hi(wv[c].w), a);
-          acc[t] = a;
+          for (int t = 0; t < GATE_TW; ++t) {
+            float a = acc[q * GATE_TW + t];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) a = fmaf(xf[t][c][j], wf[j], a);
+            acc[q * GATE_TW + t] = a;
+          }
         }
       }
     }
-    const float be = bias ? bias[e] : 0.f;
+    static_assert(GR * GATE_TW == 8, "the reduction below folds eight chains");
+    float u[4], v2[2];
 #pragma unroll
-    for (int t = 0; t < GATE_TT; ++t) {
-      float a = acc[t];
-#pragma unroll
-      for (int m = 32; m >= 1; m >>= 1) a = a + __shfl_xor(a, m, 64);
-      if (lane == 0 && t < nt) logits[(size_t)(t0 + t) * ldl + e] = bias ? a + be : a;
+    for (int i = 0; i < 4; ++i) {
+      const float keep = h32 ? acc[2 * i + 1] : acc[2 * i], send = h32 ? acc[2 * i] : acc[2 * i + 1];
+      u[i] = keep + __shfl_xor(send, 32, 64);
     }
 #pragma unroll
-    for (int c = 0; c < 8; ++c) wv[c] = wn[c];
+    for (int i = 0; i < 2; ++i) {
+      const float keep = h16 ? u[2 * i + 1] : u[2 * i], send = h16 ? u[2 * i] : u[2 * i + 1];
+      v2[i] = keep + __shfl_xor(send, 16, 64);
+    }
+    float z;
+    {
+      const float keep = h8 ? v2[1] : v2[0], send = h8 ? v2[0] : v2[1];
+      z = keep + __shfl_xor(send, 8, 64);
+    }
+    z = z + __shfl_xor(z, 4, 64);
+    z = z + __shfl_xor(z, 2, 64);
+    z = z + __shfl_xor(z, 1, 64);
+    const int rq = r + (mine >> 1), tq = t0 + (mine & 1);
+    if ((lane & 7) == 0 && rq < nrow && tq < T)
+      logits[(size_t)tq * ldl + e0 + rq] = bias ? z + bias[e0 + rq] : z;
   }
 }
 
@@ -303,6 +324,137 @@ __global__ __launch_bounds__(DISP_THREADS) void k_dispatch(
       sorted_tok[pos] = p / k;
     }
     __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// k2 for prefill batches: the same arrays from P / 1024 workgroups in one launch.  A workgroup ranks its own
+// (at most 1024) consecutive pairs as k_dispatch does and stores its per-expert counts; once every workgroup
+// has done so (a counter in the workspace tells; all of them are resident, the grid is at most 64) each one adds
+// up the counts of all (the totals, hence the offsets) and of the workgroups before it (where its own pairs of an
+// expert start), and scatters.  The barrier words are zero at launch and are left zero.  A workgroup that waits
+// longer than a second raises the error word and goes on with what it has (positions stay inside the arrays).
+// ---------------------------------------------------------------------------
+#define DISPM_MAXB 64
+__global__ __launch_bounds__(DISP_THREADS) void k_dispatch_multi(
+    const int *__restrict__ idx, int P, int chunk, int k, int E, int nbits, int *__restrict__ counts,
+    int *__restrict__ offsets, int *__restrict__ sorted_pair, int *__restrict__ pos_of_pair,
+    int *__restrict__ sorted_tok, moe_unit *__restrict__ units, int *__restrict__ n_active,
+    long long *__restrict__ active_ids, int max_units, int *hist, unsigned *sync, int *err) {
+  __shared__ int s_base[256], s_all[256], s_pre[256];  // E <= 256 (checked by the launcher)
+  __shared__ int s_wsum[16], s_wact[16], s_tot;
+  extern __shared__ int s_w[];  // [16][E]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int b = blockIdx.x, NB = gridDim.x;
+  // ---- stable rank of the workgroup's pairs among themselves ---------------------------------------
+  const int p0 = b * chunk;
+  const int np = (P - p0) < chunk ? (P - p0) : chunk;
+  const int p = p0 + tid;
+  const int e = tid < np ? idx[p] : -1;
+  for (int i = tid; i < 16 * E; i += DISP_THREADS) s_w[i] = 0;
+  if (tid < 256) { s_all[tid] = 0; s_pre[tid] = 0; }
+  __syncthreads();
+  const bool valid = (unsigned)e < (unsigned)E;
+  unsigned long long peers = __ballot(valid);
+  for (int bit_i = 0; bit_i < nbits; ++bit_i) {
+    const bool bit = (e >> bit_i) & 1;
+    const unsigned long long bal = __ballot(valid && bit);
+    peers &= bit ? bal : ~bal;
+  }
+  const int rank = __popcll(peers & ((1ull << lane) - 1ull));
+  if (valid && rank == 0) s_w[w * E + e] = __popcll(peers);
+  __syncthreads();
+  for (int ee = tid; ee < E; ee += DISP_THREADS) {
+    int run = 0;
+    for (int ww = 0; ww < 16; ++ww) {
+      const int c = s_w[ww * E + ee];
+      s_w[ww * E + ee] = run;
+      run += c;
+    }
+    __hip_atomic_store(hist + (size_t)b * E + ee, run, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  // ---- every workgroup's counts are out ------------------------------------------------------------
+  // (the counts are stored and read at device scope, past the caches that are not coherent between workgroups;
+  // one thread orders them: its release follows the workgroup's barrier, its acquire precedes the next one)
+  __syncthreads();
+  if (tid == 0) {
+    __hip_atomic_fetch_add(sync, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    const long long t_start = wall_clock64();
+    int polls = 0;
+    while (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)NB) {
+      if ((++polls & 63) == 0 && wall_clock64() - t_start > 100000000ll) {  // one second of the 100 MHz counter
+        moe_raise_err(err);
+        break;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+  // ---- totals, the counts of the workgroups in front, exclusive scan over experts (thread e owns expert e) ----
+  {
+    // all NB * E counts are requested at once (a thread per count, then LDS adds): one trip to memory
+    for (int i = tid; i < NB * E; i += DISP_THREADS) {
+      const int cb = __hip_atomic_load(hist + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int bb = i / E, ee = i - bb * E;
+      if (cb) {
+        atomicAdd(&s_all[ee], cb);
+        if (bb < b) atomicAdd(&s_pre[ee], cb);
+      }
+    }
+    __syncthreads();
+    const int c = tid < E ? s_all[tid] : 0, pre = tid < E ? s_pre[tid] : 0;
+    const int a = c > 0 ? 1 : 0;
+    int sc = c, sa = a;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int oc = __shfl_up(sc, d, 64), oa = __shfl_up(sa, d, 64);
+      if (lane >= d) { sc += oc; sa += oa; }
+    }
+    if (lane == 63) { s_wsum[w] = sc; s_wact[w] = sa; }
+    __syncthreads();
+    int bc = 0, ba = 0;
+    for (int i = 0; i < w; ++i) { bc += s_wsum[i]; ba += s_wact[i]; }
+    const int excl = bc + sc - c, uidx = ba + sa - a;
+    if (tid < E) {
+      s_base[tid] = excl + pre;
+      if (b == 0) {
+        counts[tid] = c;
+        offsets[tid] = excl;
+        if (a && uidx < max_units) {
+          moe_unit u; u.expert = tid; u.m = c; u.row0 = excl; u.pad = 0;
+          units[uidx] = u;
+          active_ids[uidx] = tid;
+        }
+      }
+    }
+    if (tid == DISP_THREADS - 1) {
+      const int tot_act = ba + sa;
+      if (b == 0) {
+        offsets[E] = bc + sc;
+        *n_active = tot_act < max_units ? tot_act : max_units;
+      }
+      s_tot = tot_act;
+    }
+    __syncthreads();
+    if (b == 0)
+      for (int u = s_tot + tid; u < max_units; u += DISP_THREADS) {
+        moe_unit z; z.expert = -1; z.m = 0; z.row0 = 0; z.pad = 0;
+        units[u] = z;
+        active_ids[u] = -1;
+      }
+  }
+  if (valid) {
+    const int pos = s_base[e] + s_w[w * E + e] + rank;
+    sorted_pair[pos] = p;
+    pos_of_pair[p] = pos;
+    sorted_tok[pos] = p / k;
+  }
+  // the last workgroup through the barrier clears it for the next launch
+  if (tid == 0) {
+    if (__hip_atomic_fetch_add(sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)NB - 1u) {
+      __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(sync + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
@@ -502,16 +654,16 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
     }
   }
   // ---- who is last? ------------------------------------------------------------------------
-  __threadfence();
+  // (one thread orders the workgroup's logits: its release follows the barrier, and the last workgroup's acquire
+  // precedes the next one; a fence by every wave costs several microseconds of cache write-backs)
   __syncthreads();
   if (tid == 0) {
-    const unsigned prev = atomicAdd(a.counter, 1u);
+    const unsigned prev = __hip_atomic_fetch_add(a.counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     s_last = prev == gridDim.x * gridDim.y - 1u;
+    if (s_last) __hip_atomic_store(a.counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   if (!s_last) return;
-  if (tid == 0) atomicExch(a.counter, 0u);
-  __threadfence();
   route_tail<4>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
 }
 
@@ -1711,33 +1863,38 @@ extern "C" int moe_gate_logits(const void *x, const void *wg, const float *bias,
     return MOE_EINVAL;
   }
   if (T == 0) return MOE_OK;
-  const size_t tile_lds = (size_t)GATE_TT * H * 2;
   // up to 128 tokens a wave per (token, gate row) is faster than the token-tile kernel (8 us against 18 us
   // at 128 tokens, 2048 columns, 64 rows)
-  if (T > 128 && H <= 4096 && tile_lds <= 150 * 1024) {
+  if (T > 128 && H <= 4096) {
+    // about two workgroups per compute unit, and at most 72 KB of gate rows per workgroup so that two fit the LDS
     static bool attr_set = false;
-    if (tile_lds > 64 * 1024 && !attr_set) {
-      if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gate_logits_tile,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                 "hipFuncSetAttribute(k_gate_logits_tile)"))
-        return rc;
+    if (!attr_set) {
+      for (const void *f : {(const void *)k_gate_logits_rows<2>, (const void *)k_gate_logits_rows<4>,
+                            (const void *)k_gate_logits_rows<8>})
+        if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024),
+                                   "hipFuncSetAttribute(k_gate_logits_rows)"))
+          return rc;
       attr_set = true;
     }
-    // enough workgroups to fill the chip: split the gate rows when there are few token tiles
     const int tiles = (T + GATE_TT - 1) / GATE_TT;
-    int split = 1;
-    // (as many workgroups as the chip holds at once: two per CU while the token tile takes at most half the
-    // LDS, else one; more, smaller ones restage the tile for fewer gate rows each: 2048 tokens x 2048 x 64
-    // 38.7 us with 1024 workgroups, 35.1 with 512, 58 with 256; 4096 x 4096 x 8 37.5 / 37.0 / 27.3 us)
-    const int target = tile_lds <= 80 * 1024 ? 512 : 256;
-    while (tiles * split < target && split * 4 < E) split *= 2;
-    const int rows_per_block = (((E + split - 1) / split) + 3) & ~3;
+    int rows_per_block = E;
+    while (rows_per_block > 1 && ((size_t)rows_per_block * H * 2 > 72 * 1024 ||
+                                  (size_t)tiles * ((E + rows_per_block - 1) / rows_per_block) < 512))
+      rows_per_block = (rows_per_block + 1) / 2;
+    const size_t lds = (size_t)rows_per_block * H * 2;
     dim3 grid(tiles, (E + rows_per_block - 1) / rows_per_block);
     moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
-    hipLaunchKernelGGL(k_gate_logits_tile, grid, dim3(256), tile_lds, (hipStream_t)stream, (const uint16_t *)x,
-                       (const uint16_t *)wg, bias, logits, T, H, E, ldl, rows_per_block);
+    if (H <= 1024)
+      hipLaunchKernelGGL(k_gate_logits_rows<2>, grid, dim3(64 * GATE_WAVES), lds, (hipStream_t)stream, (const uint16_t *)x,
+                         (const uint16_t *)wg, bias, logits, T, H, E, ldl, rows_per_block);
+    else if (H <= 2048)
+      hipLaunchKernelGGL(k_gate_logits_rows<4>, grid, dim3(64 * GATE_WAVES), lds, (hipStream_t)stream, (const uint16_t *)x,
+                         (const uint16_t *)wg, bias, logits, T, H, E, ldl, rows_per_block);
+    else
+      hipLaunchKernelGGL(k_gate_logits_rows<8>, grid, dim3(64 * GATE_WAVES), lds, (hipStream_t)stream, (const uint16_t *)x,
+                         (const uint16_t *)wg, bias, logits, T, H, E, ldl, rows_per_block);
     moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
-    return moe_check_launch("k_gate_logits_tile");
+    return moe_check_launch("k_gate_logits_rows");
   }
   dim3 grid((E + 3) / 4, T);
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
@@ -1780,6 +1937,43 @@ extern "C" int moe_dispatch(const int *idx, int T, int k, int E, int *counts, in
                      units, n_active, (long long *)active_ids, max_units);
   moe_ktimer_end(MOE_K_DISPATCH, (hipStream_t)stream);
   return moe_check_launch("k_dispatch");
+}
+
+// Dispatch with a workspace: P = T*k >= 2048 pairs of E <= 256 experts go to k_dispatch_multi (one workgroup per
+// 1024 pairs, at most 64), anything else to moe_dispatch.  The workspace starts with the two barrier words, which
+// must be zero before the first call and are zero again after every call.
+extern "C" int64_t moe_dispatch_workspace_bytes(int T, int k, int E) {
+  const long long P = (long long)T * k;
+  if (T <= 0 || k <= 0 || E <= 0 || E > 256 || P < 2048 || P > (long long)DISPM_MAXB * DISP_THREADS) return 0;
+  const long long nb = (P + DISP_THREADS - 1) / DISP_THREADS;
+  return 64 + nb * E * (long long)sizeof(int);
+}
+
+extern "C" int moe_dispatch_ws(const int *idx, int T, int k, int E, int *counts, int *offsets,
+                               int *sorted_pair, int *pos_of_pair, int *sorted_tok, moe_unit *units,
+                               int *n_active, int64_t *active_ids, int max_units, void *ws, int64_t ws_bytes,
+                               int *err, void *stream) {
+  const int64_t need = moe_dispatch_workspace_bytes(T, k, E);
+  if (need == 0 || !ws || ws_bytes < need || !err)
+    return moe_dispatch(idx, T, k, E, counts, offsets, sorted_pair, pos_of_pair, sorted_tok, units, n_active,
+                        active_ids, max_units, stream);
+  if (!idx || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok || !units || !n_active ||
+      !active_ids || max_units < 0 || ((uintptr_t)ws & 3)) {
+    moe_set_error("moe_dispatch_ws: bad argument (T=%d k=%d E=%d)", T, k, E);
+    return MOE_EINVAL;
+  }
+  const int P = T * k;
+  const int nb = (P + DISP_THREADS - 1) / DISP_THREADS;
+  const int chunk = (P + nb - 1) / nb;
+  int nbits = 0;
+  while ((1 << nbits) < E) ++nbits;
+  const size_t lds = (size_t)16 * E * sizeof(int);
+  moe_ktimer_begin(MOE_K_DISPATCH, (hipStream_t)stream);
+  hipLaunchKernelGGL(k_dispatch_multi, dim3(nb), dim3(DISP_THREADS), lds, (hipStream_t)stream, idx, P, chunk, k, E,
+                     nbits, counts, offsets, sorted_pair, pos_of_pair, sorted_tok, units, n_active,
+                     (long long *)active_ids, max_units, (int *)((char *)ws + 64), (unsigned *)ws, err);
+  moe_ktimer_end(MOE_K_DISPATCH, (hipStream_t)stream);
+  return moe_check_launch("k_dispatch_multi");
 }
 
 template <int TMAX, bool SW, int CH>

@@ -60,13 +60,36 @@ class Dispatch:
         self.units = torch.empty(max(max_units, 1), 4, **i32)
         self.n_active = torch.empty(1, **i32)
         self.active_ids = torch.empty(max(max_units, 1), dtype=torch.int64, device=device)
+        self.err = torch.zeros(1, **i32)
+
+    def check(self):
+        """Raises if the multi-workgroup dispatch kernel reported a time-out (synchronises)."""
+        if int(self.err.item()):
+            raise L.MoeError("moe_dispatch_ws: a workgroup did not get the others' counts in time")
 
 
-def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispatch | None = None) -> Dispatch:
+_dispatch_ws: dict = {}
+
+
+def dispatch(idx: torch.Tensor, E: int, max_units: int | None = None, out: Dispatch | None = None,
+             single_workgroup: bool = False) -> Dispatch:
     T, k = idx.shape
     if max_units is None:
         max_units = min(E, T * k)
     d = out if out is not None else Dispatch(T, k, E, max_units, idx.device)
+    ws_bytes = 0 if single_workgroup else int(lib.moe_dispatch_workspace_bytes(T, k, E))
+    if ws_bytes:
+        # prefill batches: one workgroup per 1024 pairs.  One workspace per device, zeroed when it is made (the
+        # kernel leaves its barrier words zero); calls on a device must not overlap.  d.err is raised by a
+        # workgroup that did not get the others' counts within a second (Dispatch.check reads it).
+        ws = _dispatch_ws.get(idx.device)
+        if ws is None or ws.numel() * 4 < ws_bytes:
+            ws = _dispatch_ws[idx.device] = torch.zeros(ws_bytes // 4 + 1, dtype=torch.int32, device=idx.device)
+        check(lib.moe_dispatch_ws(ptr(_dev(idx)), T, k, E, ptr(d.counts), ptr(d.offsets), ptr(d.sorted_pair),
+                                  ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units), ptr(d.n_active),
+                                  ptr(d.active_ids), max_units, ptr(ws), ws_bytes, ptr(d.err), cur_stream()),
+              "moe_dispatch_ws")
+        return d
     check(lib.moe_dispatch(ptr(_dev(idx)), T, k, E, ptr(d.counts), ptr(d.offsets), ptr(d.sorted_pair),
                            ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units), ptr(d.n_active),
                            ptr(d.active_ids), max_units, cur_stream()), "moe_dispatch")

@@ -7,6 +7,7 @@
 STUB(moe_gate_logits)
 STUB(moe_topk)
 STUB(moe_dispatch)
+STUB(moe_dispatch_ws)
 STUB(moe_route_decode)
 STUB(moe_topk_dispatch)
 STUB(moe_experts_decode_int4)
@@ -17,3 +18,4 @@ STUB(moe_combine)
 STUB(moe_combine_splits)
 extern "C" int moe_decode_shared_splits(...) { return 1; }
 extern "C" int64_t moe_prefill_workspace_bytes(...) { return 0; }
+extern "C" int64_t moe_dispatch_workspace_bytes(...) { return 0; }

@@ -50,18 +50,25 @@ def test_topk_routing(cuda, T, E, k, mode):
     assert np.allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
 
 
-@pytest.mark.parametrize("T,k,E", [(1, 6, 64), (4, 6, 64), (16, 6, 64), (2048, 4, 60), (4096, 2, 8),
-                                   (515, 8, 64), (300, 3, 200), (0, 6, 64)])
-def test_dispatch_bit_exact(cuda, T, k, E):
+@pytest.mark.parametrize("T,k,E,single", [(1, 6, 64, False), (4, 6, 64, False), (16, 6, 64, False),
+                                          (2048, 4, 60, False), (4096, 2, 8, False), (515, 8, 64, False),
+                                          (300, 3, 200, False), (0, 6, 64, False),
+                                          # P >= 2048 pairs, E <= 256: one workgroup per 1024 pairs (ragged last one)
+                                          (342, 6, 64, False), (700, 6, 256, False), (2048, 6, 64, False),
+                                          (10000, 6, 64, False), (8192, 8, 128, False),
+                                          # and the one-workgroup kernel on the same sizes
+                                          (2048, 4, 60, True), (515, 8, 64, True), (700, 6, 300, False)])
+def test_dispatch_bit_exact(cuda, T, k, E, single):
     from promoe_amd import ops
-    print(f"case dispatch T={T} k={k} E={E}", flush=True)
+    print(f"case dispatch T={T} k={k} E={E} single={single}", flush=True)
     rng = np.random.default_rng(T + k + E)
     # distinct experts per token, skewed popularity
     p = 1.0 / np.arange(1, E + 1) ** 1.2
     p /= p.sum()
     idx = np.stack([rng.choice(E, size=k, replace=False, p=p) for _ in range(T)]).astype(np.int32) \
         if T else np.zeros((0, k), np.int32)
-    d = ops.dispatch(torch.from_numpy(idx).to(cuda).reshape(T, k), E)
+    d = ops.dispatch(torch.from_numpy(idx).to(cuda).reshape(T, k), E, single_workgroup=single)
+    d.check()
     counts, offsets, sp, pp = O.dispatch(idx, E)
     P = T * k
     assert np.array_equal(d.counts.cpu().numpy(), counts)
@@ -78,6 +85,33 @@ def test_dispatch_bit_exact(cuda, T, k, E):
     assert np.array_equal(units[:, 2], offsets[act[:n_act]])
     assert np.array_equal(d.active_ids.cpu().numpy()[:n_act], act[:n_act])
     assert np.all(d.units.cpu().numpy()[n_act:d.max_units, 1] == 0)
+
+
+def test_dispatch_workspace_reused(cuda):
+    """Calls that share one workspace: the barrier words are zero again after each call, whatever the grid."""
+    from promoe_amd import ops
+    from promoe_amd._lib import lib, ptr, cur_stream, check
+    E, k = 64, 6
+    ws_bytes = int(lib.moe_dispatch_workspace_bytes(4096, k, E))
+    assert ws_bytes > 0 and int(lib.moe_dispatch_workspace_bytes(300, k, E)) == 0
+    ws = torch.zeros(ws_bytes // 4 + 1, dtype=torch.int32, device=cuda)
+    err = torch.zeros(1, dtype=torch.int32, device=cuda)
+    rng = np.random.default_rng(5)
+    for T in (4096, 400, 2048, 3, 4096):
+        print(f"case dispatch_ws T={T}", flush=True)
+        idx = np.stack([rng.choice(E, size=k, replace=False) for _ in range(T)]).astype(np.int32)
+        d = ops.Dispatch(T, k, E, min(E, T * k), cuda)
+        check(lib.moe_dispatch_ws(ptr(torch.from_numpy(idx).to(cuda)), T, k, E, ptr(d.counts), ptr(d.offsets),
+                                  ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                  ptr(d.n_active), ptr(d.active_ids), d.max_units, ptr(ws), ws_bytes, ptr(err),
+                                  cur_stream()), "moe_dispatch_ws")
+        counts, offsets, sp, pp = O.dispatch(idx, E)
+        assert int(err.item()) == 0
+        assert np.array_equal(d.counts.cpu().numpy(), counts)
+        assert np.array_equal(d.offsets.cpu().numpy(), offsets)
+        assert np.array_equal(d.sorted_pair.cpu().numpy()[:T * k], sp)
+        assert np.array_equal(d.pos_of_pair.cpu().numpy()[:T * k], pp)
+        assert not ws[:16].any().item()
 
 
 def run_layer_gpu(layer, x, k, mode, dev, resident=None, host_units=False):
