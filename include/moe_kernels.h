@@ -159,6 +159,19 @@ int moe_experts_decode_int4(const void *x_bf16, int T, int H, int I, int I_sh, i
                             const moe_unit *units_host, const uint64_t *expert_ptr_host,
                             int phases, void *stream);
 
+/* The same, with the step's unit list sent to the host by the w13 launch (T >= 2, device unit list, phase bit 0):
+ * one more workgroup copies units[0 .. *n_active) and the count into units_host_out / n_active_host_out (pinned
+ * HOST memory) and then, once those stores have completed, stores seq_value into *seq_host_out, while the other
+ * workgroups stream weights.  A routing launch that publishes itself (moe_topk_dispatch with its host arguments)
+ * is held by those stores for about 2 us; here nothing waits for them.  units_host_out NULL: moe_experts_decode_int4. */
+int moe_experts_decode_int4_publish(const void *x_bf16, int T, int H, int I, int I_sh, int k,
+                                    const moe_unit *units, int max_units, const int *sorted_tok,
+                                    const uint64_t *expert_ptr, const void *shared_ptr, void *h_r,
+                                    void *h_s, float *part_r, float *part_s, int *err,
+                                    const moe_unit *units_host, const uint64_t *expert_ptr_host,
+                                    int phases, const int *n_active, moe_unit *units_host_out,
+                                    int *n_active_host_out, int *seq_host_out, int seq_value, void *stream);
+
 /* k1b + k2 + k3 for ONE token: the w13 kernel derives the routing itself from the gate logits
  * (same selection, tie rule and weights as moe_topk, same arrays as moe_dispatch, bit for bit)
  * and publishes it for the w2 pass, moe_combine and the host, so a decode step is

@@ -52,6 +52,8 @@ _sig("moe_dispatch_workspace_bytes", [i32, i32, i32], C.c_int64)
 _sig("moe_dispatch_ws", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, i64, vp, vp])
 _sig("moe_route_decode", [vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp])
 _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
+_sig("moe_experts_decode_int4_publish", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32,
+                                          vp, vp, vp, vp, i32, vp])
 _sig("moe_topk_dispatch", [vp, i32, i32, i32, i32, i32] + [vp] * 10 + [i32, vp, vp, vp, i32, vp])
 _sig("moe_noalloc_scratch_bytes", [], i64)
 _sig("moe_decode_token_int4_noalloc", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp])

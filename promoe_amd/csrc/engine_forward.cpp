@@ -238,9 +238,11 @@ static bool use_prefill(const moe_layer_desc &d, int T) {
   return T > gemv_tmax && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
 }
 
+// pub / pub_seq: the pending slot whose pinned unit list the w13 launch fills (decode_publishes), or null
 static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
                      const moe_unit *units_dev, const moe_unit *units_host, int n_units, bool with_shared,
-                     int layer, const uint64_t *table, hipStream_t st) {
+                     int layer, const uint64_t *table, hipStream_t st, LayerState::Pending *pub = nullptr,
+                     int pub_seq = 0) {
   if (use_prefill(d, T))
     return moe_experts_prefill(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
                                s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
@@ -251,9 +253,16 @@ static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, co
                                   s->part_r, s->part_s, s->err_host + layer, 3, st);
   // the host knows the units and the slot addresses: they travel in the kernel arguments
   const uint64_t *table_host = units_host ? eng->h_table + (size_t)layer * eng->cfg.num_expert : nullptr;
-  return moe_experts_decode_int4(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
-                                 s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
-                                 s->part_r, s->part_s, s->err_host + layer, units_host, table_host, 3, st);
+  return moe_experts_decode_int4_publish(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
+                                         s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
+                                         s->part_r, s->part_s, s->err_host + layer, units_host, table_host, 3,
+                                         s->n_active, pub ? pub->units : nullptr, pub ? pub->n_active : nullptr,
+                                         pub ? pub->seq : nullptr, pub_seq, st);
+}
+
+// a decode batch whose w13 launch can send the unit list to the host itself (int4 GEMV kernels, 2 tokens and more)
+static bool decode_publishes(const moe_layer_desc &d, int T, int max_units) {
+  return d.fmt == MOE_FMT_INT4_G128 && T >= 2 && !use_prefill(d, T) && max_units > 0 && d.I > 0;
 }
 
 // pieces the expert launch of run_units leaves the shared expert's partial rows in
@@ -452,7 +461,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
   }
-  bool routed_by_tail = false;
+  bool routed_by_tail = false, w13_publishes = false;
   int tail_seq = 0;
   if (all_resident && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
@@ -468,9 +477,13 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     LayerState::Pending &pn = s->pend[s->pend_head];
     if (pn.busy && (rc = moe_forward_harvest(eng, true))) return rc;
     tail_seq = ++s->seq_counter;
+    // the unit list reaches the host from the w13 launch where that one can carry it (its stores to pinned memory
+    // hold the routing launch for about 2 us, and nothing in the w13 launch waits for them), else from here
+    w13_publishes = decode_publishes(d, T, max_units);
     if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
                                 s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                max_units, pn.units, pn.n_active, pn.seq, tail_seq, st)))
+                                max_units, w13_publishes ? nullptr : pn.units, w13_publishes ? nullptr : pn.n_active,
+                                w13_publishes ? nullptr : pn.seq, tail_seq, st)))
       return rc;
     routed_by_tail = true;
   } else if (T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
@@ -514,7 +527,9 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
-    if ((rc = run_units(eng, d, s, x, T, s->units, nullptr, max_units, d.I_sh > 0, layer, table, st))) return rc;
+    if ((rc = run_units(eng, d, s, x, T, s->units, nullptr, max_units, d.I_sh > 0, layer, table, st,
+                        w13_publishes ? &p : nullptr, tail_seq)))
+      return rc;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k,
                                  shared_pieces(d, T), st)))

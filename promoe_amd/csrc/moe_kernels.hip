@@ -714,6 +714,10 @@ struct GemvArgs {
   moe_unit *r_units; int *r_n_active; long long *r_active_ids;
   // optional copy of the unit list straight into pinned host memory, then a sequence word
   moe_unit *r_host_units; int *r_host_seq; int r_host_seq_val, r_pad2;
+  // w13 launches of a decode batch can carry the step's unit list (made by an earlier launch) to the host:
+  // one more workgroup at the end of the grid copies it into pinned host memory and then stores the sequence word
+  moe_unit *p_host_units; int *p_host_n_active; int *p_host_seq; const int *p_n_active;
+  int p_seq_val, p_max_units;
   KUnit *r_kunits;              // routing publisher: resolved units (slot address, rows) for the w2 pass
   float *r_unit_w;              // and the routing weight per unit position
   const KUnit *kunits_dev;      // device-side resolved units: one load instead of unit -> table -> address
@@ -728,18 +732,36 @@ struct GemvWork {
   const unsigned char *base;
   int m, row0, b;
 };
+// The publishing workgroup of a w13 launch (the last one of its grid): the unit list of the step goes from device
+// memory to the host's pinned copy while the other workgroups stream weights, then the sequence word the host
+// polls.  In the routing kernel itself these stores held the launch for 1.8 us; here nothing waits for them.
+static __device__ __forceinline__ void gemv_publish_units(const GemvArgs &a) {
+  const int tid = threadIdx.x;
+  int n = *a.p_n_active;
+  n = n < a.p_max_units ? n : a.p_max_units;
+  for (int u = tid; u < n; u += 256) {
+    const moe_unit un = a.units[u];
+    host_store_unit(a.p_host_units, u, un.expert, un.m, un.row0);
+  }
+  if (tid == 0) host_store_i32(a.p_host_n_active, n);
+  host_stores_done();
+  __syncthreads();
+  if (tid == 0) __hip_atomic_store(a.p_host_seq, a.p_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// bx: the workgroup's index among the working ones (launches with a publishing workgroup put that one first)
 template <bool DEVUNITS>
-static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a) {
+static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const int bx) {
   GemvWork wk;
   const GemvClass c0 = a.cls[0], c1 = a.cls[1];
   const int n_sh = a.n_sh_blocks;
-  const bool sh = (int)blockIdx.x < n_sh;
+  const bool sh = bx < n_sh;
   GemvClass &c = wk.c;
   c.act = sh ? c0.act : c1.act; c.gather = sh ? c0.gather : c1.gather; c.out = sh ? c0.out : c1.out;
   c.off_q = sh ? c0.off_q : c1.off_q; c.off_s = sh ? c0.off_s : c1.off_s; c.off_z = sh ? c0.off_z : c1.off_z;
   c.K = sh ? c0.K : c1.K; c.G = sh ? c0.G : c1.G; c.act_stride = sh ? c0.act_stride : c1.act_stride;
   c.out_stride = sh ? c0.out_stride : c1.out_stride; c.nblk = sh ? c0.nblk : c1.nblk; c.ksplit = sh ? c0.ksplit : c1.ksplit;
-  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
+  const int rr = sh ? bx : bx - n_sh;
   const int u = sh ? 0 : rr / c.nblk;
   wk.b = rr - u * c.nblk;
   if (DEVUNITS) {
@@ -948,7 +970,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  const GemvWork wk = ROUTE ? gemv_resolve_route(a, lane, w) : gemv_resolve<DEVUNITS>(a);
+  const GemvWork wk = ROUTE ? gemv_resolve_route(a, lane, w) : gemv_resolve<DEVUNITS>(a, (int)blockIdx.x);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -1349,7 +1371,14 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
+  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
+  if (publishes && blockIdx.x == 0) {
+    gemv_publish_units(a);
+    return;
+  }
+  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -1360,7 +1389,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   }
   const int K = c.K, G = c.G;
   // block pairs of this workgroup: the shared expert sees every token, so its workgroups take fewer
-  const int RPW = (int)blockIdx.x < a.n_sh_blocks ? RPW_S : RPW_R;
+  const int RPW = bx < a.n_sh_blocks ? RPW_S : RPW_R;
   const int XS = K * 2 + 16;  // padded row stride (bytes): 16 token rows hit 16 distinct bank quads
   unsigned char *xs = smem;                                           // [TB][XS]
   float *xsum = (float *)(smem + (size_t)TB * XS);                    // [TB][G]
@@ -1569,7 +1598,14 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   const int r = lane & 15, qd = lane >> 4;
   const int kh = w % KS;  // which part of every chunk this wave takes
 
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a);
+  // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
+  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
+  if (publishes && blockIdx.x == 0) {
+    gemv_publish_units(a);
+    return;
+  }
+  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -2079,7 +2115,7 @@ static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t ld
     while (rpw_s < rpw && a.cls[0].nblk % (rpw_s * 2) == 0) rpw_s *= 2;
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= rpw_s; a.n_sh_blocks /= rpw_s; }
   a.cls[1].nblk /= rpw;
-  const int grid = a.n_sh_blocks + units * a.cls[1].nblk;
+  const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma<SW, CH, true>,
@@ -2117,7 +2153,7 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   }
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
   a.cls[1].nblk /= PW;
-  const int grid = a.n_sh_blocks + units * a.cls[1].nblk;
+  const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
   const size_t lds = gemv_mfma_kc_lds(NT, CG);
   static bool attr_set = false;
   if (!attr_set) {
@@ -2207,6 +2243,25 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                                        void *h_r, void *h_s, float *part_r, float *part_s,
                                        int *err, const moe_unit *units_host,
                                        const uint64_t *expert_ptr_host, int phases, void *stream) {
+  return moe_experts_decode_int4_publish(x, T, H, I, I_sh, k, units, max_units, sorted_tok, expert_ptr, shared_ptr, h_r,
+                                         h_s, part_r, part_s, err, units_host, expert_ptr_host, phases, nullptr,
+                                         nullptr, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int I, int I_sh, int k,
+                                               const moe_unit *units, int max_units, const int *sorted_tok,
+                                               const uint64_t *expert_ptr, const void *shared_ptr,
+                                               void *h_r, void *h_s, float *part_r, float *part_s,
+                                               int *err, const moe_unit *units_host,
+                                               const uint64_t *expert_ptr_host, int phases,
+                                               const int *n_active, moe_unit *units_host_out, int *n_active_host_out,
+                                               int *seq_host_out, int seq_value, void *stream) {
+  if (units_host_out && (T < 2 || !units || units_host || !n_active || !n_active_host_out || !seq_host_out ||
+                         !(phases & 1) || max_units <= 0)) {
+    moe_set_error("moe_experts_decode_int4_publish: publishing needs T >= 2, the device unit list, its length and "
+                  "the w13 phase (T=%d phases=%d)", T, phases);
+    return MOE_EINVAL;
+  }
   if (!x || T <= 0 || H <= 0 || H % 128 || I < 0 || I % 128 || I_sh < 0 || I_sh % 128 || !err ||
       (max_units > 0 && ((!units && !units_host) || !sorted_tok || (!expert_ptr && !expert_ptr_host) || !h_r || !part_r || I == 0)) ||
       (shared_ptr && (!h_s || !part_s || I_sh == 0))) {
@@ -2232,6 +2287,10 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
       a.ku[u].m = h.m; a.ku[u].row0 = h.row0;
       a.ku[u].base = (h.m > 0 && h.expert >= 0) ? expert_ptr_host[h.expert] : 0;
     }
+  }
+  if (units_host_out) {
+    a.p_host_units = units_host_out; a.p_host_n_active = n_active_host_out; a.p_host_seq = seq_host_out;
+    a.p_n_active = n_active; a.p_seq_val = seq_value; a.p_max_units = max_units;
   }
   // pass 1: w13 + SwiGLU
   // one token: every row reads activation row 0 (stride 0), no gather load on the critical path

@@ -107,6 +107,8 @@ class PrefetchMngr:
         self._h = h
         self._keep = []   # host buffers registered with the engine
         self.backend = backend
+        self._compute_stream_handle = None
+        self._ext_stream = None
 
     def close(self):
         if getattr(self, "_h", None) and lib is not None:
@@ -305,11 +307,30 @@ class PrefetchMngr:
     def forward_prepare(self, max_tokens: int):
         check(lib.moe_forward_prepare(self._h, max_tokens), "forward_prepare")
 
-    def forward(self, layer_id: int, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, layer_id: int, x: torch.Tensor, out: torch.Tensor | None = None,
+                stream_guard: bool = True) -> torch.Tensor:
+        """One MoE layer on the engine's compute stream.  Created from torch's legacy default stream (handle 0)
+        the engine has a private non-blocking stream, as the reference has (prefetcher.cpp:407-413); callers are
+        meant to make it torch's current stream (utils/__init__.py:293; `hf.inject_model` does).  When torch's
+        current stream is another one, stream_guard orders the two around the call (x is complete before the
+        kernels read it, the output before torch uses it); a caller that has synchronised itself passes False."""
         assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous()
         if out is None:
             out = torch.empty_like(x)
+        guard = None
+        if stream_guard and self.backend == L.BACKEND_HIP:
+            cur = torch.cuda.current_stream(x.device)
+            cs = self._compute_stream_handle
+            if cs is None:
+                cs = self._compute_stream_handle = self.compute_stream
+            if cur.cuda_stream != cs:
+                if self._ext_stream is None:
+                    self._ext_stream = torch.cuda.ExternalStream(cs, device=x.device)
+                guard = (cur, self._ext_stream)
+                guard[1].wait_stream(cur)
         check(lib.moe_forward(self._h, layer_id, x.data_ptr(), x.shape[0], out.data_ptr()), "moe_forward")
+        if guard is not None:
+            guard[0].wait_stream(guard[1])
         return out
 
     def last_routing(self):

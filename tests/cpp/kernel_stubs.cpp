@@ -11,6 +11,7 @@ STUB(moe_dispatch_ws)
 STUB(moe_route_decode)
 STUB(moe_topk_dispatch)
 STUB(moe_experts_decode_int4)
+STUB(moe_experts_decode_int4_publish)
 STUB(moe_decode_token_int4)
 STUB(moe_experts_decode_q4k)
 STUB(moe_experts_prefill)

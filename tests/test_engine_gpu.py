@@ -335,3 +335,54 @@ def test_one_token_path_under_wrong_prefetches(cuda):
           flush=True)
     assert worst <= TOL
     assert c["prefetch_miss"] > 0 and c["evictions"] > 0 and c["miss"] > 0
+
+
+@pytest.mark.parametrize("cached", [False, True])
+def test_engines_without_a_synchronisation_per_call(cuda, cached):
+    """Forwards issued back to back, nothing synchronised in between, inputs made by torch right before the
+    call on torch's own stream: a second engine over the same layers must give the first one's outputs.
+    cached = False: both hold every expert (bit-identical outputs; this is what the stream guard of
+    PrefetchMngr.forward is for: from the default stream each engine has a private compute stream).
+    cached = True: the second one runs at cache rate 0.3 with a predictor whose models are right for half of
+    the layer pairs and random for the other half, so demand fetches, prefetches and evictions go on under the
+    kernels of both.  MOE_SOAK_STEPS lengthens the run (30000 steps = 120000 forwards were run this way)."""
+    import os
+    print(f"case engine_async cached={cached}", flush=True)
+    steps = int(os.environ.get("MOE_SOAK_STEPS", "400"))
+    Lyr, E, k, H, I, I_sh = 4, 32, 4, 1024, 512, 512
+    layers = [Int4Layer(H=H, I=I, E=E, I_sh=I_sh, seed=70 + l, zipf=1.1) for l in range(Lyr)]
+    A = build_engine(layers, k, cuda, cache_rate=1.0, cache_policy="lru")
+    if cached:
+        B = build_engine(layers, k, cuda, cache_rate=0.3, cache_policy="lru", num_predict_expert_per_layer=k,
+                         layer_predict_interval=1, layer_predict_max_window=2, limit_layer_0_window=2)
+        g = torch.Generator().manual_seed(5)
+        for src, (a, b) in enumerate(B.predictor_windows()):
+            for dst in range(a, b):
+                m = (torch.from_numpy(layers[dst].wg) if (src + dst) % 2 else torch.randn(E, H, generator=g))
+                B.set_predictor_model(src, dst, m.to(torch.bfloat16).to(cuda), None)
+        B.start_predictor()
+    else:
+        B = build_engine(layers, k, cuda, cache_rate=1.0, cache_policy="lru")
+    rng = np.random.default_rng(0)
+    gx = torch.Generator(device=cuda).manual_seed(100)
+    pend, worst = [], 0.0
+    for s in range(steps):
+        T = int(rng.choice([1, 1, 1, 1, 1, 1, 2, 4, 16, 40]))
+        for l in range(Lyr):
+            x = torch.randn(T, H, device=cuda, generator=gx).to(torch.bfloat16)
+            pend.append((s, l, T, A.forward(l, x), B.forward(l, x)))
+        if s % 100 == 99 or s == steps - 1:
+            torch.cuda.synchronize()
+            for (s_, l_, T_, ya, yb) in pend:
+                a, b = ya.float(), yb.float()
+                err = float((a - b).abs().max() / a.abs().max().clamp_min(1e-6))
+                assert err <= (1e-2 if cached else 0.0), f"step {s_} layer {l_} T {T_}: {err:.3e}"
+                worst = max(worst, err)
+            pend = []
+    A.drain(); B.drain()
+    c = B.counters()
+    A.close(); B.close()
+    print(f"  {steps} steps, worst {worst:.2e}, misses {c['miss']}, prefetch hits {c['prefetch_hit']}, "
+          f"evictions {c['evictions']}", flush=True)
+    if cached:
+        assert c["miss"] > 0 and c["evictions"] > 0 and c["prefetch_hit"] > 0
