@@ -87,6 +87,14 @@ int moe_q4k_layout_make(int H, int I, moe_int4_layout *out);
 int moe_gate_logits(const void *x_bf16, const void *wg_bf16, const float *bias, float *logits,
                     int T, int H, int E, int ldl, void *stream);
 
+/* moe_gate_logits for two matrices over the same activations in ONE launch (T <= 128): wg [E, H] (+ bias) into
+ * logits (row stride ldl), wg2 [E2, H] (+ bias2) into logits2 (row stride ldl2); the same bits as two calls.
+ * The engine uses it to let the built-in predictor's score rows (engine_predict.cpp; the reference evaluates its
+ * per-pair models in PredictWorker, worker.cpp:6-77) ride in the layer's own gate launch. */
+int moe_gate_logits_pair(const void *x_bf16, const void *wg_bf16, const float *bias, float *logits, int T, int H,
+                         int E, int ldl, const void *wg2_bf16, const float *bias2, float *logits2, int E2,
+                         int ldl2, void *stream);
+
 /* k1b: top-k routing.  Selection on the logits, ties toward the lower expert index.
  * idx [T,k] int32, w [T,k] fp32.  E <= 256, k <= 32. */
 int moe_topk(const float *logits, int T, int E, int ldl, int k, int mode, int *idx, float *w,

@@ -46,6 +46,7 @@ def _sig(name, argtypes, restype=i32):
 _sig("moe_last_error", [], C.c_char_p)
 _sig("moe_int4_layout_make", [i32, i32, C.POINTER(Int4Layout)])
 _sig("moe_gate_logits", [vp, vp, vp, vp, i32, i32, i32, i32, vp])
+_sig("moe_gate_logits_pair", [vp, vp, vp, vp, i32, i32, i32, i32, vp, vp, vp, i32, i32, vp])
 _sig("moe_topk", [vp, i32, i32, i32, i32, i32, vp, vp, vp])
 _sig("moe_dispatch", [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
 _sig("moe_dispatch_workspace_bytes", [i32, i32, i32], C.c_int64)

@@ -845,13 +845,16 @@ extern "C" int moe_expert_num_ready(moe_engine *eng, int layer, int expert) {
 // ---------------------------------------------------------------------------
 // hook sequence
 // ---------------------------------------------------------------------------
-extern "C" int moe_report_layer_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H) {
+int moe_report_layer_logits_bookkeeping(moe_engine *eng, int layer, int S) {
   ENG_GUARD(eng);
   if (layer < 0 || layer > eng->cfg.num_layer) { moe_set_error("bad layer %d", layer); return MOE_EINVAL; }
-  {
-    std::lock_guard<std::mutex> lk(eng->mu);
-    if (layer == 0) eng->s_seqlen.push_back((uint64_t)S);  // prefetcher.cpp:452-455
-  }
+  std::lock_guard<std::mutex> lk(eng->mu);
+  if (layer == 0) eng->s_seqlen.push_back((uint64_t)S);  // prefetcher.cpp:452-455
+  return MOE_OK;
+}
+
+extern "C" int moe_report_layer_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H) {
+  if (int rc = moe_report_layer_logits_bookkeeping(eng, layer, S)) return rc;
   return moe_predictor_on_logits(eng, layer, hidden, B, S, H);  // prefetcher.cpp:451-452
 }
 

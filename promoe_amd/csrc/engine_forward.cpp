@@ -293,7 +293,14 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // hook order of the reference (utils/hooks.py:216-223)
   // the layer hook's pre_forward: this block's input (decode: what the built-in predictor reads)
   if ((rc = moe_forward_check_kernels(eng))) return rc;  // of earlier calls: the words arrive without a copy
-  if ((rc = moe_report_layer_logits(eng, layer, x, 1, T, d.H))) return rc;
+  // (a one-token step that will launch its gate kernel below takes the predictor's score rows into that launch)
+  const bool token_kernels = T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 &&
+                             eng->cfg.early_preempt && eng->cfg.reorder_experts && (size_t)d.H * 2 + 8192 <= 60 * 1024;
+  const void *pred_w = nullptr; const float *pred_b = nullptr; float *pred_out = nullptr; int pred_rows = 0;
+  bool pred_fused = token_kernels && moe_predictor_fused_rows(eng, layer, d.H, &pred_w, &pred_b, &pred_out, &pred_rows);
+  if (pred_fused) {
+    if ((rc = moe_report_layer_logits_bookkeeping(eng, layer, T))) return rc;
+  } else if ((rc = moe_report_layer_logits(eng, layer, x, 1, T, d.H))) return rc;
   const int max_units = (int)std::min<size_t>(E, (size_t)T * k);
   if ((rc = moe_forward_harvest(eng, false))) return rc;
   // Every expert of the layer resident, and the layer's slot group can hold them all: there
@@ -346,10 +353,21 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // reference's order (hits were computed already, misses are fetched and computed one by one) while the GPU
   // works.  From the table snapshot until the hooks have marked the hits, the layer's slot group is guarded:
   // prefetch and demand traffic may evict, but no copy into one of its slots starts.
-  const bool optimistic = !all_resident && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 &&
-                          eng->cfg.early_preempt && eng->cfg.reorder_experts && (size_t)d.H * 2 + 8192 <= 60 * 1024;
+  const bool optimistic = !all_resident && token_kernels;
+  if (pred_fused && !optimistic) {  // (cannot happen while a predictor rules out the all-resident short cut)
+    pred_fused = false;
+    if ((rc = moe_predictor_on_logits(eng, layer, x, 1, T, d.H))) return rc;
+  }
   if (optimistic) {
-    if (!d.gate_bias) {
+    const int rows1 = d.gate_bias ? E : n_gate_rows;
+    if (pred_fused) {
+      if ((rc = moe_gate_logits_pair(x, d.gate_w, d.gate_bias, s->logits, T, d.H, rows1, ldl, pred_w, pred_b, pred_out,
+                                     pred_rows, pred_rows, st)))
+        return rc;
+      if (d.gate_bias && d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    } else if (!d.gate_bias) {
       if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
     } else {
       if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
@@ -374,6 +392,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                     s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
                                     nullptr, nullptr, st)))
       return rc;
+    // the predictor's scores came out of the gate launch above: complete once this kernel's sequence word arrives
+    if (pred_fused && (rc = moe_predictor_scores_pending(eng, layer, s->opt_seq, seq))) return rc;
     // The w2 pass with the combine goes out at once as well, as if nothing were missing: in most steps nothing
     // is, and then the GPU has this layer's kernels queued while the host runs the hooks and is never waited
     // for.  When an expert turns out to be missing, its output is recomputed below (the kernel skips the

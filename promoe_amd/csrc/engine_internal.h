@@ -226,6 +226,10 @@ int engine_fail(moe_engine *eng, const char *fmt, ...) __attribute__((format(pri
 void moe_forward_free(LayerState *);
 void moe_predictor_free(moe_engine *eng);
 int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H);
+bool moe_predictor_fused_rows(moe_engine *eng, int layer, int H, const void **w, const float **bias, float **out, int *rows);
+int moe_predictor_scores_pending(moe_engine *eng, int layer, const int *seq_word, int seq_value);
+// moe_report_layer_logits without the predictor's part (the caller runs that part itself)
+int moe_report_layer_logits_bookkeeping(moe_engine *eng, int layer, int S);
 // launching -> using without an event: the experts count as in use until *seq_ptr reaches seq_need
 // slot table of `layer` to the device (if changed) and the same residency as a byte vector, taken in one
 // critical section together with raising the group's guard; moe_guard_release lowers it again

@@ -23,7 +23,12 @@
 #include "moe_kernels.h"
 
 struct PredictModel { const void *w = nullptr; const float *bias = nullptr; };
-struct PredictJob { int src = 0; int seq_len = 0; };
+struct PredictJob {
+  int src = 0; int seq_len = 0;
+  // scores written by a launch the caller queued itself: they are complete once *seq_word has reached seq_value
+  // (a later kernel of the stream stores it when it starts); no event
+  const volatile int *seq_word = nullptr; int seq_value = 0;
+};
 
 struct PredictorState {
   std::vector<std::pair<int, int>> window;          // [L + 1]: destination layers [first, second) of source l
@@ -132,7 +137,21 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
     }
     const auto win = p->window[job.src];
     bool decode = job.seq_len == 1;
-    if (decode && !p->host_math && eng->be->event_sync(p->events[job.src]) != 0) { predictor_fail(eng, p, "event"); decode = false; }
+    if (decode && job.seq_word) {
+      const auto t0 = std::chrono::steady_clock::now();
+      unsigned spins = 0;
+      while (*job.seq_word - job.seq_value < 0) {
+        if ((++spins & 255u) == 0) {
+          if (std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) {  // not within 2 ms: the stream itself
+            if (hipStreamSynchronize((hipStream_t)eng->be->compute_stream()) != hipSuccess) { predictor_fail(eng, p, "stream"); decode = false; }
+            break;
+          }
+          std::lock_guard<std::mutex> lk(p->mu);
+          if (p->exit) return;
+        }
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    } else if (decode && !p->host_math && eng->be->event_sync(p->events[job.src]) != 0) { predictor_fail(eng, p, "event"); decode = false; }
     for (int dst = win.first; dst < win.second; ++dst) {
       int64_t n = 0;
       if (decode) {  // prefill: an empty request per layer keeps the progress count in step (predictor.cpp:513-517)
@@ -266,6 +285,38 @@ int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int 
     std::lock_guard<std::mutex> lk(p->mu);
     if (!p->error.empty()) { moe_set_error("predictor thread: %s", p->error.c_str()); return MOE_ESTATE; }
     p->q.push_back(PredictJob{layer, decode ? 1 : std::max(S, 2)});
+  }
+  p->cv.notify_all();
+  return MOE_OK;
+}
+
+// A one-token forward that launches the gate-logits kernel itself can take the window's score rows into that
+// launch (moe_gate_logits_pair): this hands out the stacked models of `layer` and where their scores go.  False:
+// nothing to fuse (no predictor, the host backend, an empty window, another hidden width).
+bool moe_predictor_fused_rows(moe_engine *eng, int layer, int H, const void **w, const float **bias, float **out, int *rows) {
+  PredictorState *p = eng->pred;
+  if (!p || !p->started || p->host_math || layer < 0 || layer >= (int)p->window.size()) return false;
+  const auto win = p->window[layer];
+  if (win.first >= win.second || H != p->H || !p->stack_w[layer]) return false;
+  const int E = eng->cfg.num_expert;
+  *w = p->stack_w[layer];
+  *bias = p->stack_b[layer];
+  *out = p->scores_dev + (size_t)layer * p->max_win * E;
+  *rows = (win.second - win.first) * E;
+  return true;
+}
+
+// ... and this queues the job: the scores are complete once *seq_word has reached seq_value, which a later kernel
+// of the same stream stores into pinned memory when it starts.  The thread polls that word instead of waiting for
+// an event, which would cost the stream a few microseconds per step.
+int moe_predictor_scores_pending(moe_engine *eng, int layer, const int *seq_word, int seq_value) {
+  PredictorState *p = eng->pred;
+  if (!p || !p->started) return MOE_OK;
+  {
+    std::lock_guard<std::mutex> lk(p->mu);
+    if (!p->error.empty()) { moe_set_error("predictor thread: %s", p->error.c_str()); return MOE_ESTATE; }
+    PredictJob j; j.src = layer; j.seq_len = 1; j.seq_word = seq_word; j.seq_value = seq_value;
+    p->q.push_back(j);
   }
   p->cv.notify_all();
   return MOE_OK;

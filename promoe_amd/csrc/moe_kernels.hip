@@ -14,13 +14,23 @@
 // ---------------------------------------------------------------------------
 // k1a gate logits: one wave per (token, expert row)
 // ---------------------------------------------------------------------------
+// (wg2, bias2, logits2, E2, ldl2: a second matrix over the same activations whose rows follow the first one's in
+// the grid, or E2 = 0: the built-in predictor's score rows ride in the layer's own gate launch)
 __global__ __launch_bounds__(256) void k_gate_logits(const uint16_t *__restrict__ x,
                                                       const uint16_t *__restrict__ wg,
                                                       const float *__restrict__ bias,
                                                       float *__restrict__ logits, int H, int E,
-                                                      int ldl) {
+                                                      int ldl, const uint16_t *__restrict__ wg2,
+                                                      const float *__restrict__ bias2,
+                                                      float *__restrict__ logits2, int E2, int ldl2) {
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int e = blockIdx.x * 4 + w, t = blockIdx.y;
+  int e = blockIdx.x * 4 + w;
+  const int t = blockIdx.y;
+  const int nb1 = (E + 3) >> 2;
+  if ((int)blockIdx.x >= nb1) {  // uniform per workgroup
+    e = ((int)blockIdx.x - nb1) * 4 + w;
+    wg = wg2; bias = bias2; logits = logits2; E = E2; ldl = ldl2;
+  }
   if (e >= E) return;
   const uint16_t *xr = x + (size_t)t * H;
   const uint16_t *wr = wg + (size_t)e * H;
@@ -1935,7 +1945,26 @@ extern "C" int moe_gate_logits(const void *x, const void *wg, const float *bias,
   dim3 grid((E + 3) / 4, T);
   moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
   hipLaunchKernelGGL(k_gate_logits, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
-                     (const uint16_t *)wg, bias, logits, H, E, ldl);
+                     (const uint16_t *)wg, bias, logits, H, E, ldl, (const uint16_t *)nullptr, (const float *)nullptr,
+                     (float *)nullptr, 0, 0);
+  moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
+  return moe_check_launch("k_gate_logits");
+}
+
+// Two matrices over the same activations in one launch (decode batches, T <= 128): rows of wg into logits, rows
+// of wg2 into logits2, each (token, row) sum with the bits of moe_gate_logits.
+extern "C" int moe_gate_logits_pair(const void *x, const void *wg, const float *bias, float *logits, int T, int H,
+                                    int E, int ldl, const void *wg2, const float *bias2, float *logits2, int E2,
+                                    int ldl2, void *stream) {
+  if (!x || !wg || !logits || !wg2 || !logits2 || T <= 0 || T > 128 || H <= 0 || H % 8 || E <= 0 || ldl < E ||
+      E2 <= 0 || ldl2 < E2) {
+    moe_set_error("moe_gate_logits_pair: bad argument (T=%d H=%d E=%d E2=%d)", T, H, E, E2);
+    return MOE_EINVAL;
+  }
+  dim3 grid((E + 3) / 4 + (E2 + 3) / 4, T);
+  moe_ktimer_begin(MOE_K_GATE, (hipStream_t)stream);
+  hipLaunchKernelGGL(k_gate_logits, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
+                     (const uint16_t *)wg, bias, logits, H, E, ldl, (const uint16_t *)wg2, bias2, logits2, E2, ldl2);
   moe_ktimer_end(MOE_K_GATE, (hipStream_t)stream);
   return moe_check_launch("k_gate_logits");
 }

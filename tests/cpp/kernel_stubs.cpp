@@ -5,6 +5,7 @@
 
 #define STUB(name) extern "C" int name(...) { fprintf(stderr, "kernel entry " #name " called in the host-only build\n"); return -1; }
 STUB(moe_gate_logits)
+STUB(moe_gate_logits_pair)
 STUB(moe_topk)
 STUB(moe_dispatch)
 STUB(moe_dispatch_ws)
