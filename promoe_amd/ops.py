@@ -35,6 +35,17 @@ def gate_logits(x: torch.Tensor, wg: torch.Tensor, bias: torch.Tensor | None = N
     return out
 
 
+def gate_logits_pair(x: torch.Tensor, wg: torch.Tensor, bias, wg2: torch.Tensor, bias2):
+    """Two matrices over the same activations in one launch (T <= 128): (logits [T,E], logits2 [T,E2])."""
+    T, H = x.shape
+    E, E2 = wg.shape[0], wg2.shape[0]
+    out = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    out2 = torch.empty(T, E2, dtype=torch.float32, device=x.device)
+    check(lib.moe_gate_logits_pair(ptr(_dev(x)), ptr(_dev(wg)), ptr(bias), ptr(out), T, H, E, E, ptr(_dev(wg2)),
+                                   ptr(bias2), ptr(out2), E2, E2, cur_stream()), "moe_gate_logits_pair")
+    return out, out2
+
+
 def topk(logits: torch.Tensor, k: int, mode: int = L.ROUTE_SOFTMAX_TOPK, E: int | None = None):
     T = logits.shape[0]
     E = logits.shape[1] if E is None else E

@@ -33,6 +33,19 @@ def test_gate_logits_bit_exact(cuda, T, H, E):
     assert np.allclose(got, (x.astype(np.float64) @ wg.astype(np.float64).T), rtol=0, atol=1e-4)
 
 
+@pytest.mark.parametrize("T,H,E,E2", [(1, 2048, 65, 640), (1, 2048, 64, 192), (3, 256, 8, 5), (16, 4096, 8, 70)])
+def test_gate_logits_pair_bit_exact(cuda, T, H, E, E2):
+    """Two matrices in one launch (the predictor's score rows behind the gate's): the bits of two launches."""
+    from promoe_amd import ops
+    print(f"case gate_logits_pair T={T} H={H} E={E} E2={E2}", flush=True)
+    x = bf16_dev(O.synth_acts(T, H, seed=4), cuda)
+    wg = bf16_dev(O.round_bf16(O.synth_weights((E, H), seed=5)), cuda)
+    wg2 = bf16_dev(O.round_bf16(O.synth_weights((E2, H), seed=6)), cuda)
+    b2 = torch.from_numpy(np.linspace(-1, 1, E2).astype(np.float32)).to(cuda)
+    a, b = ops.gate_logits_pair(x, wg, None, wg2, b2)
+    assert torch.equal(a, ops.gate_logits(x, wg)) and torch.equal(b, ops.gate_logits(x, wg2, b2))
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 @pytest.mark.parametrize("T,E,k", [(1, 64, 6), (16, 64, 6), (33, 60, 4), (5, 8, 2), (9, 64, 8), (4, 200, 8)])
 def test_topk_routing(cuda, T, E, k, mode):
