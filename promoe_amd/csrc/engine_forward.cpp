@@ -470,7 +470,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       if ((rc = moe_flush_table(eng, layer, st))) return rc;
       moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
       *slot_h = unit_of[(int)id];
-      HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
+      // (an int4 decode launch of one unit takes it in the kernel arguments: no device copy of the unit)
       if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
       s->sub_cursor++;
       if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
@@ -482,7 +482,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     return moe_layer_done(eng, layer);
   }
   bool routed_by_tail = false, w13_publishes = false;
-  int tail_seq = 0;
+  int tail_seq = 0, host_seq = 0;  // host_seq != 0: the unit list comes to units_host with this value in *opt_seq
   if (all_resident && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory
@@ -506,6 +506,23 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                                 w13_publishes ? nullptr : pn.seq, tail_seq, st)))
       return rc;
     routed_by_tail = true;
+  } else if (T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
+    // decode batch whose routing the host has to see before it can go on (experts may be missing): logits, then
+    // top-k + dispatch in one launch that stores the unit list into pinned host memory and, behind it, a sequence
+    // word; the host polls the word below.  Two copies, an event and a blocking wait for it took 15-20 us per step.
+    if (!d.gate_bias) {
+      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+    } else {
+      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+      if (d.shared_gated &&
+          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+        return rc;
+    }
+    host_seq = ++s->seq_counter;
+    if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
+                                s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                max_units, s->units_host, s->n_active_host, s->opt_seq, host_seq, st)))
+      return rc;
   } else if (T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
     // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
     // single workgroup behind a device-scope counter, which beats two more launches only
@@ -558,10 +575,23 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     return moe_layer_done(eng, layer);
   }
   // the active expert list comes back to the host
-  HIPC(hipMemcpyAsync(s->units_host, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
-  HIPC(hipMemcpyAsync(s->n_active_host, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
-  HIPC(hipEventRecord(s->ev, st));
-  HIPC(hipEventSynchronize(s->ev));
+  if (host_seq) {
+    volatile int *sq = s->opt_seq;
+    const auto t0 = std::chrono::steady_clock::now();
+    unsigned spins = 0;
+    while (*sq != host_seq) {
+      if ((++spins & 1023u) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
+        HIPC(hipStreamSynchronize(st));
+        if (*sq != host_seq) { moe_set_error("routing of layer %d never reached the host", layer); return MOE_EHIP; }
+      }
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  } else {
+    HIPC(hipMemcpyAsync(s->units_host, s->units, sizeof(moe_unit) * max_units, hipMemcpyDeviceToHost, st));
+    HIPC(hipMemcpyAsync(s->n_active_host, s->n_active, sizeof(int), hipMemcpyDeviceToHost, st));
+    HIPC(hipEventRecord(s->ev, st));
+    HIPC(hipEventSynchronize(s->ev));
+  }
   const int n_act = *s->n_active_host;
   std::vector<int64_t> ids(n_act);
   std::unordered_map<int, moe_unit> unit_of;
@@ -585,9 +615,14 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     eng->ctr.ready += (uint64_t)n_now;
   }
   if ((rc = moe_flush_table(eng, layer, st))) return rc;
+  // int4 decode launches of up to 64 units take the units and their slot addresses in the kernel arguments
+  // (run_units hands over the host copies): the device copy of a sub-list is then never read, and its
+  // host-to-device copy would only put 4 us into the stream in front of the launch
+  const bool by_value = d.fmt == MOE_FMT_INT4_G128 && !use_prefill(d, T);
   const moe_unit *units_now = s->units;
   if (!later.empty() || n_now != n_act) {
-    if (n_now) HIPC(hipMemcpyAsync(s->units_sub, sub_h, sizeof(moe_unit) * n_now, hipMemcpyHostToDevice, st));
+    if (n_now && !(by_value && n_now <= 64))
+      HIPC(hipMemcpyAsync(s->units_sub, sub_h, sizeof(moe_unit) * n_now, hipMemcpyHostToDevice, st));
     units_now = s->units_sub;
     s->sub_cursor = n_now;
   }
@@ -604,7 +639,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
     moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
     *slot_h = unit_of[(int)id];
-    HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
+    if (!by_value) HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
     if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
     s->sub_cursor++;
     if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
