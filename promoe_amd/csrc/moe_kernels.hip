@@ -177,53 +177,69 @@ __global__ __launch_bounds__(64 * GATE_WAVES) void k_gate_logits_rows(const uint
 // ---------------------------------------------------------------------------
 // k1b top-k: one wave per token, E <= 256
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_topk(const float *__restrict__ logits, int T, int E,
-                                               int ldl, int k, int mode, int *__restrict__ idx,
-                                               float *__restrict__ wout) {
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int t = blockIdx.x * 4 + w;
-  if (t >= T) return;
+// The top-k of one token by one wave: lane l holds logits l, l + 64, ... (NR columns in use, E <= 64 NR).  k rounds of
+// a wave-wide maximum (DPP row shifts and broadcasts: no LDS round trips); the winner of a round is the lowest expert
+// id that holds the maximum (lowest column first, then lowest lane).  Lane j keeps the j-th choice, so the softmax
+// terms of the choices are one expf per lane, added in choice order.  COH: the logits were written by other
+// workgroups of this very launch and are read at device scope, past the L1.  s_idx / s_mask (LDS, optional): the
+// indices again and the token's experts as a bit mask [4 x 64], for a dispatch in the same kernel.
+template <int NR, bool COH>
+static __device__ __forceinline__ void topk_token(const float *__restrict__ row, const int E, const int k, const int mode,
+                                                  const int lane, int *__restrict__ idx, float *__restrict__ wout,
+                                                  int *s_idx, unsigned long long *s_mask) {
   const float NEG = -__builtin_inff();
-  float v[4];
+  float v[NR], v0[NR];
+  unsigned long long msel[NR];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
+  for (int r = 0; r < NR; ++r) {
     const int e = lane + 64 * r;
-    v[r] = (e < E) ? logits[(size_t)t * ldl + e] : NEG;
+    v[r] = (e < E) ? (COH ? __hip_atomic_load(row + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : row[e]) : NEG;
+    v0[r] = v[r];
+    msel[r] = 0ull;
   }
-  // row max (== first selected value) and softmax denominator over all E
-  float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-  float den = 0.f;
-#pragma unroll
-  for (int r = 0; r < 4; ++r)
-    if (lane + 64 * r < E) den += expf(v[r] - mx);
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
-
-  float sel_v = 0.f;  // lane j keeps the j-th selected logit
-  float sum_sel = 0.f;
+  float my_v = 0.f;  // lane j keeps the j-th selected logit
   for (int j = 0; j < k; ++j) {
-    // the maximum (DPP row shifts and broadcasts: no LDS round trips), then the lowest expert id that holds
-    // it: lowest 64-wide column first, then lowest lane
-    const float bv = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
+    float bvl = v[0];
+#pragma unroll
+    for (int r = 1; r < NR; ++r) bvl = fmaxf(bvl, v[r]);
+    const float bv = wave_max_f32(bvl);
     int wr = -1, wl = 0;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < NR; ++r) {
       const unsigned long long mr = __ballot(v[r] == bv);
       if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
     }
     if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
-    const int bi = wl + 64 * wr;
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (bi == lane + 64 * r) v[r] = NEG;
-    if (lane == j) sel_v = bv;
-    if (lane == 0) idx[(size_t)t * k + j] = bi;
-    sum_sel += expf(bv - mx);
+    for (int r = 0; r < NR; ++r)
+      if (r == wr) {
+        if (lane == wl) v[r] = NEG;
+        msel[r] |= 1ull << wl;
+      }
+    if (lane == j) {
+      my_v = bv;
+      const int bi = wl + 64 * wr;
+      idx[j] = bi;
+      if (s_idx) s_idx[j] = bi;
+    }
   }
-  // weights
-  const float ex = expf(sel_v - mx);
+  if (s_mask && lane == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s_mask[r] = r < NR ? msel[r < NR ? r : 0] : 0ull;
+  }
+  // weights: the row maximum is the first choice; the softmax denominator over all E per lane in column order, then
+  // the xor butterfly; the sum over the choices in choice order
+  const float mx = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_v), 0));
+  float den = 0.f;
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
+    if (lane + 64 * r < E) den += expf(v0[r] - mx);
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
+  const float ex = expf(my_v - mx);
+  float sum_sel = 0.f;
+  for (int j = 0; j < k; ++j)
+    sum_sel += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ex), j));
   float wgt;
   if (mode == MOE_ROUTE_TOPK_SOFTMAX) {
     wgt = ex / sum_sel;
@@ -231,7 +247,22 @@ __global__ __launch_bounds__(256) void k_topk(const float *__restrict__ logits, 
     wgt = ex / den;
     if (mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
   }
-  if (lane < k) wout[(size_t)t * k + lane] = wgt;
+  if (lane < k) wout[lane] = wgt;
+}
+
+__global__ __launch_bounds__(256) void k_topk(const float *__restrict__ logits, int T, int E,
+                                               int ldl, int k, int mode, int *__restrict__ idx,
+                                               float *__restrict__ wout) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + w;
+  if (t >= T) return;
+  const float *row = logits + (size_t)t * ldl;
+  int *ir = idx + (size_t)t * k;
+  float *wr = wout + (size_t)t * k;
+  // one instantiation per number of 64-wide logit columns: a 64-expert layer pays for one
+  if (E <= 64) topk_token<1, false>(row, E, k, mode, lane, ir, wr, nullptr, nullptr);
+  else if (E <= 128) topk_token<2, false>(row, E, k, mode, lane, ir, wr, nullptr, nullptr);
+  else topk_token<4, false>(row, E, k, mode, lane, ir, wr, nullptr, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -492,65 +523,29 @@ struct RouteArgs {
 // top-k (one wave per token) and stable dispatch by ONE workgroup of NW waves; the bodies of
 // k_topk and k_dispatch.  With host_units set the unit list also goes straight into pinned host
 // memory, followed (once those stores have completed) by the sequence word the host polls.
-template <int NW>
-static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx, int *s_cnt, int *s_off, int *s_run,
-                                                  int *s_w, int *s_wsum, int *s_wact, int &s_tot) {
+// NR: 64-wide logit columns in use (E <= 64 NR); COH: the logits were written by other workgroups of this very launch
+// and are read at device scope, past the L1 (k_route_decode); a launch of its own reads them plainly
+template <int NW, int NR, bool COH>
+static __device__ __forceinline__ void route_tail_n(const RouteArgs &a, int *s_idx, unsigned long long *s_mask, int *s_off,
+                                                    int *s_wsum, int *s_wact, int &s_tot) {
   constexpr int NT = NW * 64;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int E = a.E, T = a.T, k = a.k, P = T * k;
-  // ---- phase 2: top-k, wave w takes tokens w, w+NW, ... (body of k_topk) ----------------------
-  const float NEG = -__builtin_inff();
-  for (int t = w; t < T; t += NW) {
-    float v[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int e = lane + 64 * r;
-      // written by other workgroups of this launch: read at device scope, past the L1
-      v[r] = (e < E) ? __hip_atomic_load(a.logits + (size_t)t * a.ldl + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : NEG;
-    }
-    const float mx = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-    float den = 0.f;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (lane + 64 * r < E) den += expf(v[r] - mx);
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) den = den + __shfl_xor(den, m, 64);
-    float sel_v = 0.f, sum_sel = 0.f;
-    for (int j = 0; j < k; ++j) {
-      // the maximum, then the lowest expert id that holds it: lowest column first, then lowest lane
-      const float bv = wave_max_f32(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])));
-      int wr = -1, wl = 0;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const unsigned long long mr = __ballot(v[r] == bv);
-        if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
-      }
-      if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
-      const int bi = wl + 64 * wr;
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (bi == lane + 64 * r) v[r] = NEG;
-      if (lane == j) sel_v = bv;
-      if (lane == 0) { a.idx[(size_t)t * k + j] = bi; s_idx[t * k + j] = bi; }
-      sum_sel += expf(bv - mx);
-    }
-    const float ex = expf(sel_v - mx);
-    float wgt;
-    if (a.mode == MOE_ROUTE_TOPK_SOFTMAX) {
-      wgt = ex / sum_sel;
-    } else {
-      wgt = ex / den;
-      if (a.mode == MOE_ROUTE_SOFTMAX_TOPK_RENORM) wgt = wgt / (sum_sel / den);
-    }
-    if (lane < k) a.w[(size_t)t * k + lane] = wgt;
-  }
-  // ---- phase 3: dispatch (k_dispatch with NW waves; thread e owns expert e) -------------
-  if (tid < E) { s_cnt[tid] = 0; s_run[tid] = 0; }
+  // ---- phase 2: top-k, wave w takes tokens w, w+NW, ... (the selection, tie rule and weights of k_topk) -------
+  // besides the indices, every token leaves the set of its experts as a bit mask: the dispatch below counts bits
+  for (int t = w; t < T; t += NW)
+    topk_token<NR, COH>(a.logits + (size_t)t * a.ldl, E, k, a.mode, lane, a.idx + (size_t)t * k, a.w + (size_t)t * k,
+                        s_idx + t * k, s_mask + t * 4);
   __syncthreads();
-  for (int p = tid; p < P; p += NT) atomicAdd(&s_cnt[s_idx[p]], 1);
-  __syncthreads();
+  // ---- phase 3: dispatch (the arrays of k_dispatch).  A token holds an expert at most once, so the pairs of an
+  // expert in pair order are its tokens in token order: count of expert e = tokens whose mask has bit e, position of
+  // pair (t, e) = offset of e + tokens before t whose mask has bit e.  Thread e owns expert e; three barriers. ----
   {
-    const int c = (tid < E) ? s_cnt[tid] : 0;
+    int c = 0;
+    if (tid < E) {
+      const int r = tid >> 6, bit = tid & 63;
+      for (int t = 0; t < T; ++t) c += (int)((s_mask[t * 4 + r] >> bit) & 1ull);
+    }
     const int act = c > 0 ? 1 : 0;
     int sc = c, sa = act;
 #pragma unroll
@@ -588,39 +583,15 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
       a.active_ids[u] = -1;
     }
   }
-  __syncthreads();
-  for (int base = 0; base < P; base += NT) {
-    for (int i = tid; i < NW * E; i += NT) s_w[i] = 0;
-    __syncthreads();
-    const int p = base + tid;
-    const int e = (p < P) ? s_idx[p] : -1;
-    const bool valid = e >= 0;
-    unsigned long long peers = __ballot(valid);
-    for (int b = 0; b < a.nbits; ++b) {
-      const bool bit = (e >> b) & 1;
-      const unsigned long long bal = __ballot(valid && bit);
-      peers &= bit ? bal : ~bal;
-    }
-    const int rank = __popcll(peers & ((1ull << lane) - 1ull));
-    if (valid && rank == 0) s_w[w * E + e] = __popcll(peers);
-    __syncthreads();
-    if (tid < E) {
-      int run = s_run[tid];
-      for (int ww = 0; ww < NW; ++ww) {
-        const int c = s_w[ww * E + tid];
-        s_w[ww * E + tid] = run;
-        run += c;
-      }
-      s_run[tid] = run;
-    }
-    __syncthreads();
-    if (valid) {
-      const int pos = s_off[e] + s_w[w * E + e] + rank;
-      a.sorted_pair[pos] = p;
-      a.pos_of_pair[p] = pos;
-      a.sorted_tok[pos] = p / k;
-    }
-    __syncthreads();
+  for (int p = tid; p < P; p += NT) {
+    const int e = s_idx[p], t = p / k;
+    const int r = e >> 6, bit = e & 63;
+    int rank = 0;
+    for (int tt = 0; tt < t; ++tt) rank += (int)((s_mask[tt * 4 + r] >> bit) & 1ull);
+    const int pos = s_off[e] + rank;
+    a.sorted_pair[pos] = p;
+    a.pos_of_pair[p] = pos;
+    a.sorted_tok[pos] = t;
   }
   if (a.host_units) {
     host_stores_done();
@@ -629,10 +600,20 @@ static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx
   }
 }
 
+template <int NW, bool COH>
+static __device__ __forceinline__ void route_tail(const RouteArgs &a, int *s_idx, unsigned long long *s_mask, int *s_off,
+                                                  int *s_wsum, int *s_wact, int &s_tot) {
+  // one instantiation per number of logit columns: a 64-expert layer pays for one
+  if (a.E <= 64) route_tail_n<NW, 1, COH>(a, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
+  else if (a.E <= 128) route_tail_n<NW, 2, COH>(a, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
+  else route_tail_n<NW, 4, COH>(a, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
+}
+
 __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
   __shared__ int s_last;
   __shared__ int s_idx[ROUTE_MAXP];
-  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[4 * 256];
+  __shared__ unsigned long long s_mask[ROUTE_MAXT * 4];
+  __shared__ int s_off[257];
   __shared__ int s_wsum[4], s_wact[4], s_tot;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int H = a.H, E = a.E, T = a.T, k = a.k, P = T * k;
@@ -674,7 +655,7 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
   }
   __syncthreads();
   if (!s_last) return;
-  route_tail<4>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
+  route_tail<4, true>(a, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
 }
 
 // k1b + k2 in one launch for decode batches whose logits exist already: one workgroup of NW waves
@@ -682,9 +663,10 @@ __global__ __launch_bounds__(256) void k_route_decode(const RouteArgs a) {
 template <int NW>
 __global__ __launch_bounds__(64 * NW) void k_topk_dispatch(const RouteArgs a) {
   __shared__ int s_idx[ROUTE_MAXP];
-  __shared__ int s_cnt[256], s_off[257], s_run[256], s_w[NW * 256];
+  __shared__ unsigned long long s_mask[ROUTE_MAXT * 4];
+  __shared__ int s_off[257];
   __shared__ int s_wsum[NW], s_wact[NW], s_tot;
-  route_tail<NW>(a, s_idx, s_cnt, s_off, s_run, s_w, s_wsum, s_wact, s_tot);
+  route_tail<NW, false>(a, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
 }
 
 // ---------------------------------------------------------------------------
