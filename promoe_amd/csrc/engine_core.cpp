@@ -904,6 +904,18 @@ static int wait_expert_locked(moe_engine *eng, Expert *e, std::unique_lock<std::
   }
   const auto t0 = std::chrono::steady_clock::now();
   eng->cv_work.notify_all();
+  // a demand copy is over in about 100 us: poll the expert's state (an atomic) without the lock for that long before
+  // sleeping on the condition variable, whose wake-up alone costs 10-50 us per miss
+  lk.unlock();
+  while (e->status.load(std::memory_order_acquire) != kLaunching &&
+         std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(400)) {
+#if defined(__x86_64__)
+    for (int i = 0; i < 64; ++i) __builtin_ia32_pause();
+#else
+    std::this_thread::yield();
+#endif
+  }
+  lk.lock();
   eng->cv_state.wait(lk, [&] { return e->status.load() == kLaunching || eng->exiting || !eng->fatal.empty(); });
   eng->ctr.wait_us += (uint64_t)std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count();
   if (!eng->fatal.empty()) { moe_set_error("engine failed while waiting: %s", eng->fatal.c_str()); return MOE_ESTATE; }
