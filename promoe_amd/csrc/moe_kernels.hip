@@ -1000,6 +1000,7 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
   const int n_sc = 2 * G * SCB / 4;   // dwords of section s
   const int n_zz = 2 * G * ZZB / 4;   // dwords of section z
   constexpr int XT = TMAX < 2 ? TMAX : 2;  // rows whose first 256 vectors are staged through registers
+  const Q4Consts q4c = q4_consts();
 
   for (int t0 = 0; t0 < m; t0 += TMAX) {
     const int mc = (m - t0) < TMAX ? (m - t0) : TMAX;
@@ -1098,11 +1099,11 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
             const uint4 *xp = (const uint4 *)(xs + (size_t)t * K + g * 128 + qd * 32);
             const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
             const float xq = xsum[t * KS + g * 4 + qd];
-            float dA = dot8_q4(wa[j].x, x0, 0.f);
-            float dB = dot8_q4(wb[j].x, x0, 0.f);
-            dA = dot8_q4(wa[j].y, x1, dA); dB = dot8_q4(wb[j].y, x1, dB);
-            dA = dot8_q4(wa[j].z, x2, dA); dB = dot8_q4(wb[j].z, x2, dB);
-            dA = dot8_q4(wa[j].w, x3, dA); dB = dot8_q4(wb[j].w, x3, dB);
+            float dA = dot8_q4(wa[j].x, x0, 0.f, q4c);
+            float dB = dot8_q4(wb[j].x, x0, 0.f, q4c);
+            dA = dot8_q4(wa[j].y, x1, dA, q4c); dB = dot8_q4(wb[j].y, x1, dB, q4c);
+            dA = dot8_q4(wa[j].z, x2, dA, q4c); dB = dot8_q4(wb[j].z, x2, dB, q4c);
+            dA = dot8_q4(wa[j].w, x3, dA, q4c); dB = dot8_q4(wb[j].w, x3, dB, q4c);
             if (Q4K) {
               accA[t] = fmaf(fsa, dA, fmaf(-fza, xq, accA[t]));
               accB[t] = fmaf(fsb, dB, fmaf(-fzb, xq, accB[t]));
@@ -1225,6 +1226,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
     const bool miss = (lane < k || (lane == k && I_sh > 0)) && ub_lo == 0 && ub_hi == 0;
     if (__ballot(miss) != 0ull && lane == 0) moe_raise_err(a.err);
   }
+  const Q4Consts q4c = q4_consts();
   float acc = 0.f;
   // cursor of the wave's current group of NI items: first item = unit u (k = the shared expert), group g
   int u = 0, g = NI * w;
@@ -1304,8 +1306,8 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
       const uint4 *xp = (const uint4 *)(hs + hoff);
       const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
       const float xq = xsum[hoff >> 5];
-      const float d0 = dot8_q4(wt[c].x, x0, 0.f), d1 = dot8_q4(wt[c].y, x1, 0.f);
-      const float d2 = dot8_q4(wt[c].z, x2, 0.f), d3 = dot8_q4(wt[c].w, x3, 0.f);
+      const float d0 = dot8_q4(wt[c].x, x0, 0.f, q4c), d1 = dot8_q4(wt[c].y, x1, 0.f, q4c);
+      const float d2 = dot8_q4(wt[c].z, x2, 0.f, q4c), d3 = dot8_q4(wt[c].w, x3, 0.f, q4c);
       const float d = (d0 + d1) + (d2 + d3);
       const float fs = half_bits_to_f32((uint16_t)sc[c]);
       const float fz = 128.f + (float)((zz[c] >> zsh) & 15);
@@ -1344,8 +1346,8 @@ static __device__ __forceinline__ float4 scale_zero_pair(u32 sc, u32 z) {
 }
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-static __device__ __forceinline__ bf16x8_t deq8_bf16(u32 w) {
-  const u32 M = 0x000f000fu, C = 0x43004300u;
+static __device__ __forceinline__ bf16x8_t deq8_bf16(u32 w, const Q4Consts &q) {
+  const u32 M = q.M, C = q.C;  // in vector registers: one v_and_or_b32 per pair
   u32x4_t v;
   v.x = (w & M) | C; v.y = ((w >> 4) & M) | C; v.z = ((w >> 8) & M) | C; v.w = ((w >> 12) & M) | C;
   return __builtin_bit_cast(bf16x8_t, v);
@@ -1362,6 +1364,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
+  const Q4Consts q4c = q4_consts();
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
   const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
@@ -1501,13 +1504,13 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 #pragma unroll
           for (int n = 0; n < NB; ++n) d[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].x), x0, d[n], 0, 0, 0);
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].x, q4c), x0, d[n], 0, 0, 0);
 #pragma unroll
-          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].y), x1, d[n], 0, 0, 0);
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].y, q4c), x1, d[n], 0, 0, 0);
 #pragma unroll
-          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].z), x2, d[n], 0, 0, 0);
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].z, q4c), x2, d[n], 0, 0, 0);
 #pragma unroll
-          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].w), x3, d[n], 0, 0, 0);
+          for (int n = 0; n < NB; ++n) d[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(deq8_bf16(wt[j][n].w, q4c), x3, d[n], 0, 0, 0);
 #pragma unroll
           for (int n = 0; n < NB; ++n) {
             // (s, -s (128 + z)) of the 4 rows this lane owns in D: rows 4qd..4qd+3
@@ -1588,6 +1591,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
+  const Q4Consts q4c = q4_consts();
   const int kh = w % KS;  // which part of every chunk this wave takes
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
@@ -1718,8 +1722,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
           }
 #pragma unroll
           for (int n = 0; n < NB; ++n) {
-            const bf16x8_t w0 = deq8_bf16(cur[j][n].x), w1 = deq8_bf16(cur[j][n].y);
-            const bf16x8_t w2 = deq8_bf16(cur[j][n].z), w3 = deq8_bf16(cur[j][n].w);
+            const bf16x8_t w0 = deq8_bf16(cur[j][n].x, q4c), w1 = deq8_bf16(cur[j][n].y, q4c);
+            const bf16x8_t w2 = deq8_bf16(cur[j][n].z, q4c), w3 = deq8_bf16(cur[j][n].w, q4c);
             // (s, -s (128 + z)) of the 4 rows this lane owns in D: rows 4qd..4qd+3
             const float4 *sf = (const float4 *)(sfw + ((n * GW + gl) * 16 + 4 * qd) * 2);
             const float4 f0 = sf[0], f1 = sf[1];

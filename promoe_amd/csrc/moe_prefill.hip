@@ -325,8 +325,17 @@ static __device__ __forceinline__ u32 pf_bf16x2_to_f16x2(u32 d) {
   return __builtin_bit_cast(u32, h);
 }
 // s2 / nz2: the row's scale and -(1024 + zero) as fp16 bit patterns replicated in both halves
-static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2) {
-  const u32 M = 0x000f000fu, C = 0x64006400u;
+// nibble mask and the fp16 pattern of 1024 held in vector registers, made once per kernel: (d & M) | C is then ONE
+// v_and_or_b32 (a VOP3 instruction takes no literal and one scalar operand on this target; with literals the
+// compiler emits an and and an or, 4 more operations per 8 weights in kernels bound by exactly these operations)
+struct PfDeqConsts { u32 M, C; };
+static __device__ __forceinline__ PfDeqConsts pf_deq_consts() {
+  PfDeqConsts q{0x000f000fu, 0x64006400u};
+  asm volatile("" : "+v"(q.M), "+v"(q.C));
+  return q;
+}
+static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2, const PfDeqConsts &q) {
+  const u32 M = q.M, C = q.C;
   u32x4_t v;
   v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
   const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1024 + q, exact
@@ -337,8 +346,8 @@ static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2) {
 
 // q4_K flavour: w = s*q - m with the lane's own sub-block scale s = d*sc and min m = dmin*mn.
 // s2 / nm2: fp16 bit patterns of s and -m replicated in both halves.
-static __device__ __forceinline__ f16x8_t pf_deq8_q4k(u32 d, u32 s2, u32 nm2) {
-  const u32 M = 0x000f000fu, C = 0x64006400u;
+static __device__ __forceinline__ f16x8_t pf_deq8_q4k(u32 d, u32 s2, u32 nm2, const PfDeqConsts &q) {
+  const u32 M = q.M, C = q.C;
   u32x4_t v;
   v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
   const f16x8_t h = __builtin_bit_cast(f16x8_t, v);
@@ -375,6 +384,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   const int lane = tid & 63, g = tid >> 8;
   const int r = lane & 15, qd = lane >> 4;
   const int ch = tid & 15, r0 = tid >> 4;  // staging: row r0 + 32 i (block i), 16-byte chunk ch of the 128-k group
+  const PfDeqConsts dqc = pf_deq_consts();
   u32x4_t ra[3], wA[4], wB[4];
   PiMeta mA, mB;
   // activations of the next group travel in two halves (row blocks 0..2, then 3..5) through
@@ -431,7 +441,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
       const int j = j0 + jj;
       f16x8_t wd[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wd[t] = Q4K ? pf_deq8_q4k(wq[t][j], s2[t], z2[t]) : pf_deq8_f16(wq[t][j], s2[t], z2[t]);
+      for (int t = 0; t < 4; ++t) wd[t] = Q4K ? pf_deq8_q4k(wq[t][j], s2[t], z2[t], dqc) : pf_deq8_f16(wq[t][j], s2[t], z2[t], dqc);
 #pragma unroll
       for (int tb = 0; tb < 2 * NBW; ++tb) {
         const f16x8_t xa = *(const f16x8_t *)(A_ + (64 * (tb >> 1) + 16 * (tb & 1)) * PI_LDK + 8 * j);
