@@ -240,6 +240,8 @@ int moe_experts_decode_q4k(const void *x_bf16, int T, int H, int I, int I_sh, in
  *   tiles_ws  : device workspace of moe_prefill_workspace_bytes(T, k, max_units) bytes; the
  *               list of row tiles per expert is built there by a kernel, so the host
  *               needs no copy of the dispatch counts.
+ * Between the two passes h_r / h_s hold bf16 for MOE_FMT_BF16 and fp16 for the nibble formats (whose matrix-core
+ * operands are fp16: the w2 pass then stages them without a conversion); both passes of a batch go through this entry.
  * H % 256 == 0, I % 128 == 0, I_sh % 128 == 0.  The reference leaves this product to the
  * framework's own expert modules (SimulateMoeLayer.forward, transformers-deepseek-moe.py:36-49). */
 int64_t moe_prefill_workspace_bytes(int T, int k, int max_units);

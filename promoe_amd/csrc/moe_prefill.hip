@@ -309,7 +309,8 @@ __global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
 // 0x000f000f is OR-ed into 0x6400 (fp16 1024+q), then (h - (1024+z)) * s with two packed
 // fp16 operations per pair (the subtraction is exact).  gfx950 has packed fp16 arithmetic
 // but no packed bf16 arithmetic, hence fp16 operands: activations are converted bf16 -> fp16
-// while they are staged into LDS (exact for |x| < 65504 outside the fp16 subnormal range).
+// while they are staged into LDS (exact for |x| < 65504 outside the fp16 subnormal range); the h rows
+// between the two passes are written as fp16 by the w13 epilogue, so the w2 pass stages them as they are.
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
@@ -378,7 +379,9 @@ static __device__ __forceinline__ u32 pf_f2h(float f) {  // fp32 -> fp16 bits (r
 
 struct PiMeta { u32 sc[4]; u32 zz[4]; };  // raw fp16 scale bits / zero nibble of the lane's row in the 4 tiles
 
-template <int NBW, bool Q4K>
+// ACT16: the activations are fp16 already (the h rows this kernel's w13 pass wrote, or a converted copy of x):
+// staged as they are, without the three vector operations per pair of the bf16 -> fp16 conversion
+template <int NBW, bool Q4K, bool ACT16>
 static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_t *As, const rsrc_t rx, const u32 (&a_off)[6],
                                                    const rsrc_t rq, const rsrc_t rs, const rsrc_t rz, int G, int nb, int tid) {
   const int lane = tid & 63, g = tid >> 8;
@@ -399,9 +402,11 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
 #pragma unroll
     for (int i = 0; i < 3; ++i)
       if (3 * half + i < nb) {
-        u32x4_t v;
-        v.x = pf_bf16x2_to_f16x2(ra[i].x); v.y = pf_bf16x2_to_f16x2(ra[i].y);
-        v.z = pf_bf16x2_to_f16x2(ra[i].z); v.w = pf_bf16x2_to_f16x2(ra[i].w);
+        u32x4_t v = ra[i];
+        if (!ACT16) {
+          v.x = pf_bf16x2_to_f16x2(ra[i].x); v.y = pf_bf16x2_to_f16x2(ra[i].y);
+          v.z = pf_bf16x2_to_f16x2(ra[i].z); v.w = pf_bf16x2_to_f16x2(ra[i].w);
+        }
         *(u32x4_t *)(A_ + (r0 + 32 * (3 * half + i)) * PI_LDK + ch * 8) = v;
       }
   };
@@ -483,7 +488,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   }
 }
 
-template <bool SWIGLU, bool Q4K>
+template <bool SWIGLU, bool Q4K, bool ACT16>
 __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   extern __shared__ __align__(16) uint16_t As[];  // [2][PI_BM][PI_LDK] fp16
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane((tid >> 6) & 3), g = tid >> 8;
@@ -534,10 +539,10 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   const int nb = (tile.rows + 31) >> 5;
   const int nbw = (nb - g + 1) >> 1;
   switch (nbw) {
-    case 0: pi_mainloop<0, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 1: pi_mainloop<1, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 2: pi_mainloop<2, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    default: pi_mainloop<3, Q4K>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 0: pi_mainloop<0, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 1: pi_mainloop<1, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 2: pi_mainloop<2, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    default: pi_mainloop<3, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
   }
   // epilogue.  acc[t][tb] element i of lane l: weight row r of tile t, token row
   // 32*(2*(tb/2)+g) + 16*(tb%2) + 4*qd + i of the tile
@@ -552,7 +557,7 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
 #pragma unroll
           for (int b = 0; b < 2; ++b) {
             const float gt = acc[2 * b][tb][i], up = acc[2 * b + 1][tb][i];
-            ((__bf16 *)c.out)[orow + 16 * (rb0 / 2 + b) + r] = (__bf16)pf_silu_mul(gt, up);
+            ((_Float16 *)c.out)[orow + 16 * (rb0 / 2 + b) + r] = (_Float16)pf_silu_mul(gt, up);  // h in fp16: what the w2 pass stages
           }
         } else {
 #pragma unroll
@@ -571,20 +576,24 @@ static int pf_slab_step(int nk) {
 }
 
 template <bool Q4K>
-static int pi_launch(bool swiglu, const PfArgs &a, hipStream_t s) {
+static int pi_launch(bool swiglu, bool x16, const PfArgs &a, hipStream_t s) {
   if (a.n_blocks_total <= 0) return MOE_OK;
   const int grid = ((a.c[0].n_blocks + 7) & ~7) + ((a.c[1].n_blocks + 7) & ~7);
   const size_t lds = (size_t)2 * PI_BM * PI_LDK * 2;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute((const void *)k_prefill_int4<true, Q4K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    hipError_t e2 = hipFuncSetAttribute((const void *)k_prefill_int4<false, Q4K>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (int rc = moe_check_hip(e1 != hipSuccess ? e1 : e2, "hipFuncSetAttribute(k_prefill_int4)")) return rc;
+    for (const void *f : {(const void *)k_prefill_int4<true, Q4K, false>, (const void *)k_prefill_int4<true, Q4K, true>,
+                          (const void *)k_prefill_int4<false, Q4K, true>})
+      if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                                 "hipFuncSetAttribute(k_prefill_int4)"))
+        return rc;
     attr_set = true;
   }
   moe_ktimer_begin(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
-  if (swiglu) hipLaunchKernelGGL((k_prefill_int4<true, Q4K>), dim3(grid), dim3(512), lds, s, a);
-  else hipLaunchKernelGGL((k_prefill_int4<false, Q4K>), dim3(grid), dim3(512), lds, s, a);
+  // the w2 pass reads the fp16 h rows of the w13 pass; the w13 pass reads bf16 x, or its fp16 copy when there is one
+  if (swiglu && x16) hipLaunchKernelGGL((k_prefill_int4<true, Q4K, true>), dim3(grid), dim3(512), lds, s, a);
+  else if (swiglu) hipLaunchKernelGGL((k_prefill_int4<true, Q4K, false>), dim3(grid), dim3(512), lds, s, a);
+  else hipLaunchKernelGGL((k_prefill_int4<false, Q4K, true>), dim3(grid), dim3(512), lds, s, a);
   moe_ktimer_end(swiglu ? MOE_K_PREFILL_W13 : MOE_K_PREFILL_W2, s);
   return moe_check_launch("k_prefill_int4");
 }
@@ -756,7 +765,7 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
       c.slab_step = pf_slab_step(c.K / PF_BK);
       a.n_blocks_total += c.n_blocks;
     }
-    if (int rc = q4k ? pi_launch<true>(!w2, a, s) : (int4 ? pi_launch<false>(!w2, a, s) : pf_launch(!w2, a, s))) return rc;
+    if (int rc = q4k ? pi_launch<true>(!w2, false, a, s) : (int4 ? pi_launch<false>(!w2, false, a, s) : pf_launch(!w2, a, s))) return rc;
   }
   return MOE_OK;
 }
