@@ -801,16 +801,19 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
 // lowest expert id that holds the maximum - the order and the tie rule of k_topk.  One spare
 // workgroup publishes the routing (indices, weights, dispatch arrays, unit list) for the
 // later kernels and the host.
+// Block order: the routed experts' workgroups, then one workgroup that only publishes the routing (its first
+// wave), then the shared expert's.  With the shared expert's workgroups in front, their tile requests (issued 0.3 us
+// after the launch, nothing to wait for) stood in the compute units' memory pipelines ahead of the logit loads of
+// the routed workgroups that share those compute units, and a tenth of the routed workgroups knew their expert
+// 2 us later than the others.
 template <int NR>
 static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &a, int lane, int w) {
   GemvWork wk;
-  const int n_sh = a.n_sh_blocks;
-  const bool sh = (int)blockIdx.x < n_sh;
-  wk.c = sh ? a.cls[0] : a.cls[1];
-  const int rr = sh ? (int)blockIdx.x : (int)blockIdx.x - n_sh;
   const int E = a.r_E, k = a.r_k;
-  // one extra workgroup at the end of the grid only publishes the routing (its first wave);
-  // it finishes long before the workgroups that stream weights
+  const int n_rt = k * a.cls[1].nblk + 1;
+  const bool sh = (int)blockIdx.x >= n_rt;
+  wk.c = sh ? a.cls[0] : a.cls[1];
+  const int rr = sh ? (int)blockIdx.x - n_rt : (int)blockIdx.x;
   const bool publisher = !sh && rr == k * wk.c.nblk;
   const int u = (sh || publisher) ? 0 : rr / wk.c.nblk;
   wk.b = rr - u * wk.c.nblk;
@@ -956,13 +959,13 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   return gemv_resolve_route_n<4>(a, lane, w);
 }
 
-template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false, bool ROUTE = false>
+template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false>
 __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
 
-  const GemvWork wk = ROUTE ? gemv_resolve_route(a, lane, w) : gemv_resolve<DEVUNITS>(a, (int)blockIdx.x);
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a, (int)blockIdx.x);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -1150,6 +1153,135 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
       }
     }
     if (t0 + TMAX < m) __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// w13 + SwiGLU for ONE token with the routing derived in the kernel (int4-g128): the kernel of a one-token step.
+// Same work split and the same order of every sum as k_gemv_int4<1, true, CH> (bit-identical h), but after the
+// barrier that hands the routing over, a wave depends on no other wave until the final reduction: it reads
+// the 256 bytes of the activation row that each of its own groups needs (16 bytes per lane), the 32 + 8 bytes of
+// scales and zeros of each of its own tiles (one dword per lane each) and its tiles, in that order, and keeps the
+// small ones in a wave-private LDS area (a wave's LDS operations complete in order: no barrier).  With the whole
+// row and both scale sections staged by all four waves, a barrier stood between the requests and the first
+// product, and the last wave's small loads gated all four.
+// Measured with a time stamp per wave in the barrier form: routing known 1.5-1.8 us after entry (3.7-4.2 us for
+// the workgroups that shared a compute unit with the shared expert's, hence the block order of
+// gemv_resolve_route_n), activations and scales staged 1.6 us later, products 4 x 0.28 us.
+// LDS per wave: [CH][128] bf16 activations, [CH][4] sums, [2 CH][8] scale dwords, [2 CH][2] zero dwords; then
+// [4][2][16] partial sums.
+// ---------------------------------------------------------------------------
+#define W13T_WAVE_DW(ch) ((ch) * 64 + (ch) * 4 + (ch) * 16 + (ch) * 4)
+static size_t w13_token_lds(int ch) { return (size_t)4 * W13T_WAVE_DW(ch) * 4 + 4 * 2 * 16 * 4; }
+
+template <int CH>
+__global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, qd = lane >> 4;
+  const GemvWork wk = gemv_resolve_route(a, lane, w);  // ends with a barrier (routed workgroups)
+  const GemvClass &c = wk.c;
+  const unsigned char *base = wk.base;
+  if (wk.m <= 0) return;
+  if (base == nullptr) {
+    if (tid == 0 && wk.b == 0) moe_raise_err(a.err);  // one store per missing unit (the word may be host memory)
+    return;
+  }
+  const int G = c.G, b = wk.b;
+  u32 *wl = (u32 *)smem + w * W13T_WAVE_DW(CH);
+  uint16_t *xs = (uint16_t *)wl;                        // [CH][128]
+  float *xsum = (float *)(wl + CH * 64);                // [CH][4]
+  u32 *wsc = wl + CH * 68;                              // [2 CH][8]: block A's groups, then block B's
+  u32 *wzz = wsc + CH * 16;                             // [2 CH][2]
+  float *red = (float *)((u32 *)smem + 4 * W13T_WAVE_DW(CH));  // [4][2][16]
+  const int GPW = (G - w + 3) >> 2;  // groups of this wave: g = w + 4j, j < GPW
+  const int rbA = 2 * b;             // tiles of block A then block B are contiguous: 2 G KiB
+  const rsrc_t rx = make_rsrc((const unsigned char *)c.act, (u32)c.K * 2u);
+  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)(2 * G) * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)(2 * G) * 32u);
+  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)(2 * G) * 8u);
+  const int zsh = (r & 1) * 4;
+  const Q4Consts q4c = q4_consts();
+  // the lane's share of the wave's small loads: 16 bytes of group xj's activations, dword scd of scale chunk scj
+  // (chunks: block A's groups 0..CH-1, then block B's), dword zzd of zero chunk zzj
+  const int xj = lane >> 4, xpart = lane & 15, scj = lane >> 3, scd = lane & 7, zzj = lane >> 1, zzd = lane & 1;
+  const uint16_t *wsc_h = (const uint16_t *)wsc;
+  const unsigned char *wzz_b = (const unsigned char *)wzz;
+  float accA = 0.f, accB = 0.f;
+  for (int jc = 0; jc < GPW; jc += CH) {
+    uint4 xv = make_uint4(0u, 0u, 0u, 0u);
+    u32 sd = 0, zd = 0;
+    if (xj < CH) {
+      const int g = jc + xj < GPW ? w + 4 * (jc + xj) : 0;  // clamped: group 0 always exists
+      xv = bload16(rx, g * 256 + xpart * 16, 0);
+    }
+    if (scj < 2 * CH) {
+      const int j = scj < CH ? scj : scj - CH;
+      const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
+      sd = bload4(rs, (((scj < CH ? 0 : G) + g) * 8 + scd) * 4, 0);
+    }
+    if (zzj < 2 * CH) {
+      const int j = zzj < CH ? zzj : zzj - CH;
+      const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
+      zd = bload4(rz, (((zzj < CH ? 0 : G) + g) * 2 + zzd) * 4, 0);
+    }
+    uint4 wa[CH], wb[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int g = jc + j < GPW ? w + 4 * (jc + j) : 0;
+      wa[j] = bload16(rq, lane * 16, g * 1024);
+      wb[j] = bload16(rq, lane * 16, (G + g) * 1024);
+    }
+    {
+      float ps = sum8_bf16(xv);
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      if (xj < CH) {
+        ((uint4 *)xs)[lane] = xv;
+        if ((lane & 3) == 0) xsum[lane >> 2] = ps;
+      }
+    }
+    if (scj < 2 * CH) wsc[lane] = sd;
+    if (zzj < 2 * CH) wzz[lane] = zd;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const bool valid = jc + j < GPW;
+      // a clamped (duplicate) tile contributes through a zero scale
+      const float fsa_ = half_bits_to_f32(wsc_h[j * 16 + r]), fsb_ = half_bits_to_f32(wsc_h[(CH + j) * 16 + r]);
+      const float fsa = valid ? fsa_ : 0.f, fsb = valid ? fsb_ : 0.f;
+      const float fza = 128.f + (float)((wzz_b[j * 8 + (r >> 1)] >> zsh) & 15);
+      const float fzb = 128.f + (float)((wzz_b[(CH + j) * 8 + (r >> 1)] >> zsh) & 15);
+      const uint4 *xp = (const uint4 *)(xs + j * 128 + qd * 32);
+      const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+      const float xq = xsum[j * 4 + qd];
+      float dA = dot8_q4(wa[j].x, x0, 0.f, q4c);
+      float dB = dot8_q4(wb[j].x, x0, 0.f, q4c);
+      dA = dot8_q4(wa[j].y, x1, dA, q4c); dB = dot8_q4(wb[j].y, x1, dB, q4c);
+      dA = dot8_q4(wa[j].z, x2, dA, q4c); dB = dot8_q4(wb[j].z, x2, dB, q4c);
+      dA = dot8_q4(wa[j].w, x3, dA, q4c); dB = dot8_q4(wb[j].w, x3, dB, q4c);
+      accA = fmaf(fsa, dA - fza * xq, accA);
+      accB = fmaf(fsb, dB - fzb * xq, accB);
+      // keep the scheduler from hoisting the next tile's LDS reads (register pressure)
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // reduce the four k-quarters of the wave, then the four waves
+  accA += __shfl_xor(accA, 16, 64); accA += __shfl_xor(accA, 32, 64);
+  accB += __shfl_xor(accB, 16, 64); accB += __shfl_xor(accB, 32, 64);
+  if (lane < 16) {
+    red[(w * 2 + 0) * 16 + lane] = accA;
+    red[(w * 2 + 1) * 16 + lane] = accB;
+  }
+  __syncthreads();
+  if (tid < 16) {
+    float ga = 0.f, up = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < 4; ++ww) {
+      ga += red[(ww * 2 + 0) * 16 + tid];
+      up += red[(ww * 2 + 1) * 16 + tid];
+    }
+    const float hv = ga / (1.f + expf(-ga)) * up;
+    ((uint16_t *)c.out)[(size_t)wk.row0 * c.out_stride + b * 16 + tid] = f32_to_bf16(hv);
   }
 }
 
@@ -2336,9 +2468,9 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
 template <int CH>
 static int launch_gemv_route(const GemvArgs &a, int grid, size_t lds, hipStream_t s) {
   moe_ktimer_begin(MOE_K_W13, s);
-  hipLaunchKernelGGL((k_gemv_int4<1, true, CH, true, false, true>), dim3(grid), dim3(256), lds, s, a);
+  hipLaunchKernelGGL((k_w13_token<CH>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(MOE_K_W13, s);
-  return moe_check_launch("k_gemv_int4<route>");
+  return moe_check_launch("k_w13_token");
 }
 
 extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, int k, int mode, int H, int I,
@@ -2380,8 +2512,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
     const int gpw = (H / 128 + 3) / 4;
     int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
     if (ch < 1) ch = 1;
-    const size_t lds = gemv_lds(1, H);
-    if (lds > 64 * 1024) { moe_set_error("moe_decode_token_int4: H=%d does not fit LDS", H); return MOE_EINVAL; }
+    const size_t lds = w13_token_lds(ch);
     int rc = MOE_OK;
     if (phases & 1) switch (ch) {
       case 1: rc = launch_gemv_route<1>(a, grid, lds, s); break;
