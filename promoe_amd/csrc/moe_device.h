@@ -104,4 +104,10 @@ static __device__ __forceinline__ uint4 bload16(rsrc_t r, int voff, int soff) {
 static __device__ __forceinline__ u32 bload4(rsrc_t r, int voff, int soff) {
   return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
 }
+static __device__ __forceinline__ u32 bload2(rsrc_t r, int voff, int soff) {
+  return (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+}
+static __device__ __forceinline__ u32 bload1(rsrc_t r, int voff, int soff) {
+  return (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(r, voff, soff, 0);
+}
 

@@ -1289,11 +1289,13 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
 // k3 (w2) + k5 for ONE token in one launch: a workgroup of 16 waves owns 8 output rows and walks
 // the w2 tiles of those rows over ALL units (the k routed experts and the shared expert), weighting
 // each unit as it accumulates, so the combine needs no launch of its own and no partial rows in memory.
-//   item i < k*G : unit i / G, quantisation group i % G;  items k*G .. : the shared expert's groups
-//   A tile holds 16 rows; the workgroup wants 8 of them, so a wave reads the halves of TWO items with
-//   one load: lanes whose tile row is 0..7 take item 2s, the others item 2s + 1, each its row & 7 of
-//   the workgroup's half.  Wave w takes the item pairs s = w, w+16, ...; up to six loads per wave are
-//   requested before the activations (the h vectors of all units) are staged in LDS.
+//   An item is one quantisation group (128 columns) of one unit.  A tile holds 16 rows; the workgroup wants 8
+//   of them, so a wave reads the halves of TWO items with one load: lanes whose tile row is 0..7 take the first,
+//   the others the second, each its row & 7 of the workgroup's half.  The two items of a load are groups 2j and
+//   2j + 1 of ONE unit (a unit with an odd number of groups ends with a load whose second item does not exist and
+//   reads zeros).  Wave w takes the loads w, w + 16, ... of the list (unit 0's loads, unit 1's, ..., the shared
+//   expert's) and requests up to W2C_CHUNK of them, each with the 256 bytes of the unit's h vector that its
+//   items need, before the first product; it shares nothing with the other waves until the final sum.
 //   H/8 workgroups: twice the compute units of a 16-row split, which is what the load latency wants.
 // ---------------------------------------------------------------------------
 #define W2C_WAVES 16
@@ -1322,22 +1324,14 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   const int mine = r / RW;                                  // which item of the group this lane works on
   const int rr = RW * part + (r % RW);                      // its row inside the 16-row tile
   const int k = a.k, I = a.I, I_sh = a.I_sh, G = a.G, G_sh = a.G_sh;
-  const int n_h = k * I + I_sh;                       // staged activation elements
-  uint16_t *hs = (uint16_t *)wsm;                     // [k][I] then [I_sh]
-  float *xsum = (float *)(wsm + (size_t)n_h * 2);     // sums over 32 consecutive elements
-  float *red = xsum + (n_h >> 5);                     // [W2C_WAVES][RW]
+  // wave-private LDS: the 128 activations of each item of the wave's current chunk, and their 32-wide sums.
+  // A wave stages what its own items need and nothing else: no barrier between the requests and the products.
+  constexpr int WAVE_DW = W2C_CHUNK * NI * 64 + W2C_CHUNK * NI * 4;
+  uint16_t *hs = (uint16_t *)((u32 *)wsm + w * WAVE_DW);   // [W2C_CHUNK][NI][128] bf16
+  float *xsum = (float *)((u32 *)wsm + w * WAVE_DW + W2C_CHUNK * NI * 64);  // [W2C_CHUNK][NI][4]
+  float *red = (float *)((u32 *)wsm + W2C_WAVES * WAVE_DW);  // [W2C_WAVES][RW]
   const int zsh = (rr & 1) * 4;
-  // the activations are requested first: they depend on nothing, and memory answers a wave in order,
-  // so asked for after the tiles they would arrive after them
-  constexpr int HV = 2;  // vectors per thread held in registers (16 K activations); more go through the loop below
-  const int nvec = n_h >> 3;
-  uint4 hv[HV];
-#pragma unroll
-  for (int j = 0; j < HV; ++j) {
-    const int v = tid + j * 64 * W2C_WAVES;
-    const int el = (v < nvec ? v : 0) * 8;
-    hv[j] = el < k * I ? *(const uint4 *)(a.h_r + el) : *(const uint4 *)(a.h_s + (el - k * I));
-  }
+  const int lj = lane >> 4, lpart = lane & 15;  // staging: 16 bytes of item lj of a group (lanes < 16 NI)
   // lane u holds unit u's slot address and weight (lane k: the shared expert); read back with readlane
   u32 ub_lo = 0, ub_hi = 0;
   float uw = 0.f;
@@ -1360,84 +1354,71 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   }
   const Q4Consts q4c = q4_consts();
   float acc = 0.f;
-  // cursor of the wave's current group of NI items: first item = unit u (k = the shared expert), group g
-  int u = 0, g = NI * w;
-  while (u < k && g >= G) { g -= G; ++u; }
-  bool staged = false;
-  do {  // a wave without items still takes part in the staging barrier
+  // A unit's groups are padded to a multiple of NI, so the NI items a wave reads with one load belong to ONE unit
+  // and everything about them but the lane's own byte offsets is wave-uniform: per load the scalar unit builds
+  // four buffer descriptors (tiles, scales, zeros, the unit's h vector) whose lengths end at the unit's real
+  // groups, and a padded, absent or not resident item reads zeros through them (zero weights, scale and
+  // activations: no branch and no per-lane bookkeeping).  With the items enumerated without padding, a load's items
+  // could straddle two units and every lane walked them with selects and 64-bit address arithmetic: 370 vector
+  // operations per wave in front of the first request, 2 us on a SIMD that runs four such waves.
+  const int GP = (G + NI - 1) / NI, GP_sh = (G_sh + NI - 1) / NI;  // loads per routed unit, for the shared expert
+  // cursor of the wave's current load: unit u (k = the shared expert), load gp of that unit
+  int u = 0, gp = w;
+  while (u < k && gp >= GP) { gp -= GP; ++u; }
+  // the lane's byte offsets inside a load's tiles, scale and zero sections and activations
+  const int vq = mine * 1024 + (qd * 16 + rr) * 16, vs = mine * 32 + 2 * rr, vz = mine * 8 + (rr >> 1);
+  const int vh = lj * 256 + lpart * 16;
+  while (u < k || gp < GP_sh) {
     u32x4_t wt[W2C_CHUNK];
     u32 sc[W2C_CHUNK], zz[W2C_CHUNK];
     float wgt[W2C_CHUNK];
-    int ho[W2C_CHUNK];  // where the lane's item keeps its 128 activations in the staged vector
-    // ---- request this chunk's tiles --------------------------------------------------
+    uint4 hv[W2C_CHUNK];  // the lane's 16 bytes of the load's activations on their way into LDS
+    // ---- request this chunk --------------------------------------------------------------------
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
-      // the group's items are consecutive; pick the lane's own while walking them (all uniform but the selects)
-      int uj = u, gj = g;
-      bool on = false;
-      int lu = 0, lg = 0;
-      unsigned long long base = 0ull;
-      float lw = 0.f;
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        const bool onj = uj < k || gj < G_sh;
-        const int ul = onj ? uj : 0;
-        const u32 lo = __builtin_amdgcn_readlane(ub_lo, ul), hi = __builtin_amdgcn_readlane(ub_hi, ul);
-        const float wj = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), ul));
-        const unsigned long long bj = ((unsigned long long)hi << 32) | lo;
-        if (mine == j) { on = onj && bj != 0ull; lu = uj; lg = gj; base = bj; lw = wj; }
-        ++gj;  // next item
-        if (uj < k && gj >= G) { gj -= G; ++uj; }
-      }
-      const bool shd = lu >= k;
+      const bool valid = u < k || gp < GP_sh;
+      const bool shd = u >= k;
+      const u32 lo = __builtin_amdgcn_readlane(ub_lo, u), hi = __builtin_amdgcn_readlane(ub_hi, u);
+      wgt[c] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(u32, uw), u));
+      const unsigned char *bp = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+      const bool live = valid && bp != nullptr;
       const int Gu = shd ? G_sh : G;
-      wgt[c] = lw;
-      ho[c] = on ? (shd ? k * I : lu * I) + lg * 128 : 0;
-      wt[c] = u32x4_t{0u, 0u, 0u, 0u}; sc[c] = 0; zz[c] = 0;
-      if (on) {
-        const unsigned char *bp = (const unsigned char *)base;
-        const size_t t_idx = (size_t)b16 * Gu + lg;
-        wt[c] = *(g_uint4 *)(bp + (shd ? a.sh_off_q : a.off_q) + t_idx * 1024 + (qd * 16 + rr) * 16);
-        sc[c] = *(const __attribute__((address_space(1))) uint16_t *)(bp + (shd ? a.sh_off_s : a.off_s) + t_idx * 32 + 2 * rr);
-        zz[c] = *(const __attribute__((address_space(1))) unsigned char *)(bp + (shd ? a.sh_off_z : a.off_z) + t_idx * 8 + (rr >> 1));
-      }
-      if (u < k || g < G_sh) {  // next group of this wave
-        g += NI * W2C_WAVES;
-        while (u < k && g >= G) { g -= G; ++u; }
+      const u32 n = live ? (u32)Gu : 0u;  // groups the descriptors cover: none for a load that does not exist
+      const size_t blk = (size_t)b16 * Gu;
+      const rsrc_t rq = make_rsrc(bp + (shd ? a.sh_off_q : a.off_q) + blk * 1024, n * 1024u);
+      const rsrc_t rs = make_rsrc(bp + (shd ? a.sh_off_s : a.off_s) + blk * 32, n * 32u);
+      const rsrc_t rz = make_rsrc(bp + (shd ? a.sh_off_z : a.off_z) + blk * 8, n * 8u);
+      const rsrc_t rh = make_rsrc(shd ? a.h_s : a.h_r + (size_t)u * I, n * 256u);
+      const int g0 = NI * gp;
+      // the activations first: memory answers a wave in order, and the products need them with the first tile
+      hv[c] = make_uint4(0u, 0u, 0u, 0u);
+      if (lj < NI) hv[c] = bload16(rh, vh + g0 * 256, 0);
+      const uint4 t4 = bload16(rq, vq + g0 * 1024, 0);
+      wt[c] = u32x4_t{t4.x, t4.y, t4.z, t4.w};
+      sc[c] = bload2(rs, vs + g0 * 32, 0);
+      zz[c] = bload1(rz, vz + g0 * 8, 0);
+      if (valid) {  // next load of this wave
+        gp += W2C_WAVES;
+        while (u < k && gp >= GP) { gp -= GP; ++u; }
       }
     }
-    // ---- first chunk: stage every unit's h vector (+ 32-wide sums) while the tiles travel --------
-    if (!staged) {
-#pragma unroll
-      for (int j = 0; j < HV; ++j) {
-        const int v = tid + j * 64 * W2C_WAVES;
-        float ps = sum8_bf16(hv[j]);
-        ps += __shfl_xor(ps, 1, 64);
-        ps += __shfl_xor(ps, 2, 64);
-        if (v < nvec) {
-          ((uint4 *)hs)[v] = hv[j];
-          if ((tid & 3) == 0) xsum[v >> 2] = ps;
-        }
-      }
-      for (int v = tid + HV * 64 * W2C_WAVES; v < nvec; v += 64 * W2C_WAVES) {
-        const int el = v * 8;
-        const uint4 x4 = el < k * I ? *(const uint4 *)(a.h_r + el) : *(const uint4 *)(a.h_s + (el - k * I));
-        float ps = sum8_bf16(x4);
-        ps += __shfl_xor(ps, 1, 64);
-        ps += __shfl_xor(ps, 2, 64);
-        ((uint4 *)hs)[v] = x4;
-        if ((tid & 3) == 0) xsum[v >> 2] = ps;
-      }
-      __syncthreads();
-      staged = true;
-    }
-    // ---- products: no branch, an absent item has zero weights and a zero scale and reads the first activations
+    // ---- the chunk's activations (+ 32-wide sums) into the wave's own LDS area ----------------------
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
-      const int hoff = ho[c] + qd * 32;  // the lane's 32 activations
-      const uint4 *xp = (const uint4 *)(hs + hoff);
+      float ps = sum8_bf16(hv[c]);
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      if (lj < NI) {
+        ((uint4 *)hs)[(c * NI + lj) * 16 + lpart] = hv[c];
+        if ((lane & 3) == 0) xsum[(c * NI + lj) * 4 + (lpart >> 2)] = ps;
+      }
+    }
+    // ---- products: no branch, an absent item has zero weights, a zero scale and zero activations
+#pragma unroll
+    for (int c = 0; c < W2C_CHUNK; ++c) {
+      const uint4 *xp = (const uint4 *)(hs + (c * NI + mine) * 128 + qd * 32);  // the lane's 32 activations
       const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
-      const float xq = xsum[hoff >> 5];
+      const float xq = xsum[(c * NI + mine) * 4 + qd];
       const float d0 = dot8_q4(wt[c].x, x0, 0.f, q4c), d1 = dot8_q4(wt[c].y, x1, 0.f, q4c);
       const float d2 = dot8_q4(wt[c].z, x2, 0.f, q4c), d3 = dot8_q4(wt[c].w, x3, 0.f, q4c);
       const float d = (d0 + d1) + (d2 + d3);
@@ -1445,7 +1426,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
       const float fz = 128.f + (float)((zz[c] >> zsh) & 15);
       acc = fmaf(wgt[c] * fs, d - fz * xq, acc);
     }
-  } while (u < k || g < G_sh);
+  }
   // the items of the groups, the four k quarters of the wave, then the waves
 #pragma unroll
   for (int m = RW; m < 16; m <<= 1) acc += __shfl_xor(acc, m, 64);
@@ -2536,30 +2517,17 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
     c.sh_off_q = ls.off2_q; c.sh_off_s = ls.off2_s; c.sh_off_z = ls.off2_z;
     c.k = k; c.I = I; c.I_sh = sh ? I_sh : 0; c.H = H; c.G = I / 128; c.G_sh = sh ? I_sh / 128 : 0;
     c.y = (uint16_t *)y_bf16; c.err = err;
-    const size_t n_h = (size_t)k * I + c.I_sh;
-    const size_t lds = n_h * 2 + (n_h / 32) * 4 + W2C_WAVES * 16 * 4;
-    if (lds > 150 * 1024) {
-      moe_set_error("moe_decode_token_int4: fused w2 + combine does not fit LDS (k=%d I=%d)", k, I);
-      return MOE_EINVAL;
-    }
     // two workgroups per 16-row tile (8 rows each): 256 workgroups at H = 2048, one per compute unit; one
     // workgroup per tile took 10.0 us where two take 6.8 us, four no less
-    static bool attr_set = false;
-    if (lds > 64 * 1024 && !attr_set) {
-      for (const void *f : {(const void *)k_w2_combine_token<2, 3>, (const void *)k_w2_combine_token<2, 6>,
-                            (const void *)k_w2_combine_token<1, 7>})
-        if (int rc = moe_check_hip(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                   "hipFuncSetAttribute(k_w2_combine_token)"))
-          return rc;
-      attr_set = true;
-    }
     moe_ktimer_begin(MOE_K_W2, s);
     // loads per wave: the (unit, group) items, two per load, over the 16 waves
-    const int loads_per_wave = ((k * c.G + c.G_sh + 1) / 2 + W2C_WAVES - 1) / W2C_WAVES;
-    if (loads_per_wave <= 3) hipLaunchKernelGGL((k_w2_combine_token<2, 3>), dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+    const int loads_per_wave = (k * ((c.G + 1) / 2) + (c.G_sh + 1) / 2 + W2C_WAVES - 1) / W2C_WAVES;
+    // LDS: per wave the activations and sums of one chunk's items, then the partial sums of the waves
+    auto lds = [](int ni, int chunk) { return (size_t)W2C_WAVES * (chunk * ni * 68) * 4 + W2C_WAVES * 16 * 4; };
+    if (loads_per_wave <= 3) hipLaunchKernelGGL((k_w2_combine_token<2, 3>), dim3(H / 8), dim3(64 * W2C_WAVES), lds(2, 3), s, c);
     else if (H / 16 >= 256)  // one workgroup per 16-row tile already gives every compute unit one: whole tiles
-      hipLaunchKernelGGL((k_w2_combine_token<1, 7>), dim3(H / 16), dim3(64 * W2C_WAVES), lds, s, c);
-    else hipLaunchKernelGGL((k_w2_combine_token<2, 6>), dim3(H / 8), dim3(64 * W2C_WAVES), lds, s, c);
+      hipLaunchKernelGGL((k_w2_combine_token<1, 7>), dim3(H / 16), dim3(64 * W2C_WAVES), lds(1, 7), s, c);
+    else hipLaunchKernelGGL((k_w2_combine_token<2, 6>), dim3(H / 8), dim3(64 * W2C_WAVES), lds(2, 6), s, c);
     moe_ktimer_end(MOE_K_W2, s);
     return moe_check_launch("k_w2_combine_token");
   }
