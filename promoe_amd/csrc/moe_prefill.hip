@@ -305,9 +305,9 @@ __global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
 // weight rows and the 32-row blocks g, g+2, ...), K advances one quantisation group (128) at
 // a time.  The int4 tiles of the slot layout are already in the operand order of
 // v_mfma_f32_16x16x32_f16 (lane = row l&15, k quarter l>>4, dword j = 8 consecutive k), so a
-// wave loads them straight into registers and dequantises there: the nibble pair under mask
-// 0x000f000f is OR-ed into 0x6400 (fp16 1024+q), then (h - (1024+z)) * s with two packed
-// fp16 operations per pair (the subtraction is exact).  gfx950 has packed fp16 arithmetic
+// wave loads them straight into registers and dequantises there: a nibble pair is shifted and masked
+// into the mantissas of two fp16 values 1 + q/16 and one packed fma per pair applies scale and zero
+// (pf_deq8 below).  gfx950 has packed fp16 arithmetic
 // but no packed bf16 arithmetic, hence fp16 operands: activations are converted bf16 -> fp16
 // while they are staged into LDS (exact for |x| < 65504 outside the fp16 subnormal range); the h rows
 // between the two passes are written as fp16 by the w13 epilogue, so the w2 pass stages them as they are.
@@ -325,37 +325,30 @@ static __device__ __forceinline__ u32 pf_bf16x2_to_f16x2(u32 d) {
   auto h = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(d << 16), __uint_as_float(d & 0xffff0000u));
   return __builtin_bit_cast(u32, h);
 }
-// s2 / nz2: the row's scale and -(1024 + zero) as fp16 bit patterns replicated in both halves
-// nibble mask and the fp16 pattern of 1024 held in vector registers, made once per kernel: (d & M) | C is then ONE
-// v_and_or_b32 (a VOP3 instruction takes no literal and one scalar operand on this target; with literals the
-// compiler emits an and and an or, 4 more operations per 8 weights in kernels bound by exactly these operations)
+// Dequantisation of 8 nibbles of a dword into 8 fp16 weights with ONE packed fma per pair: a nibble is masked into
+// mantissa bits 6..9 of an fp16 with the exponent of 1.0, which makes the exact value h = 1 + q/16; with S = 16 s and
+// C = -(16 + zero) s (int4) or C = -(16 s + m) (q4_K), both prepared once per group and row, h S + C = (q - zero) s
+// or q s - m.  The product is exact inside the fma; C carries the one extra rounding (2^-11 of at most 31 s, i.e.
+// 0.015 of a quantisation step, a bias common to the 128 weights of a group row).  The form before this one
+// ((h - (1024 + zero)) s with h = 1024 + q) was exact up to the final rounding and cost a packed subtract and
+// a packed multiply per pair (three operations for q4_K), in kernels that are bound by these operations.
+// Mask and exponent pattern are held in vector registers, made once per kernel: (x & M) | C is then ONE
+// v_and_or_b32 (a VOP3 instruction takes no literal and one scalar operand on this target).
 struct PfDeqConsts { u32 M, C; };
 static __device__ __forceinline__ PfDeqConsts pf_deq_consts() {
-  PfDeqConsts q{0x000f000fu, 0x64006400u};
+  PfDeqConsts q{0x03c003c0u, 0x3c003c00u};
   asm volatile("" : "+v"(q.M), "+v"(q.C));
   return q;
 }
-static __device__ __forceinline__ f16x8_t pf_deq8_f16(u32 d, u32 s2, u32 nz2, const PfDeqConsts &q) {
+// s2 / c2: fp16 bit patterns of S and C replicated in both halves
+static __device__ __forceinline__ f16x8_t pf_deq8(u32 d, u32 s2, u32 c2, const PfDeqConsts &q) {
   const u32 M = q.M, C = q.C;
   u32x4_t v;
-  v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
-  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1024 + q, exact
-  const f16x8_t nz8 = __builtin_bit_cast(f16x8_t, u32x4_t{nz2, nz2, nz2, nz2});
+  v.x = ((d << 6) & M) | C; v.y = ((d << 2) & M) | C; v.z = ((d >> 2) & M) | C; v.w = ((d >> 6) & M) | C;
+  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1 + q/16, exact
   const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
-  return (h + nz8) * s8;                                // exact difference, then one rounding
-}
-
-// q4_K flavour: w = s*q - m with the lane's own sub-block scale s = d*sc and min m = dmin*mn.
-// s2 / nm2: fp16 bit patterns of s and -m replicated in both halves.
-static __device__ __forceinline__ f16x8_t pf_deq8_q4k(u32 d, u32 s2, u32 nm2, const PfDeqConsts &q) {
-  const u32 M = q.M, C = q.C;
-  u32x4_t v;
-  v.x = (d & M) | C; v.y = ((d >> 4) & M) | C; v.z = ((d >> 8) & M) | C; v.w = ((d >> 12) & M) | C;
-  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);
-  const f16x8_t n1024 = __builtin_bit_cast(f16x8_t, u32x4_t{0xe400e400u, 0xe400e400u, 0xe400e400u, 0xe400e400u});
-  const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
-  const f16x8_t nm8 = __builtin_bit_cast(f16x8_t, u32x4_t{nm2, nm2, nm2, nm2});
-  return (h + n1024) * s8 + nm8;  // q exact, then s*q - m
+  const f16x8_t c8 = __builtin_bit_cast(f16x8_t, u32x4_t{c2, c2, c2, c2});
+  return __builtin_elementwise_fma(h, s8, c8);
 }
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
@@ -423,30 +416,33 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
       }
     }
   };
-  auto compute2 = [&](int st, const u32x4_t(&wq)[4], const PiMeta &m, int j0) {
-    const uint16_t *A_ = As + st * PI_BM * PI_LDK + (32 * g + r) * PI_LDK + 32 * qd;
-    u32 s2[4], z2[4];
+  // S = 16 s and C of pf_deq8 for the lane's row in the 4 tiles of a group, once per group
+  auto prep = [&](const PiMeta &m, u32 (&s2)[4], u32 (&c2)[4]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
+      float s16, cz;
       if (Q4K) {
-        const float dsc = __builtin_bit_cast(float, pf_h2f(m.zz[t] & 0xffffu)) * (float)(m.sc[t] & 0xffu);
+        s16 = 16.f * __builtin_bit_cast(float, pf_h2f(m.zz[t] & 0xffffu)) * (float)(m.sc[t] & 0xffu);
         const float dmn = __builtin_bit_cast(float, pf_h2f(m.zz[t] >> 16)) * (float)((m.sc[t] >> 8) & 0xffu);
-        const u32 sb = pf_f2h(dsc), mb = pf_f2h(-dmn);
-        s2[t] = sb | (sb << 16);
-        z2[t] = mb | (mb << 16);
+        cz = -s16 - dmn;
       } else {
-        const u32 sb = m.sc[t] & 0xffffu;
-        s2[t] = sb | (sb << 16);
-        const u32 zb = 0xe400u | ((m.zz[t] >> (4 * (r & 1))) & 15u);  // -(1024 + zero)
-        z2[t] = zb | (zb << 16);
+        const float sf = __builtin_bit_cast(float, pf_h2f(m.sc[t] & 0xffffu));
+        s16 = 16.f * sf;
+        cz = -(16.f + (float)((m.zz[t] >> (4 * (r & 1))) & 15u)) * sf;
       }
+      const u32 sb = pf_f2h(s16), cb = pf_f2h(cz);
+      s2[t] = sb | (sb << 16);
+      c2[t] = cb | (cb << 16);
     }
+  };
+  auto compute2 = [&](int st, const u32x4_t(&wq)[4], const u32 (&s2)[4], const u32 (&z2)[4], int j0) {
+    const uint16_t *A_ = As + st * PI_BM * PI_LDK + (32 * g + r) * PI_LDK + 32 * qd;
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
       const int j = j0 + jj;
       f16x8_t wd[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wd[t] = Q4K ? pf_deq8_q4k(wq[t][j], s2[t], z2[t], dqc) : pf_deq8_f16(wq[t][j], s2[t], z2[t], dqc);
+      for (int t = 0; t < 4; ++t) wd[t] = pf_deq8(wq[t][j], s2[t], z2[t], dqc);
 #pragma unroll
       for (int tb = 0; tb < 2 * NBW; ++tb) {
         const f16x8_t xa = *(const f16x8_t *)(A_ + (64 * (tb >> 1) + 16 * (tb & 1)) * PI_LDK + 8 * j);
@@ -464,11 +460,13 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
     gloadA(gn, 0);
     if (NBW > 0) gloadW(nxt, mn, gn);
     __builtin_amdgcn_sched_barrier(0);
-    if (NBW > 0) compute2(gi & 1, cur, mc, 0);
+    u32 s2[4], c2[4];
+    if (NBW > 0) prep(mc, s2, c2);
+    if (NBW > 0) compute2(gi & 1, cur, s2, c2, 0);
     if (more) sstore((gi + 1) & 1, 0);
     gloadA(gn, 1);
     __builtin_amdgcn_sched_barrier(0);
-    if (NBW > 0) compute2(gi & 1, cur, mc, 2);
+    if (NBW > 0) compute2(gi & 1, cur, s2, c2, 2);
     if (more) {
       if (nb > 3) sstore((gi + 1) & 1, 1);
       __syncthreads();
