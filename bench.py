@@ -447,7 +447,7 @@ def main():
     D_k = float(np.mean([int(r.n_active.cpu()[0]) for r in routed]))
     w13_bytes_k = D_k * lay_r["off2_q"] + lay_s["off2_q"] + 2 * T * H
     achieved = w13_bytes_k / (w13_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": "k_gemv_int4 (w13 + SwiGLU%s)" % (", routing in the kernel" if T == 1 else ""),
+    roofline = {"bound": "hbm", "kernel": ("k_w13_token (w13 + SwiGLU, routing in the kernel)" if T == 1 else "k_gemv_int4_mfma (w13 + SwiGLU)"),
                 "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this kernel at this
