@@ -1243,25 +1243,34 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
     }
     if (scj < 2 * CH) wsc[lane] = sd;
     if (zzj < 2 * CH) wzz[lane] = zd;
+    // everything the products need besides the tiles is read and converted before the first tile is waited
+    // for: what a wave does after its last byte has arrived (all tiles of a wave arrive together) is the tail
+    // of the launch, and only the unpacking and the dot products have to be in it
+    float fsa[CH], fsb[CH], fza[CH], fzb[CH], xq[CH];
+    uint4 xr[CH][4];
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       const bool valid = jc + j < GPW;
       // a clamped (duplicate) tile contributes through a zero scale
       const float fsa_ = half_bits_to_f32(wsc_h[j * 16 + r]), fsb_ = half_bits_to_f32(wsc_h[(CH + j) * 16 + r]);
-      const float fsa = valid ? fsa_ : 0.f, fsb = valid ? fsb_ : 0.f;
-      const float fza = 128.f + (float)((wzz_b[j * 8 + (r >> 1)] >> zsh) & 15);
-      const float fzb = 128.f + (float)((wzz_b[(CH + j) * 8 + (r >> 1)] >> zsh) & 15);
+      fsa[j] = valid ? fsa_ : 0.f;
+      fsb[j] = valid ? fsb_ : 0.f;
+      xq[j] = xsum[j * 4 + qd];
+      fza[j] = 128.f + (float)((wzz_b[j * 8 + (r >> 1)] >> zsh) & 15);
+      fzb[j] = 128.f + (float)((wzz_b[(CH + j) * 8 + (r >> 1)] >> zsh) & 15);
       const uint4 *xp = (const uint4 *)(xs + j * 128 + qd * 32);
-      const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
-      const float xq = xsum[j * 4 + qd];
-      float dA = dot8_q4(wa[j].x, x0, 0.f, q4c);
-      float dB = dot8_q4(wb[j].x, x0, 0.f, q4c);
-      dA = dot8_q4(wa[j].y, x1, dA, q4c); dB = dot8_q4(wb[j].y, x1, dB, q4c);
-      dA = dot8_q4(wa[j].z, x2, dA, q4c); dB = dot8_q4(wb[j].z, x2, dB, q4c);
-      dA = dot8_q4(wa[j].w, x3, dA, q4c); dB = dot8_q4(wb[j].w, x3, dB, q4c);
-      accA = fmaf(fsa, dA - fza * xq, accA);
-      accB = fmaf(fsb, dB - fzb * xq, accB);
-      // keep the scheduler from hoisting the next tile's LDS reads (register pressure)
+      xr[j][0] = xp[0]; xr[j][1] = xp[1]; xr[j][2] = xp[2]; xr[j][3] = xp[3];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      float dA = dot8_q4(wa[j].x, xr[j][0], 0.f, q4c);
+      float dB = dot8_q4(wb[j].x, xr[j][0], 0.f, q4c);
+      dA = dot8_q4(wa[j].y, xr[j][1], dA, q4c); dB = dot8_q4(wb[j].y, xr[j][1], dB, q4c);
+      dA = dot8_q4(wa[j].z, xr[j][2], dA, q4c); dB = dot8_q4(wb[j].z, xr[j][2], dB, q4c);
+      dA = dot8_q4(wa[j].w, xr[j][3], dA, q4c); dB = dot8_q4(wb[j].w, xr[j][3], dB, q4c);
+      accA = fmaf(fsa[j], dA - fza[j] * xq[j], accA);  // (the expression of k_gemv_int4: the same bits)
+      accB = fmaf(fsb[j], dB - fzb[j] * xq[j], accB);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
