@@ -260,7 +260,12 @@ def test_decode_q4k_qwen2_shape(cuda):
 
 
 @pytest.mark.parametrize("H,I,E,k,mode,I_sh,zipf", [(2048, 1408, 16, 6, 0, 2816, 1.2), (256, 384, 8, 2, 2, 256, None),
-                                                    (256, 256, 60, 4, 1, 512, 1.1), (512, 128, 200, 8, 0, 0, None)])
+                                                    (256, 256, 60, 4, 1, 512, 1.1), (512, 128, 200, 8, 0, 0, None),
+                                                    # 8, 12, 28 and 1 quantisation groups per row: two and three tiles
+                                                    # in flight per wave and block, a partial second chunk, waves
+                                                    # without a group
+                                                    (1024, 256, 8, 2, 0, 128, None), (1536, 384, 8, 3, 1, 0, None),
+                                                    (3584, 256, 8, 2, 2, 256, None), (128, 128, 8, 2, 0, 128, None)])
 def test_token_decode_routes_in_kernel_like_separate_kernels(cuda, H, I, E, k, mode, I_sh, zipf):
     """One token: the w13 kernel derives the routing itself.  Indices, weights, dispatch arrays and
     the layer output must equal those of gate -> top-k -> dispatch -> experts -> combine, bit for bit."""
