@@ -210,8 +210,8 @@ int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k,
  * callers that cannot allocate or hand over workspaces (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  Inputs and outputs are the caller's: x, logits (E fp32), the slot table,
  * the shared expert, y, and the error word err (device or pinned host memory, cleared by the caller; set to 1
- * when a selected expert is not resident).  Limits: E <= 256, k <= 32, k*I + I_sh <= 71680 (what the
- * fused w2 + combine kernel stages in LDS), H <= 16384; beyond them MOE_EINVAL.  All calls on one GPU share the array:
+ * when a selected expert is not resident).  Limits: E <= 256, k <= 32, k*I + I_sh <= 71680 (the room
+ * the array has for the h vectors), H <= 16384; beyond them MOE_EINVAL.  All calls on one GPU share the array:
  * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered. */
 int64_t moe_noalloc_scratch_bytes(void);
 int moe_decode_token_int4_noalloc(const void *x_bf16, const float *logits, int E, int k, int mode, int H, int I,

@@ -2557,7 +2557,7 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
 // ---------------------------------------------------------------------------
 #define NOALLOC_MAX_E 256
 #define NOALLOC_MAX_K 32
-#define NOALLOC_MAX_H_ELEMS 71680   /* k*I + I_sh bf16 values: what the fused w2 + combine kernel can stage in LDS */
+#define NOALLOC_MAX_H_ELEMS 71680   /* k*I + I_sh bf16 values: the room the scratch array has for the h vectors */
 struct NoAllocScratch {
   int idx[NOALLOC_MAX_K];
   float w[NOALLOC_MAX_K];
