@@ -77,3 +77,49 @@ def test_no_alloc_entry_point_equals_the_workspace_one(cuda):
         ops.decode_token_int4_noalloc(xd, logits, 8, 2, 2, table, shared, 256, 36864, 256, y, err, sg_logit=sg)
     with pytest.raises(L.MoeError, match="beyond the static scratch"):
         ops.decode_token_int4_noalloc(xd, logits, 300, 2, 2, table, shared, 256, 384, 256, y, err, sg_logit=sg)
+
+
+def test_no_alloc_entry_point_in_a_replayed_graph(cuda):
+    """What the entry point is for: a caller under HIP graph capture.  The gate logits and the entry point are
+    recorded once and replayed for three different inputs, with eager work and synchronisations between the
+    replays; every replay must equal the eager workspace entry point bit for bit."""
+    from promoe_amd import ops
+    print("case no-alloc entry point recorded into a HIP graph and replayed", flush=True)
+    layer = Int4Layer(H=2048, I=1408, E=16, I_sh=2816, seed=23, zipf=1.2)
+    H, I, E, I_sh, k, mode = layer.H, layer.I, layer.E, layer.I_sh, 6, 0
+    slots = [torch.from_numpy(s).to(cuda) for s in layer.slots]
+    table = torch.tensor([s.data_ptr() for s in slots], dtype=torch.int64, device=cuda)
+    shared = torch.from_numpy(layer.shared_img).to(cuda)
+    wg = bf16_dev(layer.wg, cuda)
+    bias = None if layer.bias is None else torch.from_numpy(layer.bias).to(cuda)
+    xd = bf16_dev(O.synth_acts(1, H, seed=30), cuda)
+    logits = ops.gate_logits(xd, wg, bias)
+    y = torch.zeros(1, H, dtype=torch.bfloat16, device=cuda)
+    err = torch.zeros(1, dtype=torch.int32, device=cuda)
+    # once eagerly: the library looks up its array's address on the first call on a device
+    ops.decode_token_int4_noalloc(xd, logits, E, k, mode, table, shared, H, I, I_sh, y, err)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side, capture_error_mode="thread_local"):
+            ops.gate_logits(xd, wg, bias, out=logits)
+            ops.decode_token_int4_noalloc(xd, logits, E, k, mode, table, shared, H, I, I_sh, y, err)
+    torch.cuda.synchronize()
+    unit_ws = torch.zeros(32 * k, dtype=torch.uint8, device=cuda)
+    for seed in (31, 32, 33):
+        x_new = bf16_dev(O.synth_acts(1, H, seed=seed), cuda)
+        xd.copy_(x_new)                                    # eager work between the replays
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        lg_ref = ops.gate_logits(x_new, wg, bias)
+        y_ref = torch.full((1, H), float("nan"), dtype=torch.bfloat16, device=cuda)
+        ws = ops.decode_token_int4(x_new, lg_ref, E, k, mode, table, shared, H, I, I_sh, phases=5, unit_ws=unit_ws,
+                                   y=y_ref)
+        torch.cuda.synchronize()
+        assert int(ws[5].cpu()[0]) == 0 and int(err.cpu()[0]) == 0
+        assert torch.equal(logits, lg_ref)
+        assert torch.equal(y.view(torch.int16), y_ref.view(torch.int16)), seed
