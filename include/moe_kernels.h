@@ -252,6 +252,19 @@ int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int I_sh, int k
                         float *part_r, float *part_s, void *tiles_ws, int *err, int phases,
                         void *stream);
 
+/* The same with the shared expert's partial rows of the w2 pass in shared_pieces pieces (1, 2, 4 or 8; nibble
+ * formats only): part_s holds shared_pieces * T rows, piece s at part_s + s*T*H, each the product over one window
+ * of the I_sh columns; moe_combine_splits adds them.  moe_prefill_shared_splits(fmt, T, H, I_sh) = the number of
+ * pieces worth taking: more than 1 where the shared expert's workgroups of that pass (ceil(T/128) * H/256, each over
+ * the whole reduction) are few and the reduction is long, so that they would outlast the rest of the launch
+ * (Qwen2-57B shape at 512 tokens: 4).  No reference counterpart (see moe_decode_shared_splits). */
+int moe_prefill_shared_splits(int fmt, int T, int H, int I_sh);
+int moe_experts_prefill_pieces(const void *x_bf16, int T, int H, int I, int I_sh, int k, int fmt,
+                               const moe_unit *units, int max_units, const int *sorted_tok,
+                               const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
+                               float *part_r, float *part_s, int shared_pieces, void *tiles_ws, int *err,
+                               int phases, void *stream);
+
 /* k5: y[t,:] = sum_j w[t,j] * part_r[pos_of_pair[t*k+j],:] + g_t * part_s[t,:], bf16 out.
  * g_t = sigmoid(shared_gate_logit[t*sg_stride]) when shared_gate_logit != NULL, else 1;
  * part_s may be NULL (no shared expert). */

@@ -69,6 +69,8 @@ _sig("moe_experts_decode_q4k", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp
 _sig("moe_prefill_workspace_bytes", [i32, i32, i32], C.c_int64)
 _sig("moe_prefill_tile_rows", [])
 _sig("moe_experts_prefill", [vp, i32, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])
+_sig("moe_experts_prefill_pieces", [vp, i32, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, i32, vp])
+_sig("moe_prefill_shared_splits", [i32, i32, i32, i32])
 _sig("moe_kernel_timing", [i32])
 _sig("moe_kernel_timing_read", [i32, C.POINTER(C.c_double), C.POINTER(i32)])
 _sig("moe_combine", [vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, vp])

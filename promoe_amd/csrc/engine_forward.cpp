@@ -16,6 +16,7 @@ struct LayerState {
   int max_tokens = 0, max_k = 0, max_units = 0;
   int E = 0, H = 0, I = 0, I_sh = 0;
   float *logits = nullptr, *topk_w = nullptr, *part_r = nullptr, *part_s = nullptr;
+  size_t part_s_elems = 0;  // floats behind part_s
   int *idx = nullptr, *counts = nullptr, *offsets = nullptr, *sorted_pair = nullptr, *pos_of_pair = nullptr,
       *sorted_tok = nullptr, *n_active = nullptr;
   unsigned *route_counter = nullptr;
@@ -160,8 +161,14 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, (uint16_t **)&s->h_r, P * I);
   rc |= dalloc(s, (uint16_t **)&s->h_s, (size_t)T * I_sh);
   rc |= dalloc(s, &s->part_r, P * H);
-  // q4_K decode batches (at most 16 tokens) may leave the shared expert's partial rows in up to 8 pieces
-  rc |= dalloc(s, &s->part_s, (size_t)(T > 128 ? T : 128) * H);
+  // q4_K decode batches (at most 16 tokens) may leave the shared expert's partial rows in up to 8 pieces, and so
+  // may a prefill batch of a nibble format whose shared expert is wide (pieces x tokens rows, largest over the
+  // batch sizes the workspace admits)
+  size_t rows_s = T > 128 ? T : 128;
+  for (int t = 1; t <= T; ++t)
+    rows_s = std::max(rows_s, (size_t)t * (size_t)moe_prefill_shared_splits(MOE_FMT_Q4K, t, H, I_sh));
+  rc |= dalloc(s, &s->part_s, rows_s * H);
+  s->part_s_elems = rows_s * H;
   rc |= dalloc(s, (unsigned char **)&s->tiles_ws, (size_t)moe_prefill_workspace_bytes(T, k, s->max_units));
   s->disp_ws_bytes = moe_dispatch_workspace_bytes(T, k, E);
   if (s->disp_ws_bytes) rc |= dalloc(s, &s->disp_ws, (size_t)s->disp_ws_bytes);
@@ -238,15 +245,17 @@ static bool use_prefill(const moe_layer_desc &d, int T) {
   return T > gemv_tmax && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
 }
 
+static int shared_pieces(const moe_layer_desc &d, int T, const LayerState *s);
 // pub / pub_seq: the pending slot whose pinned unit list the w13 launch fills (decode_publishes), or null
 static int run_units(moe_engine *eng, const moe_layer_desc &d, LayerState *s, const void *x, int T,
                      const moe_unit *units_dev, const moe_unit *units_host, int n_units, bool with_shared,
                      int layer, const uint64_t *table, hipStream_t st, LayerState::Pending *pub = nullptr,
                      int pub_seq = 0) {
   if (use_prefill(d, T))
-    return moe_experts_prefill(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
-                               s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
-                               s->part_s, s->tiles_ws, s->err_host + layer, 3, st);
+    return moe_experts_prefill_pieces(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, d.fmt, units_dev, n_units,
+                                      s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s, s->part_r,
+                                      s->part_s, with_shared ? shared_pieces(d, T, s) : 1, s->tiles_ws,
+                                      s->err_host + layer, 3, st);
   if (d.fmt == MOE_FMT_Q4K)
     return moe_experts_decode_q4k(x, T, d.H, d.I, with_shared ? d.I_sh : 0, d.top_k, units_dev, n_units,
                                   s->sorted_tok, table, with_shared ? d.shared : nullptr, s->h_r, s->h_s,
@@ -266,8 +275,14 @@ static bool decode_publishes(const moe_layer_desc &d, int T, int max_units) {
 }
 
 // pieces the expert launch of run_units leaves the shared expert's partial rows in
-static int shared_pieces(const moe_layer_desc &d, int T) {
-  return d.I_sh > 0 && d.fmt == MOE_FMT_Q4K && !use_prefill(d, T) ? moe_decode_shared_splits(MOE_FMT_Q4K, T, d.H, d.I_sh) : 1;
+static int shared_pieces(const moe_layer_desc &d, int T, const LayerState *s) {
+  if (d.I_sh <= 0) return 1;
+  if (use_prefill(d, T)) {
+    // (what the workspace was sized for; a layer narrower than the widest one could ask for more pieces than fit)
+    const int sp = moe_prefill_shared_splits(d.fmt, T, d.H, d.I_sh);
+    return (size_t)sp * T * d.H <= s->part_s_elems ? sp : 1;
+  }
+  return d.fmt == MOE_FMT_Q4K ? moe_decode_shared_splits(MOE_FMT_Q4K, T, d.H, d.I_sh) : 1;
 }
 
 // what the one-token w2 + combine kernel asks of a layer (its waves stage what they need themselves, so the
@@ -567,7 +582,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       return rc;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k,
-                                 shared_pieces(d, T), st)))
+                                 shared_pieces(d, T, s), st)))
       return rc;
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
@@ -644,7 +659,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   }
   const float *sg = d.shared_gated ? s->logits + E : nullptr;
   if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg, ldl, y, T, d.H, k,
-                               shared_pieces(d, T), st)))
+                               shared_pieces(d, T, s), st)))
     return rc;
   // MoeLayerHook.post_forward (utils/hooks.py:220-223)
   if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;

@@ -48,7 +48,10 @@ struct PfClass {
   int act_stride, out_stride, K, n_ntiles, n_mtiles, n_cols_per_tile;
   int m_fastest;        // block order inside the class
   int slab_step;        // storage rotation per 128-row group: smallest odd s >= 3 coprime with K/64
-  int n_blocks;         // n_mtiles * n_ntiles
+  int n_blocks;         // n_mtiles * n_ntiles * ksplit
+  int ksplit;           // int4 / q4_K w2 pass of the shared expert: workgroups per tile, each over 1/ksplit of the
+                        // reduction, partial rows to out + split * split_stride (0 or 1: the whole reduction)
+  long long split_stride;  // elements between the pieces of out
 };
 struct PfArgs {
   PfClass c[2];
@@ -374,9 +377,11 @@ struct PiMeta { u32 sc[4]; u32 zz[4]; };  // raw fp16 scale bits / zero nibble o
 
 // ACT16: the activations are fp16 already (the h rows this kernel's w13 pass wrote, or a converted copy of x):
 // staged as they are, without the three vector operations per pair of the bf16 -> fp16 conversion
+// Gt: quantisation groups per weight row in memory; this workgroup reduces over the window [g0, g0 + G) of them
 template <int NBW, bool Q4K, bool ACT16>
 static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_t *As, const rsrc_t rx, const u32 (&a_off)[6],
-                                                   const rsrc_t rq, const rsrc_t rs, const rsrc_t rz, int G, int nb, int tid) {
+                                                   const rsrc_t rq, const rsrc_t rs, const rsrc_t rz, int Gt, int g0, int G,
+                                                   int nb, int tid) {
   const int lane = tid & 63, g = tid >> 8;
   const int r = lane & 15, qd = lane >> 4;
   const int ch = tid & 15, r0 = tid >> 4;  // staging: row r0 + 32 i (block i), 16-byte chunk ch of the 128-k group
@@ -388,7 +393,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   auto gloadA = [&](int gi, int half) {
 #pragma unroll
     for (int i = 0; i < 3; ++i)  // unconditional (blocks past the tile's end re-read its first rows): the same
-      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[3 * half + i], gi * 256, 0);  // number of loads in every iteration
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, a_off[3 * half + i], (g0 + gi) * 256, 0);  // number of loads in every iteration
   };
   auto sstore = [&](int st, int half) {
     uint16_t *A_ = As + st * PI_BM * PI_LDK;
@@ -406,13 +411,14 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   auto gloadW = [&](u32x4_t(&wq)[4], PiMeta &m, int gi) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      wq[t] = __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, (t * G + gi) * 1024, 0);
+      const int gm = g0 + gi;  // the group in memory
+      wq[t] = __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, (t * Gt + gm) * 1024, 0);
       if (Q4K) {  // (sc, m) byte pair of the lane's sub-block; (d, dmin) of the row's super-block
-        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * lane, (t * G + gi) * 128, 0);
-        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b32(rz, 4 * r, (t * (G >> 1) + (gi >> 1)) * 64, 0);
+        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * lane, (t * Gt + gm) * 128, 0);
+        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b32(rz, 4 * r, (t * (Gt >> 1) + (gm >> 1)) * 64, 0);
       } else {
-        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * r, (t * G + gi) * 32, 0);
-        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, r >> 1, (t * G + gi) * 8, 0);
+        m.sc[t] = __builtin_amdgcn_raw_buffer_load_b16(rs, 2 * r, (t * Gt + gm) * 32, 0);
+        m.zz[t] = __builtin_amdgcn_raw_buffer_load_b8(rz, r >> 1, (t * Gt + gm) * 8, 0);
       }
     }
   };
@@ -495,19 +501,27 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   // block order: as in k_prefill_gemm
   int ci, pb;
   pf_block_of(a, ci, pb);
-  const int n_mt = *a.c[ci].n_tiles_real;
-  const int n_real = n_mt * a.c[ci].n_ntiles;
+  const PfClass &c = a.c[ci];
+  const int n_mt = *c.n_tiles_real;
+  // a class whose reduction is split has ksplit workgroups per tile: the pieces of one tile are `n_tiles`
+  // blocks apart, so that the first piece of every tile starts before the second of any
+  const int ks = c.ksplit > 1 ? c.ksplit : 1;
+  const int n_tiles = n_mt * c.n_ntiles;
+  const int n_real = n_tiles * ks;
   const int per_xcd = (n_real + 7) >> 3;
   if ((pb >> 3) >= per_xcd) return;
   int bid = (pb & 7) * per_xcd + (pb >> 3);
   if (bid >= n_real) return;
-  const PfClass &c = a.c[ci];
+  const int split = bid / n_tiles;
+  bid -= split * n_tiles;
   int mt, nt;
   if (c.m_fastest) { nt = bid / n_mt; mt = bid - nt * n_mt; }
   else { mt = bid / c.n_ntiles; nt = bid - mt * c.n_ntiles; }
   const PfTile tile = c.tiles[mt];
   if (tile.rows <= 0) return;
   const int K = c.K, G = K >> 7;
+  // this workgroup's window of quantisation groups (only the w2 pass is ever split: a constant 0 in the w13 pass)
+  const int Gw = SWIGLU ? G : G / ks, g0 = SWIGLU ? 0 : split * Gw;
 
   const int ch = tid & 15, r0 = tid >> 4;
   u32 a_off[6];  // byte offsets into the activation matrix (< 2^31: checked by the launcher)
@@ -537,10 +551,10 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
   const int nb = (tile.rows + 31) >> 5;
   const int nbw = (nb - g + 1) >> 1;
   switch (nbw) {
-    case 0: pi_mainloop<0, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 1: pi_mainloop<1, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    case 2: pi_mainloop<2, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
-    default: pi_mainloop<3, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, nb, tid); break;
+    case 0: pi_mainloop<0, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, g0, Gw, nb, tid); break;
+    case 1: pi_mainloop<1, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, g0, Gw, nb, tid); break;
+    case 2: pi_mainloop<2, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, g0, Gw, nb, tid); break;
+    default: pi_mainloop<3, Q4K, ACT16>(acc, As, rx, a_off, rq, rs, rz, G, g0, Gw, nb, tid); break;
   }
   // epilogue.  acc[t][tb] element i of lane l: weight row r of tile t, token row
   // 32*(2*(tb/2)+g) + 16*(tb%2) + 4*qd + i of the tile
@@ -559,7 +573,7 @@ __global__ __launch_bounds__(512, 1) void k_prefill_int4(const PfArgs a) {
           }
         } else {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) ((float *)c.out)[orow + 16 * (rb0 + t) + r] = acc[t][tb][i];
+          for (int t = 0; t < 4; ++t) ((float *)c.out)[(size_t)split * c.split_stride + orow + 16 * (rb0 + t) + r] = acc[t][tb][i];
         }
       }
     }
@@ -684,13 +698,47 @@ extern "C" int64_t moe_prefill_workspace_bytes(int T, int k, int max_units) {
   return (P / 128 + max_units + 2 * ((T + 127) / 128) + 3) * (int64_t)sizeof(PfTile);  // covers every tile height in use (>= 128)
 }
 
+// Pieces the w2 pass leaves the shared expert's partial rows in (moe_experts_prefill_pieces).  The shared expert's
+// workgroups of that pass each reduce over all of I_sh; where there are few of them (ceil(T/128) row tiles x H/256
+// column tiles) and the reduction is long, they outlast everything else in the launch: Qwen2-57B shape (H 3584,
+// I_sh 20480) at 512 tokens, 56 workgroups over 160 groups each: 371 us for the launch, 285 us with the reduction in 4
+// windows (8 windows: no shorter, and the combine reads twice the partial rows).  Then the reduction is cut into 2, 4
+// or 8 windows of at least 32 groups, a workgroup per tile and window, until there are 192 of them.
+extern "C" int moe_prefill_shared_splits(int fmt, int T, int H, int I_sh) {
+  if ((fmt != MOE_FMT_INT4_G128 && fmt != MOE_FMT_Q4K) || T <= 0 || H <= 0 || I_sh <= 0) return 1;
+  const int tiles = ((T + PF_BM_SHARED_W2 - 1) / PF_BM_SHARED_W2) * (H / (2 * PF_BNH));
+  const int G = I_sh / 128;
+  int s = 1;
+  while (s < 8 && tiles * s < 192 && G % (s * 4) == 0 && G / (s * 2) >= 32) s *= 2;
+  return s;
+}
+
 extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int I_sh, int k, int fmt,
                                    const moe_unit *units, int max_units, const int *sorted_tok,
                                    const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
                                    float *part_r, float *part_s, void *tiles_ws, int *err, int phases,
                                    void *stream) {
+  return moe_experts_prefill_pieces(x_bf16, T, H, I, I_sh, k, fmt, units, max_units, sorted_tok, expert_ptr, shared_ptr,
+                                    h_r, h_s, part_r, part_s, 1, tiles_ws, err, phases, stream);
+}
+
+extern "C" int moe_experts_prefill_pieces(const void *x_bf16, int T, int H, int I, int I_sh, int k, int fmt,
+                                          const moe_unit *units, int max_units, const int *sorted_tok,
+                                          const uint64_t *expert_ptr, const void *shared_ptr, void *h_r, void *h_s,
+                                          float *part_r, float *part_s, int shared_pieces, void *tiles_ws, int *err,
+                                          int phases, void *stream) {
   hipStream_t s = (hipStream_t)stream;
   if (T == 0) return MOE_OK;
+  if (shared_pieces != 1 && shared_pieces != 2 && shared_pieces != 4 && shared_pieces != 8) {
+    moe_set_error("moe_experts_prefill: shared_pieces = %d (1, 2, 4 or 8)", shared_pieces);
+    return MOE_EINVAL;
+  }
+  if (shared_pieces > 1 && (!shared_ptr || (fmt != MOE_FMT_INT4_G128 && fmt != MOE_FMT_Q4K) ||
+                            (I_sh / 128) % (shared_pieces * 2) != 0)) {
+    moe_set_error("moe_experts_prefill: %d pieces need an int4 / q4_K shared expert whose I_sh / 128 is a multiple of %d "
+                  "(I_sh=%d)", shared_pieces, shared_pieces * 2, I_sh);
+    return MOE_EINVAL;
+  }
   if (!x_bf16 || T < 0 || k <= 0 || max_units < 0 || !units || !sorted_tok || !expert_ptr || !tiles_ws || !err ||
       !h_r || !part_r || (shared_ptr && (!h_s || !part_s || I_sh <= 0))) {
     moe_set_error("moe_experts_prefill: NULL or negative argument");
@@ -759,7 +807,9 @@ extern "C" int moe_experts_prefill(const void *x_bf16, int T, int H, int I, int 
         c.off_s = w2 ? lay.off2_s : lay.off13_s;
         c.off_z = w2 ? lay.off2_z : lay.off13_z;
       }
-      c.n_blocks = c.n_mtiles * c.n_ntiles;
+      c.ksplit = (w2 && shared && int4) ? shared_pieces : 1;
+      c.split_stride = (long long)T * H;
+      c.n_blocks = c.n_mtiles * c.n_ntiles * c.ksplit;
       c.slab_step = pf_slab_step(c.K / PF_BK);
       a.n_blocks_total += c.n_blocks;
     }

@@ -231,7 +231,8 @@ def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.T
 
 def experts_prefill(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tensor | None,
                     H: int, I: int, I_sh: int, fmt: int = L.FMT_BF16, phases: int = 3, ws=None):
-    """MFMA grouped expert product.  Returns (part_r, part_s, err, h_r, h_s, tiles)."""
+    """MFMA grouped expert product.  Returns (part_r, part_s, err, h_r, h_s, tiles).  part_s has S*T rows, S =
+    moe_prefill_shared_splits pieces of the shared expert's w2 product (combine adds them; S = 1 mostly)."""
     T, k = d.T, d.k
     P = T * k
     dev = x.device
@@ -243,13 +244,18 @@ def experts_prefill(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.Tens
         h_s = part_s = None
         if shared is not None:
             h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
-            part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+            part_s = torch.empty(int(lib.moe_prefill_shared_splits(fmt, T, H, I_sh)) * T, H, dtype=torch.float32, device=dev)
         err = torch.zeros(1, dtype=torch.int32, device=dev)
         tiles = torch.empty(max(int(lib.moe_prefill_workspace_bytes(T, k, d.max_units)), 16), dtype=torch.uint8, device=dev)
-    check(lib.moe_experts_prefill(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k, fmt,
-                                  ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
-                                  ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s), ptr(tiles),
-                                  ptr(err), phases, cur_stream()), "moe_experts_prefill")
+    pieces = 1
+    if part_s is not None:
+        pieces = int(lib.moe_prefill_shared_splits(fmt, T, H, I_sh))
+        if part_s.shape[0] != pieces * T:   # a workspace made for another batch size or format
+            part_s = torch.empty(pieces * T, H, dtype=torch.float32, device=dev)
+    check(lib.moe_experts_prefill_pieces(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k, fmt,
+                                         ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
+                                         ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s), pieces, ptr(tiles),
+                                         ptr(err), phases, cur_stream()), "moe_experts_prefill")
     return part_r, part_s, err, h_r, h_s, tiles
 
 

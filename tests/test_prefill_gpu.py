@@ -131,3 +131,18 @@ def test_prefill_q4k_variants(cuda):
     print("case prefill_q4k_variants", flush=True)
     check_prefill(Q4KLayer(H=512, I=256, E=8, I_sh=0, seed=4), 200, 2, 2, cuda)
     check_prefill(Q4KLayer(H=256, I=256, E=60, I_sh=512, seed=5, shared_gate=True, zipf=1.1), 515, 8, 0, cuda)
+
+
+def test_prefill_wide_shared_expert_in_pieces(cuda):
+    """A shared expert much wider than the routed ones over few tokens: the w2 pass cuts its reduction into
+    windows (moe_prefill_shared_splits) and leaves one piece of partial rows per window for the combine."""
+    from promoe_amd import _lib as L
+    print("case prefill shared expert in pieces", flush=True)
+    assert L.lib.moe_prefill_shared_splits(L.FMT_Q4K, 130, 256, 16384) == 4
+    assert L.lib.moe_prefill_shared_splits(L.FMT_INT4_G128, 200, 256, 8192) == 2
+    assert L.lib.moe_prefill_shared_splits(L.FMT_BF16, 130, 256, 16384) == 1       # nibble formats only
+    assert L.lib.moe_prefill_shared_splits(L.FMT_INT4_G128, 2048, 2048, 2816) == 1  # DeepSeek shape: 22 groups
+    assert L.lib.moe_prefill_shared_splits(L.FMT_Q4K, 512, 3584, 20480) == 4        # Qwen2-57B shape
+    check_prefill(Q4KLayer(H=256, I=256, E=4, I_sh=16384, seed=6, shared_gate=True), 130, 2, 0, cuda)
+    check_prefill(Int4Layer(H=256, I=128, E=4, I_sh=8192, seed=7), 200, 2, 1, cuda)
+    check_prefill(Int4Layer(H=512, I=128, E=4, I_sh=8192, seed=8), 70, 2, 0, cuda)   # 1 x 2 tiles: 2 pieces, short last tile
