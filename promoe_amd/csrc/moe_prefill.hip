@@ -171,8 +171,8 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsign
       for (int n = 0; n < NL; ++n)
         if (n * NS / NL == g) {  // request n of this step goes out behind product group g
           if (n < NB) dma(n, kt + 3, (S + 3) % PF4_RING);
-          else if (n - NB < 4) far[0][n - NB] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB), sb0, 0);
-          else far[1][n - NB - 4] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB - 4), sb1, 0);
+          else if (n - NB < 4) far[0][n - NB] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB), sb0, 2);
+          else far[1][n - NB - 4] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB - 4), sb1, 2);
         }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -184,9 +184,9 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsign
   auto gloadB = [&](u32x4_t(&b)[2][4], int kt) {
     const int sb0 = bslab(kt, rot0), sb1 = bslab(kt, rot1) + b_delta1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[0][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb0, 0);
+    for (int j = 0; j < 4; ++j) b[0][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb0, 2);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[1][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb1, 0);
+    for (int j = 0; j < 4; ++j) b[1][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb1, 2);
   };
 #pragma unroll
   for (int t = 0; t < 3; ++t) {
