@@ -1,11 +1,16 @@
-"""Host model of the index arithmetic of the one-token decode GEMV (k_gemv_int4 with in-kernel routing,
-promoe_amd/csrc/moe_kernels.hip) and of its launcher (moe_decode_token_int4), swept over layer shapes.
+"""Host model of the index arithmetic of the two kernels of a one-token decode step (k_w13_token and
+k_w2_combine_token, promoe_amd/csrc/moe_kernels.hip) and of their launcher (moe_decode_token_int4), swept over
+layer shapes.
 
-For every workgroup of the launch the model restates which (class, unit, block) it takes, the byte ranges
-of its three buffer resources inside the expert image, every LDS offset it stages to or reads from against
-the dynamic LDS size the launcher passes, the output elements it stores against the extents of h_r / h_s,
-and what the publishing workgroup stores against the sizes moe_forward_prepare allocates.  Any index
-outside its buffer fails the sweep.  The w2 + combine kernel of the same step is modelled the same way.
+For every workgroup of the w13 launch the model restates which (class, unit, block) it takes
+(gemv_resolve_route_n: routed workgroups first, then the publisher, then the shared expert's), the byte
+ranges of its buffer descriptors inside the expert image, every offset a lane sends through them, every
+offset into the wave-private LDS areas against the dynamic LDS size the launcher passes, the output elements
+against the extents of h_r / h_s, and what the publishing workgroup stores against the sizes
+moe_forward_prepare allocates.  For the w2 + combine launch it walks the load cursor of all 16 waves and
+checks that every (unit, pair of groups) is read exactly once, that every in-range offset of the four
+descriptors of a load lies inside the image / the h vector, and that items past a unit's last group fall
+outside the descriptor (they read zeros).  Any index outside its buffer fails the sweep.
 """
 import itertools
 
@@ -14,78 +19,89 @@ import pytest
 from promoe_amd import layout as LY
 
 
-def gemv_lds(tmax, K):
-    G = K // 128
-    return tmax * K * 2 + tmax * (K // 32) * 4 + 2 * G * 32 + 2 * G * 8 + 4 * tmax * 2 * 16 * 4
+def w13_wave_dw(ch):
+    return ch * 64 + ch * 4 + ch * 16 + ch * 4
+
+
+def w13_token_lds(ch):
+    return 4 * w13_wave_dw(ch) * 4 + 4 * 2 * 16 * 4
+
+
+def launcher_ch(H):
+    gpw = (H // 128 + 3) // 4
+    ch = (4 if gpw % 4 == 0 else (3 if gpw % 3 == 0 else 4)) if gpw >= 4 else gpw
+    return max(ch, 1)
 
 
 def model_route_launch(E, k, H, I, I_sh):
-    """Returns the number of workgroups checked; asserts on any out-of-range index."""
+    """k_w13_token<CH>.  Returns the number of working workgroups checked; asserts on any out-of-range index."""
     lay_r = LY.int4_layout(H, I)
     lay_s = LY.int4_layout(H, I_sh) if I_sh else None
     K, G = H, H // 128
     n_sh = I_sh // 16 if I_sh else 0
     nblk_r = I // 16
+    n_rt = k * nblk_r + 1
     grid = n_sh + k * nblk_r + 1
-    lds = gemv_lds(1, H)
+    CH = launcher_ch(H)
+    lds = w13_token_lds(CH)
     assert lds <= 64 * 1024
-    # LDS carve-up of the kernel (TMAX = 1)
-    o_xs, o_xsum = 0, K * 2
-    o_sc = o_xsum + (K // 32) * 4
-    o_zz = o_sc + 2 * G * 32
-    o_red = o_zz + 2 * G * 8
-    assert o_red + 4 * 1 * 2 * 16 * 4 <= lds
-    vec_per_row, n_sc, n_zz = K // 8, 2 * G * 32 // 4, 2 * G * 8 // 4
-    # staging stores, all 256 threads
-    for tid in range(256):
-        if tid < vec_per_row:
-            assert o_xs + (tid + 1) * 16 <= o_xsum
-            assert o_xsum + ((tid >> 2) + 1) * 4 <= o_sc
-        for v in range(tid + 256, vec_per_row, 256):
-            assert o_xs + (v + 1) * 16 <= o_xsum and o_xsum + ((v >> 2) + 1) * 4 <= o_sc
-        for i in [tid, tid + 256] + list(range(tid + 512, n_sc, 256)):
-            if i < n_sc:
-                assert o_sc + (i + 1) * 4 <= o_zz
-        for i in [tid] + list(range(tid + 256, n_zz, 256)):
-            if i < n_zz:
-                assert o_zz + (i + 1) * 4 <= o_red
-    # reads of the product loop: every wave w, group g = w + 4j < G, lane (r, qd)
+    WDW = w13_wave_dw(CH)
+    # a wave's LDS area in dwords: xs [CH][64], xsum [CH][4], wsc [2CH][8], wzz [2CH][2]; red behind the four areas
+    o_xsum, o_wsc, o_wzz = CH * 64, CH * 68, CH * 68 + CH * 16
+    assert o_wzz + CH * 4 == WDW and (4 * WDW + 4 * 2 * 16) * 4 == lds
+    for lane in range(64):
+        r, qd = lane & 15, lane >> 4
+        xj, scj, zzj = lane >> 4, lane >> 3, lane >> 1
+        if xj < CH:                                   # ((uint4 *)xs)[lane], xsum[lane >> 2]
+            assert (lane + 1) * 4 <= o_xsum and o_xsum + (lane >> 2) < o_wsc
+        if scj < 2 * CH:
+            assert o_wsc + lane < o_wzz               # wsc[lane]
+        if zzj < 2 * CH:
+            assert o_wzz + lane < WDW                 # wzz[lane]
+        for j in range(CH):                           # reads in front of the products
+            assert (max(j, CH + j) * 16 + r) * 2 + 2 <= (o_wzz - o_wsc) * 4     # wsc_h[(CH + j) * 16 + r]
+            assert (CH + j) * 8 + (r >> 1) < (WDW - o_wzz) * 4                  # wzz_b[(CH + j) * 8 + (r >> 1)]
+            assert (j * 128 + qd * 32 + 32) * 2 <= o_xsum * 4                   # 4 x uint4 at xs + j*128 + qd*32
+            assert j * 4 + qd < o_wsc - o_xsum                                  # xsum[j * 4 + qd]
+    assert (3 * 2 + 1) * 16 + 15 < 4 * 2 * 16                                   # red[(w * 2 + ab) * 16 + lane]
+    # offsets a wave sends through its descriptors (lengths: K * 2, 2 G KiB, 2 G * 32, 2 G * 8)
     for w in range(4):
-        for g in range(w, G, 4):
-            for qd in range(4):
-                assert (g * 128 + qd * 32 + 32) * 2 <= o_xsum - o_xs
-                assert (g * 4 + qd + 1) * 4 <= o_sc - o_xsum
-            for r in range(16):
-                assert ((G + g) * 16 + r + 1) * 2 <= o_zz - o_sc
-                assert (G + g) * 8 + (r >> 1) + 1 <= o_red - o_zz
-    # reduction buffer: red[((w*TMAX + t)*2 + ab)*16 + lane], lane < 16
-    assert ((3 * 1 + 0) * 2 + 1) * 16 + 15 < 4 * 1 * 2 * 16
-
+        GPW = (G - w + 3) >> 2
+        assert GPW <= (G + 3) // 4
+        for jc in range(0, GPW, CH):
+            for j in range(CH):
+                g = w + 4 * (jc + j) if jc + j < GPW else 0
+                assert 0 <= g < G
+                assert g * 256 + 15 * 16 + 16 <= K * 2
+                for half in (0, G):
+                    assert ((half + g) * 8 + 7) * 4 + 4 <= 2 * G * 32
+                    assert ((half + g) * 2 + 1) * 4 + 4 <= 2 * G * 8
+                    assert 63 * 16 + (half + g) * 1024 + 16 <= 2 * G * 1024
     n_checked = 0
+    n_pub = 0
     for bx in range(grid):
-        sh = bx < n_sh
-        rr = bx if sh else bx - n_sh
+        sh = bx >= n_rt
+        rr = bx - n_rt if sh else bx
         nblk = (I_sh // 16) if sh else nblk_r
         publisher = (not sh) and rr == k * nblk
         u = 0 if (sh or publisher) else rr // nblk
         b = rr - u * nblk
         if publisher:
+            n_pub += 1
             continue            # m = 0: returns before any weight or LDS access
         lay = lay_s if sh else lay_r
         rows_out, out_stride = (1, I_sh) if sh else (k, I)
-        assert 0 <= u < (1 if sh else k) and 0 <= b < nblk
+        assert 0 <= u < (1 if sh else k) and 0 <= b < nblk, (bx, u, b)
         rbA = 2 * b
-        # the three buffer resources: base + section offset + rbA * G * bytes-per-tile, two blocks long
+        # the three descriptors over the image: section offset + rbA * G * bytes-per-tile, two blocks long
         for off, nxt, per_tile in (("off13_q", "off13_s", 1024), ("off13_s", "off13_z", 32), ("off13_z", "off2_q", 8)):
             lo = lay[off] + rbA * G * per_tile
             assert lay[off] <= lo and lo + 2 * G * per_tile <= lay[nxt], (bx, off)
-        # weight tiles: lane * 16 + g * 1024 and (G + g) * 1024 inside the 2 G KiB range
-        assert 63 * 16 + 16 + (G + G - 1) * 1024 <= 2 * G * 1024
-        # output: h[(row0 + t) * out_stride + b * 16 + r], row0 = u (routed) or 0 (shared), t = 0
+        # output: h[row0 * out_stride + b * 16 + tid], tid < 16; row0 = u (routed) or 0 (shared)
         row0 = 0 if sh else u
         assert row0 * out_stride + b * 16 + 15 < rows_out * out_stride, (bx, row0, b)
         n_checked += 1
-    assert n_checked == grid - 1
+    assert n_checked == grid - 1 and n_pub == 1
     # what the publisher stores, against moe_forward_prepare's allocations for max_tokens >= 1
     P = k                                   # T = 1
     max_units = min(E, P)
@@ -97,44 +113,102 @@ def model_route_launch(E, k, H, I, I_sh):
     return n_checked
 
 
-def model_w2_combine_launch(k, H, I, I_sh, NI=2):
-    """k_w2_combine_token<NI>: grid H / (16 / NI), LDS = staged h vectors + 32-wide sums + reduction."""
+W2C_WAVES = 16
+
+
+def launcher_w2c(k, H, I, I_sh):
+    G, G_sh = I // 128, (I_sh // 128 if I_sh else 0)
+    loads_per_wave = (k * ((G + 1) // 2) + (G_sh + 1) // 2 + W2C_WAVES - 1) // W2C_WAVES
+    if loads_per_wave <= 3:
+        return 2, 3
+    if H // 16 >= 256:
+        return 1, 7
+    return 2, 6
+
+
+def model_w2_combine_launch(k, H, I, I_sh, NI=2, CHUNK=3):
+    """k_w2_combine_token<NI, CHUNK>: grid H / (16 / NI); LDS = per wave the activations and 32-wide sums of a
+    chunk's items, then the waves' partial sums."""
     RW = 16 // NI
     G, G_sh = I // 128, (I_sh // 128 if I_sh else 0)
     lay_r = LY.int4_layout(H, I)
     lay_s = LY.int4_layout(H, I_sh) if I_sh else None
-    n_h = k * I + I_sh
-    lds = n_h * 2 + (n_h // 32) * 4 + 16 * 16 * 4
-    assert lds <= 150 * 1024
-    o_xsum = n_h * 2
-    o_red = o_xsum + (n_h // 32) * 4
-    assert o_red + 16 * RW * 4 <= lds
-    nvec = n_h // 8
-    for v in range(nvec):                     # staging: vector v of the concatenated h vectors
-        el = v * 8
-        assert (el + 8 <= k * I) or (el >= k * I and el - k * I + 8 <= I_sh), v   # never straddles h_r | h_s
-        assert (v + 1) * 16 <= o_xsum and ((v >> 2) + 1) * 4 <= o_red - o_xsum
+    WAVE_DW = CHUNK * NI * 64 + CHUNK * NI * 4
+    lds = W2C_WAVES * (CHUNK * NI * 68) * 4 + W2C_WAVES * 16 * 4
+    assert lds <= 150 * 1024 and k < 64 and H % 16 == 0
+    assert (W2C_WAVES * WAVE_DW + W2C_WAVES * RW) * 4 <= lds        # red[w * RW + lane], lane < RW
+    GP, GP_sh = (G + NI - 1) // NI, (G_sh + NI - 1) // NI
+    # ---- the load cursor of every wave: which (unit, load) it requests, chunk by chunk ----
+    seen = {}
+    max_gp = 0
+    for w in range(W2C_WAVES):
+        u, gp = 0, w
+        while u < k and gp >= GP:
+            gp -= GP; u += 1
+        trips = 0
+        while u < k or gp < GP_sh:
+            trips += 1
+            assert trips <= 4096
+            for c in range(CHUNK):
+                valid = u < k or gp < GP_sh
+                assert 0 <= u <= k            # readlane(ub, u): lane k holds the shared expert, k < 64
+                if valid:
+                    shd = u >= k
+                    assert gp < (GP_sh if shd else GP)
+                    key = (u, gp)
+                    assert key not in seen, key
+                    seen[key] = w
+                    max_gp = max(max_gp, gp)
+                    gp += W2C_WAVES
+                    while u < k and gp >= GP:
+                        gp -= GP; u += 1
+                else:
+                    assert u == k and gp < GP_sh + W2C_WAVES   # an absent load: descriptors of length 0
+    want = {(u, gp) for u in range(k) for gp in range(GP)} | {(k, gp) for gp in range(GP_sh)}
+    assert set(seen) == want
+    # ---- per-lane offsets of one load against its four descriptors ----
     grid = H // RW
+    for shd, Gu, lay, GPu in ((False, G, lay_r, GP), (True, G_sh, lay_s, GP_sh)):
+        if Gu == 0:
+            continue
+        # the image holds H / 16 row blocks of Gu tiles each; a descriptor covers block b16's Gu tiles
+        assert lay["off2_q"] + (H // 16) * Gu * 1024 <= lay["off2_s"]
+        assert lay["off2_s"] + (H // 16) * Gu * 32 <= lay["off2_z"]
+        assert lay["off2_z"] + (H // 16) * Gu * 8 <= lay["total_bytes"]
+        for gp in range(GPu):
+            g0 = NI * gp
+            for part in range(NI):
+                for lane in range(64):
+                    r, qd = lane & 15, lane >> 4
+                    mine, rr = r // RW, RW * part + (r % RW)
+                    assert mine < NI and rr < 16
+                    item_exists = g0 + mine < Gu
+                    vq = mine * 1024 + (qd * 16 + rr) * 16 + g0 * 1024
+                    vs = mine * 32 + 2 * rr + g0 * 32
+                    vz = mine * 8 + (rr >> 1) + g0 * 8
+                    # inside the descriptor exactly when the item exists (otherwise the load returns 0)
+                    assert (vq + 16 <= Gu * 1024) == item_exists, (gp, lane)
+                    assert (vs + 2 <= Gu * 32) == item_exists
+                    assert (vz + 1 <= Gu * 8) == item_exists
+                    lj, lpart = lane >> 4, lane & 15
+                    if lj < NI:
+                        vh = lj * 256 + lpart * 16 + g0 * 256
+                        assert (vh + 16 <= Gu * 256) == (g0 + lj < Gu)
+                        # wave-private LDS: ((uint4 *)hs)[(c * NI + lj) * 16 + lpart], xsum[(c * NI + lj) * 4 + (lpart >> 2)]
+                        c = CHUNK - 1
+                        assert ((c * NI + lj) * 16 + lpart + 1) * 4 <= CHUNK * NI * 64
+                        assert CHUNK * NI * 64 + (c * NI + lj) * 4 + (lpart >> 2) < WAVE_DW
+                    c = CHUNK - 1
+                    assert ((c * NI + mine) * 128 + qd * 32 + 32) * 2 <= CHUNK * NI * 64 * 4
+                    assert (c * NI + mine) * 4 + qd < CHUNK * NI * 4
+    # the h vectors behind the rh descriptors: unit u's I values inside h_r [k, I], the shared expert's inside h_s
+    for u in range(k):
+        assert u * I + G * 128 <= k * I
+    assert G_sh * 128 <= max(I_sh, 0)
+    # output rows
     for bx in range(grid):
         b16, part = bx // NI, bx % NI
-        for r in range(16):
-            rr = RW * part + (r % RW)
-            assert rr < 16
-            # items: (unit u < k, group g < G) and (shared, g < G_sh)
-            for shd, Gu, lay in ((False, G, lay_r), (True, G_sh, lay_s)):
-                if Gu == 0:
-                    continue
-                for lg in (0, Gu - 1):
-                    t_idx = b16 * Gu + lg
-                    for qd in range(4):
-                        assert lay["off2_q"] + t_idx * 1024 + (qd * 16 + rr) * 16 + 16 <= lay["off2_s"]
-                    assert lay["off2_s"] + t_idx * 32 + 2 * rr + 2 <= lay["off2_z"]
-                    assert lay["off2_z"] + t_idx * 8 + (rr >> 1) + 1 <= lay["total_bytes"]
-                    for u in ((k,) if shd else (0, k - 1)):
-                        ho = (k * I if shd else u * I) + lg * 128
-                        assert (ho + 3 * 32 + 32) <= n_h and ((ho + 96) >> 5) < n_h // 32
-        # output rows of this workgroup
-        assert b16 * 16 + RW * part + RW - 1 < H
+        assert b16 < H // 16 and b16 * 16 + RW * part + RW - 1 < H
     return grid
 
 
@@ -157,16 +231,17 @@ SHAPES = [
 def test_one_token_launch_stays_inside_its_buffers(E, k, H, I, I_sh):
     n = model_route_launch(E, k, H, I, I_sh)
     assert n == (I_sh // 16 if I_sh else 0) + k * (I // 16)
-    n_h = k * I + I_sh
-    if n_h * 2 + (n_h // 32) * 4 + 1024 <= 150 * 1024:   # the rule of moe_forward for the fused w2 + combine pass
-        for NI in (1, 2, 4):
-            model_w2_combine_launch(k, H, I, I_sh, NI)
+    if k < 64 and H % 16 == 0:                       # the rule of moe_forward for the fused w2 + combine pass
+        ni, chunk = launcher_w2c(k, H, I, I_sh)
+        model_w2_combine_launch(k, H, I, I_sh, ni, chunk)
+        for ni, chunk in ((2, 3), (1, 7), (2, 6)):   # every instantiation, whatever the launcher would pick
+            model_w2_combine_launch(k, H, I, I_sh, ni, chunk)
 
 
 def test_sweep_of_small_shapes():
     n = 0
     for H, I, I_sh, (E, k) in itertools.product((128, 256, 640), (128, 384), (0, 128, 512), ((1, 1), (5, 2), (64, 6), (130, 7))):
         model_route_launch(E, k, H, I, I_sh)
-        model_w2_combine_launch(k, H, I, I_sh, 2)
+        model_w2_combine_launch(k, H, I, I_sh, *launcher_w2c(k, H, I, I_sh))
         n += 1
     assert n == 72
