@@ -130,7 +130,10 @@ int moe_release_experts(moe_engine *eng, int layer, const int64_t *ids, int64_t 
 /* ---- prefetch request hook: PrefetchLayerTask (prefetcher.hpp:52-58, worker.cpp:41-68) ---- */
 /* Queue speculative copies of `ids` (ranked) for a future layer.  Takes one unit of
  * the run-ahead budget (initially max_prefetch_layer_distance, returned by
- * report_one_layer / layer_done); blocking=0 returns 1 when no budget is left. */
+ * report_one_layer / layer_done); blocking=0 returns 1 when no budget is left.
+ * With chunk_prefetch an expert is queued as one task per registered parameter (a demand
+ * fetch can overtake between tasks), except that a parameter of at most an eighth of its
+ * predecessor's bytes shares the predecessor's task. */
 int moe_prefetch_layer(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking);
 /* When 1, report_one_layer first waits until a prefetch request (possibly empty) for
  * that layer was issued (PredictWorker::consume_prefetch_layer_progress, worker.hpp:312-314). */
