@@ -480,10 +480,11 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     s->sub_cursor = 0;
     for (int64_t id : later) {
       if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
-      if ((rc = moe_flush_table(eng, layer, st))) return rc;
       moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
       *slot_h = unit_of[(int)id];
-      // (an int4 decode launch of one unit takes it in the kernel arguments: no device copy of the unit)
+      // (an int4 decode launch of one unit takes the unit and its slot address in the kernel arguments: no device
+      // copy of the unit, and the device table is not read, so its flush, a copy in the stream in front of the
+      // launch, waits for the layer's next turn)
       if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
       s->sub_cursor++;
       if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
@@ -649,7 +650,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // missed experts in the returned order, one at a time as their copies land
   for (int64_t id : later) {
     if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
-    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    if (!by_value && (rc = moe_flush_table(eng, layer, st))) return rc;  // (by value: the device table is not read)
     moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
     *slot_h = unit_of[(int)id];
     if (!by_value) HIPC(hipMemcpyAsync(s->units_sub + s->sub_cursor, slot_h, sizeof(moe_unit), hipMemcpyHostToDevice, st));
