@@ -368,10 +368,13 @@ static int cache_miss(moe_engine *eng, Expert *in, bool precise, Expert **victim
 // ---------------------------------------------------------------------------
 static inline bool in_cache(moe_engine *eng, Expert *e) { return eng->resident.count(e) != 0; }
 
+// bumped with every queued task (under the engine lock): what an idle fetch thread polls before it sleeps
+static std::atomic<unsigned> g_task_epoch{0};
 static void add_task(std::deque<CopyTask> &q, Expert *e, int start, int stop, bool precise) {
   CopyTask t;
   t.e = e; t.start = start; t.stop = stop; t.precise = precise;
   q.push_back(t);
+  g_task_epoch.fetch_add(1, std::memory_order_release);
 }
 
 // `ready -> launching` of a demand hit (prefetcher.cpp:51,105).  `using` is resolved
@@ -546,7 +549,23 @@ static void fetch_thread_main(moe_engine *eng) {
   while (!eng->exiting) {
     CopyTask t;
     if (!eng->fatal.empty() || !pop_next_task(eng, t)) {
-      eng->cv_work.wait(lk);
+      // A decode loop brings the next task within tens of microseconds, and waking this thread up from the
+      // condition variable would cost that task 10-50 us before its copy starts: poll the task counter for a
+      // while without the lock first (tasks are queued under the lock, so none can slip in between the last
+      // look at the counter below and the wait).
+      const unsigned ep = g_task_epoch.load(std::memory_order_acquire);
+      if (eng->fatal.empty()) {
+        lk.unlock();
+        const auto t0 = std::chrono::steady_clock::now();
+        for (unsigned spins = 0; g_task_epoch.load(std::memory_order_acquire) == ep; ++spins) {
+#if defined(__x86_64__)
+          __builtin_ia32_pause();
+#endif
+          if ((spins & 63u) == 63u && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(500)) break;
+        }
+        lk.lock();
+      }
+      if (g_task_epoch.load(std::memory_order_acquire) == ep && !eng->exiting) eng->cv_work.wait(lk);
       continue;
     }
     bool sent = false;
