@@ -578,7 +578,23 @@ static void fetch_thread_main(moe_engine *eng) {
     const int start = eng->current.start, stop = eng->current.stop;
     // a kernel may be reading any slot of this group through a table snapshot: the slot stays as it is
     // until the caller has seen that kernel's selection and protected what it uses
-    while (eng->group_of(e->layer).guard > 0 && !eng->exiting) eng->cv_state.wait_for(lk, std::chrono::microseconds(50));
+    // (a guard stands for the few microseconds between a one-token launch and the hooks of its layer: look again
+    // every microsecond or so, without the lock in between, before falling back to timed waits; the release
+    // notifies, but waking up from it would cost the demand copy of that very layer 10-50 us)
+    {
+      const auto g0 = std::chrono::steady_clock::now();
+      while (eng->group_of(e->layer).guard > 0 && !eng->exiting) {
+        if (std::chrono::steady_clock::now() - g0 < std::chrono::microseconds(300)) {
+          lk.unlock();
+#if defined(__x86_64__)
+          for (int i = 0; i < 32; ++i) __builtin_ia32_pause();
+#endif
+          lk.lock();
+        } else {
+          eng->cv_state.wait_for(lk, std::chrono::microseconds(50));
+        }
+      }
+    }
     if (Expert *v = eng->current.wait_victim) {
       resolve_using(eng, v, lk);
       if (v->slot == e->slot && !in_cache(eng, v)) { set_table(eng, v, false); v->slot = -1; }
