@@ -203,6 +203,27 @@ int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k,
                           void *y_bf16, void *stream);
 
 
+/* k1a + k1b + k2 + k3 for ONE token: moe_decode_token_int4 whose launch of phase bit 0 also computes the gate
+ * logits, so a decode step is two launches (this one, then w2 + combine) instead of three.  The first
+ * ceil(n_gate_rows / 4) workgroups sum the gate rows (a wave per row, the summation order of moe_gate_logits:
+ * the same bits) and hand every logit to the routing waves of the same launch through gate_ws as a (value,
+ * gate_seq) word; the routing waves poll until every word carries gate_seq (bounded: on a time-out *err |= 1).
+ *   gate_w [n_gate_rows, H] bf16, n_gate_rows = E, or E + 1 with the shared expert's gate vector as row E;
+ *   gate_bias [E] or NULL (the routed rows only); logits [n_gate_rows] fp32 is an OUTPUT here.
+ *   gate_ws: moe_gate_ws_bytes() of device memory, zeroed once by the caller; gate_seq: a nonzero number that no
+ *   earlier call with the same gate_ws used (count upwards), so nothing has to be cleared between calls.
+ * Because gate_seq is a launch argument, a HIP graph that records this call replays one number: inside a graph
+ * use moe_gate_logits + moe_decode_token_int4.  No counterpart in the reference (its gate is torch's). */
+int64_t moe_gate_ws_bytes(void);
+int moe_decode_token_int4_gate(const void *x_bf16, const void *gate_w, const float *gate_bias, int n_gate_rows,
+                               void *gate_ws, int gate_seq, float *logits, int E, int k, int mode, int H, int I,
+                               int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx, float *w,
+                               int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
+                               moe_unit *units, int *n_active, int64_t *active_ids, void *h_r, void *h_s,
+                               float *part_r, float *part_s, int *err, void *unit_ws, moe_unit *units_host_out,
+                               int *seq_host_out, int seq_value, int phases, const float *shared_gate_logit,
+                               void *y_bf16, void *stream);
+
 /* moe_decode_token_int4 with phases = 5 (routing + w13 + SwiGLU, then w2 + combine into y_bf16 [H]) that
  * allocates nothing and takes no workspace: the routing arrays, the h vectors and the resolved units live in
  * a device array of moe_noalloc_scratch_bytes() (under 160 KiB) that is part of the library image; each GPU

@@ -368,13 +368,13 @@ static int cache_miss(moe_engine *eng, Expert *in, bool precise, Expert **victim
 // ---------------------------------------------------------------------------
 static inline bool in_cache(moe_engine *eng, Expert *e) { return eng->resident.count(e) != 0; }
 
-// bumped with every queued task (under the engine lock): what an idle fetch thread polls before it sleeps
-static std::atomic<unsigned> g_task_epoch{0};
-static void add_task(std::deque<CopyTask> &q, Expert *e, int start, int stop, bool precise) {
+// every queued task bumps the engine's task counter (under the engine lock): what that engine's idle fetch thread
+// polls before it sleeps
+static void add_task(moe_engine *eng, std::deque<CopyTask> &q, Expert *e, int start, int stop, bool precise) {
   CopyTask t;
   t.e = e; t.start = start; t.stop = stop; t.precise = precise;
   q.push_back(t);
-  g_task_epoch.fetch_add(1, std::memory_order_release);
+  eng->task_epoch.fetch_add(1, std::memory_order_release);
 }
 
 // `ready -> launching` of a demand hit (prefetcher.cpp:51,105).  `using` is resolved
@@ -414,16 +414,16 @@ static int preempt_resident(moe_engine *eng, Expert *e) {
   if (e == eng->current.e) {
     eng->current.precise = true;
     if (eng->current.stop == P) return cache_hit(eng, e, true);
-    add_task(eng->precise_q, e, eng->current.stop, P, true);
+    add_task(eng, eng->precise_q, e, eng->current.stop, P, true);
     return 0;
   }
-  add_task(eng->precise_q, e, e->num_ready, P, true);
+  add_task(eng, eng->precise_q, e, e->num_ready, P, true);
   return 0;
 }
 
 static int preempt_one_expert(moe_engine *eng, int layer, int64_t id) {
   Expert *e = eng->ex(layer, (int)id);
-  if (!in_cache(eng, e)) { add_task(eng->precise_q, e, 0, eng->cfg.num_per_expert_param, true); return 0; }
+  if (!in_cache(eng, e)) { add_task(eng, eng->precise_q, e, 0, eng->cfg.num_per_expert_param, true); return 0; }
   return preempt_resident(eng, e);
 }
 
@@ -435,11 +435,11 @@ static int preempt_one_layer(moe_engine *eng, int layer, const int64_t *ids, int
     Expert *e = eng->ex(layer, (int)ids[i]);
     if (!in_cache(eng, e)) {
       preceding_in_cache = false;
-      add_task(eng->precise_q, e, 0, P, true);
+      add_task(eng, eng->precise_q, e, 0, P, true);
       continue;
     }
     if (!preceding_in_cache) {  // may be evicted by a preceding miss: redundant demand task
-      add_task(eng->precise_q, e, 0, P, true);
+      add_task(eng, eng->precise_q, e, 0, P, true);
       continue;
     }
     if (int rc = preempt_resident(eng, e)) return rc;
@@ -553,11 +553,11 @@ static void fetch_thread_main(moe_engine *eng) {
       // condition variable would cost that task 10-50 us before its copy starts: poll the task counter for a
       // while without the lock first (tasks are queued under the lock, so none can slip in between the last
       // look at the counter below and the wait).
-      const unsigned ep = g_task_epoch.load(std::memory_order_acquire);
+      const unsigned ep = eng->task_epoch.load(std::memory_order_acquire);
       if (eng->fatal.empty()) {
         lk.unlock();
         const auto t0 = std::chrono::steady_clock::now();
-        for (unsigned spins = 0; g_task_epoch.load(std::memory_order_acquire) == ep; ++spins) {
+        for (unsigned spins = 0; eng->task_epoch.load(std::memory_order_acquire) == ep; ++spins) {
 #if defined(__x86_64__)
           __builtin_ia32_pause();
 #endif
@@ -565,7 +565,7 @@ static void fetch_thread_main(moe_engine *eng) {
         }
         lk.lock();
       }
-      if (g_task_epoch.load(std::memory_order_acquire) == ep && !eng->exiting) eng->cv_work.wait(lk);
+      if (eng->task_epoch.load(std::memory_order_acquire) == ep && !eng->exiting) eng->cv_work.wait(lk);
       continue;
     }
     bool sent = false;
@@ -1141,11 +1141,11 @@ int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int6
       for (int j = 0; j < P;) {
         int j2 = j + 1;
         while (j2 < P && e->chunks[j2].nbytes * 8 <= e->chunks[j].nbytes) ++j2;
-        add_task(eng->layer_q[layer], e, j, j2, false);
+        add_task(eng, eng->layer_q[layer], e, j, j2, false);
         j = j2;
       }
     }
-    else add_task(eng->layer_q[layer], e, 0, P, false);
+    else add_task(eng, eng->layer_q[layer], e, 0, P, false);
   }
   eng->progress++;
   eng->cv_sem.notify_all();

@@ -21,6 +21,10 @@ struct LayerState {
       *sorted_tok = nullptr, *n_active = nullptr;
   unsigned *route_counter = nullptr;
   unsigned char *unit_ws = nullptr;  // resolved units of the one-token path (16 bytes each)
+  // one-token launches that compute their gate logits themselves: hand-over words (zeroed once) and the number
+  // of the last such launch (every launch takes the next one, so no word of an earlier launch passes for a new one)
+  unsigned char *gate_ws = nullptr;
+  int gate_seq = 0;
   moe_unit *units = nullptr, *units_sub = nullptr;
   int64_t *active_ids = nullptr;
   void *h_r = nullptr, *h_s = nullptr, *tiles_ws = nullptr;
@@ -155,6 +159,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->n_active, 1);
   rc |= dalloc(s, &s->route_counter, 1);
   rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
+  rc |= dalloc(s, &s->gate_ws, (size_t)moe_gate_ws_bytes());
   rc |= dalloc(s, &s->units, s->max_units);
   rc |= dalloc(s, &s->units_sub, (size_t)s->max_units * 2);
   rc |= dalloc(s, &s->active_ids, s->max_units);
@@ -193,6 +198,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   memset(s->err_spec, 0, sizeof(int) * eng->cfg.num_layer);
   s->spec_state.assign(eng->cfg.num_layer, 0);
   HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
+  HIPC(hipMemset(s->gate_ws, 0, (size_t)moe_gate_ws_bytes()));
   if (s->disp_ws) HIPC(hipMemset(s->disp_ws, 0, 64));
   *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
@@ -327,15 +333,8 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
                    eng->layer_complete[layer] == E && !eng->predictor_attached;
   }
   if (all_resident && T == 1 && d.fmt == MOE_FMT_INT4_G128 && E <= 256 && k <= 32 && (size_t)d.H * 2 + 8192 <= 60 * 1024) {
-    // one token: gate logits, then the w13 kernel routes by itself (no top-k / dispatch launches)
-    if (!d.gate_bias) {
-      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
-    } else {
-      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
-      if (d.shared_gated &&
-          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
-        return rc;
-    }
+    // one token: the w13 launch computes the gate logits in its first workgroups and routes by itself (no gate,
+    // top-k or dispatch launches): two launches per step
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
@@ -346,11 +345,13 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const int seq = ++s->seq_counter;
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     const bool w2c = w2c_fits(d, k);  // w2 and the combine in one launch
-    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
-                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
-                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws, p.units, p.seq, seq,
-                                    w2c ? 5 : 3, sg0, y, st)))
+    s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
+    if ((rc = moe_decode_token_int4_gate(x, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, E, k,
+                                         d.route_mode, d.H, d.I, d.I_sh, table,
+                                         d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                         s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                         s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws, p.units, p.seq, seq,
+                                         w2c ? 5 : 3, sg0, y, st)))
       return rc;
     *p.n_active = k;
     p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
@@ -380,14 +381,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       if (d.gate_bias && d.shared_gated &&
           (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
         return rc;
-    } else if (!d.gate_bias) {
-      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
-    } else {
-      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
-      if (d.shared_gated &&
-          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
-        return rc;
-    }
+    }  // (without the predictor's rows the w13 launch below computes the gate logits itself)
     const uint64_t *table = nullptr;
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     // what the kernel will find resident: exactly these experts get computed by it
@@ -399,12 +393,22 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       ~GuardRelease() { release(); }
     } guard{eng, layer, true};
     const int seq = ++s->seq_counter;
-    if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
-                                    d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
-                                    s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                    s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
-                                    nullptr, nullptr, st)))
-      return rc;
+    if (pred_fused) {
+      rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                 d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                 s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                 s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
+                                 nullptr, nullptr, st);
+    } else {
+      s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
+      rc = moe_decode_token_int4_gate(x, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, E, k,
+                                      d.route_mode, d.H, d.I, d.I_sh, table,
+                                      d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                      s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                      s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
+                                      nullptr, nullptr, st);
+    }
+    if (rc) return rc;
     // the predictor's scores came out of the gate launch above: complete once this kernel's sequence word arrives
     if (pred_fused && (rc = moe_predictor_scores_pending(eng, layer, s->opt_seq, seq))) return rc;
     // The w2 pass with the combine goes out at once as well, as if nothing were missing: in most steps nothing

@@ -199,6 +199,7 @@ struct moe_engine {
   std::deque<CopyTask> precise_q;
   std::vector<std::deque<CopyTask>> layer_q;
   CopyTask current;  // the one copy in flight (current.e == nullptr: none)
+  std::atomic<unsigned> task_epoch{0};  // bumped with every queued task
   std::thread fetch_thread;
   bool launched = false, exiting = false, slots_ready = false;
   std::string fatal;  // first broken invariant (the reference would have aborted)

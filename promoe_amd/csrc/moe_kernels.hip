@@ -11,6 +11,74 @@
 #include "moe_common.h"
 #include "moe_device.h"
 
+// The sum of one (token, gate row) pair by one wave, in a fixed order (bit-reproducible): lane partials over
+// k = 512 c + 8 lane + j with one fma chain, then the xor butterfly 32..1.  Every lane returns the sum.
+// All loads of the row go out back to back, without a condition around any of them (a lane past the end of the row
+// reads column 0 and drops the result): with a condition per 512-column chunk the compiler put a full wait for
+// memory between the chunks, and a 2048-wide row took four round trips to memory instead of one.
+template <int NCH>
+static __device__ __forceinline__ float gate_row_partial(const uint16_t *__restrict__ xr, const uint16_t *__restrict__ wr,
+                                                         const int H, const int lane) {
+  uint4 xq[NCH], wq[NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int k = c * 512 + 8 * lane;
+    const int kk = k < H ? k : 0;
+    xq[c] = *(const uint4 *)(xr + kk);
+    wq[c] = *(const uint4 *)(wr + kk);
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    float t = acc;
+    t = fmaf(bf16lo(xq[c].x), bf16lo(wq[c].x), t);
+    t = fmaf(bf16hi(xq[c].x), bf16hi(wq[c].x), t);
+    t = fmaf(bf16lo(xq[c].y), bf16lo(wq[c].y), t);
+    t = fmaf(bf16hi(xq[c].y), bf16hi(wq[c].y), t);
+    t = fmaf(bf16lo(xq[c].z), bf16lo(wq[c].z), t);
+    t = fmaf(bf16hi(xq[c].z), bf16hi(wq[c].z), t);
+    t = fmaf(bf16lo(xq[c].w), bf16lo(wq[c].w), t);
+    t = fmaf(bf16hi(xq[c].w), bf16hi(wq[c].w), t);
+    acc = (c * 512 + 8 * lane < H) ? t : acc;
+  }
+  return acc;
+}
+
+static __device__ __forceinline__ float gate_row_sum(const uint16_t *__restrict__ xr, const uint16_t *__restrict__ wr,
+                                                     const int H, const int lane) {
+  float acc = 0.f;
+  const int nch = (H + 511) >> 9;  // wave-uniform
+  switch (nch) {
+    case 1: acc = gate_row_partial<1>(xr, wr, H, lane); break;
+    case 2: acc = gate_row_partial<2>(xr, wr, H, lane); break;
+    case 3: acc = gate_row_partial<3>(xr, wr, H, lane); break;
+    case 4: acc = gate_row_partial<4>(xr, wr, H, lane); break;
+    case 5: acc = gate_row_partial<5>(xr, wr, H, lane); break;
+    case 6: acc = gate_row_partial<6>(xr, wr, H, lane); break;
+    case 7: acc = gate_row_partial<7>(xr, wr, H, lane); break;
+    case 8: acc = gate_row_partial<8>(xr, wr, H, lane); break;
+    default:
+      for (int c = 0; c < H; c += 512) {
+        const int k = c + 8 * lane;
+        if (k < H) {
+          const uint4 xv = *(const uint4 *)(xr + k);
+          const uint4 wv = *(const uint4 *)(wr + k);
+          acc = fmaf(bf16lo(xv.x), bf16lo(wv.x), acc);
+          acc = fmaf(bf16hi(xv.x), bf16hi(wv.x), acc);
+          acc = fmaf(bf16lo(xv.y), bf16lo(wv.y), acc);
+          acc = fmaf(bf16hi(xv.y), bf16hi(wv.y), acc);
+          acc = fmaf(bf16lo(xv.z), bf16lo(wv.z), acc);
+          acc = fmaf(bf16hi(xv.z), bf16hi(wv.z), acc);
+          acc = fmaf(bf16lo(xv.w), bf16lo(wv.w), acc);
+          acc = fmaf(bf16hi(xv.w), bf16hi(wv.w), acc);
+        }
+      }
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
+  return acc;
+}
+
 // ---------------------------------------------------------------------------
 // k1a gate logits: one wave per (token, expert row)
 // ---------------------------------------------------------------------------
@@ -32,53 +100,11 @@ __global__ __launch_bounds__(256) void k_gate_logits(const uint16_t *__restrict_
     wg = wg2; bias = bias2; logits = logits2; E = E2; ldl = ldl2;
   }
   if (e >= E) return;
-  const uint16_t *xr = x + (size_t)t * H;
-  const uint16_t *wr = wg + (size_t)e * H;
-  float acc = 0.f;
-  if (H <= 4096) {
-    // all loads of the row first (one round trip), then the same fma chain in the same order
-    uint4 xq[8], wq[8];
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int k = c * 512 + 8 * lane;
-      if (k < H) {
-        xq[c] = *(const uint4 *)(xr + k);
-        wq[c] = *(const uint4 *)(wr + k);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      const int k = c * 512 + 8 * lane;
-      if (k < H) {
-        acc = fmaf(bf16lo(xq[c].x), bf16lo(wq[c].x), acc);
-        acc = fmaf(bf16hi(xq[c].x), bf16hi(wq[c].x), acc);
-        acc = fmaf(bf16lo(xq[c].y), bf16lo(wq[c].y), acc);
-        acc = fmaf(bf16hi(xq[c].y), bf16hi(wq[c].y), acc);
-        acc = fmaf(bf16lo(xq[c].z), bf16lo(wq[c].z), acc);
-        acc = fmaf(bf16hi(xq[c].z), bf16hi(wq[c].z), acc);
-        acc = fmaf(bf16lo(xq[c].w), bf16lo(wq[c].w), acc);
-        acc = fmaf(bf16hi(xq[c].w), bf16hi(wq[c].w), acc);
-      }
-    }
-  } else
-  for (int c = 0; c < H; c += 512) {
-    const int k = c + 8 * lane;
-    if (k < H) {
-      const uint4 xv = *(const uint4 *)(xr + k);
-      const uint4 wv = *(const uint4 *)(wr + k);
-      acc = fmaf(bf16lo(xv.x), bf16lo(wv.x), acc);
-      acc = fmaf(bf16hi(xv.x), bf16hi(wv.x), acc);
-      acc = fmaf(bf16lo(xv.y), bf16lo(wv.y), acc);
-      acc = fmaf(bf16hi(xv.y), bf16hi(wv.y), acc);
-      acc = fmaf(bf16lo(xv.z), bf16lo(wv.z), acc);
-      acc = fmaf(bf16hi(xv.z), bf16hi(wv.z), acc);
-      acc = fmaf(bf16lo(xv.w), bf16lo(wv.w), acc);
-      acc = fmaf(bf16hi(xv.w), bf16hi(wv.w), acc);
-    }
-  }
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
-  if (lane == 0) logits[(size_t)t * ldl + e] = bias ? acc + bias[e] : acc;
+  // (requested in front of the row: behind the sum it is one more trip to memory)
+  const float bias_e = bias ? bias[e] : 0.f;
+  asm volatile("" :: "v"(bias_e));
+  const float acc = gate_row_sum(x + (size_t)t * H, wg + (size_t)e * H, H, lane);
+  if (lane == 0) logits[(size_t)t * ldl + e] = bias ? acc + bias_e : acc;
 }
 
 // Large T: a workgroup takes 16 tokens (8 waves x 2) and a group of gate rows.  The rows are staged in LDS once
@@ -713,7 +739,70 @@ struct GemvArgs {
   KUnit *r_kunits;              // routing publisher: resolved units (slot address, rows) for the w2 pass
   float *r_unit_w;              // and the routing weight per unit position
   const KUnit *kunits_dev;      // device-side resolved units: one load instead of unit -> table -> address
+  // one-token launches that also compute the gate logits: the first g_nblk workgroups sum the g_rows gate rows
+  // (a wave per row, once per part of the chip) and hand each logit to the routing waves of the same launch as a
+  // (value, g_seq) pair; g_nblk = 0: the logits come from an earlier launch (r_logits)
+  const uint16_t *g_w; const float *g_bias; unsigned long long *g_stamp; float *g_logits_out;
+  int g_rows, g_nbias, g_nblk, g_seq;
 };
+
+// Gate logits handed over inside a launch.  A logit travels as one 8-byte word (value, sequence number of the
+// launch), so a reader needs no flag and no fence: it polls the words until all of them carry its launch's number.
+// The numbers of successive launches on one workspace differ, so a word left by an earlier launch is never taken
+// for a new one and nothing has to be cleared.
+// The chip has eight parts (XCDs), each with its own second-level cache, which is the point of coherence for the
+// compute units of that part only.  A word written at device scope (past those caches) took 1.5 to 2.5 us to
+// become visible while the launch's weight streams were running, against 0.3 us through the second-level cache
+// of one part.  So the gate rows are summed once PER PART (the gate workgroups come in groups of eight, workgroup i
+// lands on part i mod 8; each reads its real part number from the hardware register and writes the copy of that
+// part), and a routing wave polls the copy of the part it runs on with loads that bypass the first-level cache.
+// Nothing depends on where the hardware places a workgroup: the gate workgroups of the first group also write
+// every word at device scope into a ninth copy, and a routing wave whose own part's copy stays incomplete for
+// GATE_LOCAL_SPINS polls goes on with that one.
+#define GATE_PARTS 8
+#define GATE_COPIES (GATE_PARTS + 1)  // one per part + the device-scope copy
+#define GATE_COPY_WORDS 512           // 8-byte words per copy (E + 1 <= 257 in use)
+#define GATE_LOCAL_SPINS 64u
+#define GATE_POLL_LIMIT (1u << 20)
+static __device__ __forceinline__ int xcc_id() {  // HW_REG_XCC_ID, bits 3:0
+  return (int)(__builtin_amdgcn_s_getreg(20 | (0 << 6) | ((4 - 1) << 11)) & (GATE_PARTS - 1));
+}
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+
+#ifdef MOE_STAMPS
+static __device__ unsigned long long g_stamps[1024 * 8];
+#define STAMP(i) do { if (lane == 0 && blockIdx.x < 1024) g_stamps[blockIdx.x * 8 + (i)] = wall_clock64(); } while (0)
+#define STAMPV(i, v) do { if (lane == 0 && blockIdx.x < 1024) g_stamps[blockIdx.x * 8 + (i)] = (v); } while (0)
+extern "C" int moe_debug_stamps_read(void *dst) { return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_stamps), sizeof(g_stamps)); }
+#else
+#define STAMP(i)
+#define STAMPV(i, v)
+#endif
+static __device__ __forceinline__ void gate_rows_stamped(const GemvArgs &a, const int lane, const int w) {
+  const int e = ((int)blockIdx.x >> 3) * 4 + w;   // eight workgroups (one per part of the chip) per block of four rows
+  if (e >= a.g_rows) return;
+  if (w == 0) { STAMP(0); STAMPV(7, (unsigned long long)xcc_id()); }
+  const int H = a.cls[1].K;
+  // (requested in front of the row: behind the sum it was one more trip to memory, 0.1 to 2 us)
+  const float bias_e = (a.g_bias && e < a.g_nbias) ? a.g_bias[e] : 0.f;
+  asm volatile("" :: "v"(bias_e));
+  const float acc = gate_row_sum(a.cls[1].act, a.g_w + (size_t)e * H, H, lane);
+  const float val = (a.g_bias && e < a.g_nbias) ? acc + bias_e : acc;
+  const u32x2_t word = {__float_as_uint(val), (u32)a.g_seq};
+  if (w == 0) STAMP(5);
+  if (lane == 0)  // into the second-level cache of this part
+    __builtin_amdgcn_raw_buffer_store_b64(word, make_rsrc(a.g_stamp + (size_t)xcc_id() * GATE_COPY_WORDS, GATE_COPY_WORDS * 8),
+                                          e * 8, 0, 1 /* sc0 */);
+  if (((int)blockIdx.x & 7) == 0) {
+    const unsigned long long word64 = ((unsigned long long)word.y << 32) | word.x;
+    if (lane == 1)
+      __hip_atomic_store(a.g_stamp + (size_t)GATE_PARTS * GATE_COPY_WORDS + e, word64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) a.g_logits_out[e] = val;  // for the kernels behind this launch (and the host)
+  }
+#ifdef MOE_STAMPS
+  if (w == 0) { asm volatile("" ::: "memory"); STAMP(1); asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); STAMP(2); }
+#endif
+}
 
 // Work item of a GEMV workgroup, resolved from the kernel arguments without dependent
 // loads when the units travel by value: both classes and the first 8 units are fetched
@@ -807,13 +896,13 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
 // the routed workgroups that share those compute units, and a tenth of the routed workgroups knew their expert
 // 2 us later than the others.
 template <int NR>
-static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &a, int lane, int w) {
+static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &a, int lane, int w, const int bx) {
   GemvWork wk;
   const int E = a.r_E, k = a.r_k;
   const int n_rt = k * a.cls[1].nblk + 1;
-  const bool sh = (int)blockIdx.x >= n_rt;
+  const bool sh = bx >= n_rt;
   wk.c = sh ? a.cls[0] : a.cls[1];
-  const int rr = sh ? (int)blockIdx.x - n_rt : (int)blockIdx.x;
+  const int rr = sh ? bx - n_rt : bx;
   const bool publisher = !sh && rr == k * wk.c.nblk;
   const int u = (sh || publisher) ? 0 : rr / wk.c.nblk;
   wk.b = rr - u * wk.c.nblk;
@@ -825,7 +914,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
   // LDS: four waves doing the same rounds would each take their turn on the SIMDs.  Workgroups b, b + 256, ...
   // share a compute unit when the grid is resident as a whole; they route on different SIMDs.
   __shared__ unsigned s_route_base[2];
-  const int rw = publisher ? 0 : (int)((blockIdx.x >> 8) & 3);
+  const int rw = publisher ? 0 : ((bx >> 8) & 3);
   wk.m = publisher ? 0 : 1; wk.row0 = u;
   if (w == rw) {
   const float NEG = -__builtin_inff();
@@ -834,10 +923,44 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
     const int e = lane + 64 * r;
-    v[r] = (e < E) ? a.r_logits[e] : NEG;
-    v0[r] = v[r];
+    v[r] = (e < E && a.g_nblk == 0) ? a.r_logits[e] : NEG;
     ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
   }
+  bool gate_timeout = false;
+  if (a.g_nblk) {
+    // the logits come from the gate workgroups of this launch (the first of the grid, so they are running or
+    // done when this one starts): poll the copy of this part of the chip until every word carries this launch's
+    // number; should that copy stay incomplete, go on with the device-scope copy
+    const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * GATE_COPY_WORDS, GATE_COPY_WORDS * 8);
+    const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * GATE_COPY_WORDS;
+    unsigned spins = 0;
+    STAMP(0); STAMPV(7, (unsigned long long)xcc_id());
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const int e = lane + 64 * r;
+        if (e < E) {
+          u32x2_t word;
+          if (spins < GATE_LOCAL_SPINS) {
+            word = __builtin_amdgcn_raw_buffer_load_b64(rl, e * 8, 0, 16 /* sc1: past the first-level cache */);
+          } else {
+            const unsigned long long w64 = __hip_atomic_load(cg + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+          }
+          v[r] = __uint_as_float(word.x);
+          ok = ok && (int)word.y == a.g_seq;
+        }
+      }
+      if (spins == 0) STAMP(1);
+      if (__ballot(!ok) == 0ull) break;
+      if (++spins >= GATE_POLL_LIMIT) { gate_timeout = true; break; }  // (never seen; the launch then reports an error)
+      __builtin_amdgcn_s_sleep(2);
+    }
+    STAMP(2); STAMPV(3, spins);
+  }
+#pragma unroll
+  for (int r = 0; r < NR; ++r) v0[r] = v[r];
   unsigned long long msel[NR];
 #pragma unroll
   for (int r = 0; r < NR; ++r) msel[r] = 0ull;
@@ -881,6 +1004,8 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
     }
     cum += cnt;
   }
+  if (gate_timeout) { lo = 0; hi = 0; }  // reported as a unit without a slot
+  STAMP(4);
   if (lane == 0) { s_route_base[0] = lo; s_route_base[1] = hi; }
 
   if (publisher) {  // publish the routing: weights as in k_topk, arrays as in k_dispatch (T = 1)
@@ -952,11 +1077,11 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
   return wk;
 }
 
-static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w) {
+static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a, int lane, int w, int bx) {
   // one instantiation per number of 64-wide logit columns: a 64-expert layer pays for one column only
-  if (a.r_E <= 64) return gemv_resolve_route_n<1>(a, lane, w);
-  if (a.r_E <= 128) return gemv_resolve_route_n<2>(a, lane, w);
-  return gemv_resolve_route_n<4>(a, lane, w);
+  if (a.r_E <= 64) return gemv_resolve_route_n<1>(a, lane, w, bx);
+  if (a.r_E <= 128) return gemv_resolve_route_n<2>(a, lane, w, bx);
+  return gemv_resolve_route_n<4>(a, lane, w, bx);
 }
 
 template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false>
@@ -1179,7 +1304,11 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
-  const GemvWork wk = gemv_resolve_route(a, lane, w);  // ends with a barrier (routed workgroups)
+  if ((int)blockIdx.x < a.g_nblk) {  // a gate workgroup (uniform per workgroup)
+    gate_rows_stamped(a, lane, w);
+    return;
+  }
+  const GemvWork wk = gemv_resolve_route(a, lane, w, (int)blockIdx.x - a.g_nblk);  // ends with a barrier (routed workgroups)
   const GemvClass &c = wk.c;
   const unsigned char *base = wk.base;
   if (wk.m <= 0) return;
@@ -1281,6 +1410,7 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
     red[(w * 2 + 0) * 16 + lane] = accA;
     red[(w * 2 + 1) * 16 + lane] = accB;
   }
+  if (w == 0) STAMP(5);
   __syncthreads();
   if (tid < 16) {
     float ga = 0.f, up = 0.f;
@@ -1292,6 +1422,7 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
     const float hv = ga / (1.f + expf(-ga)) * up;
     ((uint16_t *)c.out)[(size_t)wk.row0 * c.out_stride + b * 16 + tid] = f32_to_bf16(hv);
   }
+  if (w == 0) STAMP(6);
 }
 
 // ---------------------------------------------------------------------------
@@ -1329,7 +1460,16 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
   constexpr int RW = 16 / NI;  // rows of this workgroup
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
-  const int b16 = blockIdx.x / NI, part = blockIdx.x % NI;  // rows 16*b16 + RW*part .. + RW-1
+  // rows 16*b16 + RW*part .. + RW-1.  The two workgroups that share a 16-row tile (NI = 2) read the same lines of
+  // its scale and zero sections; workgroup i runs on the part of the chip i mod 8 that has its own second-level
+  // cache, so the pair is given indices that are equal mod 8 and the second one finds those lines there (with
+  // adjacent indices both fetched them from memory: 1.09 x the launch's bytes)
+  int b16 = blockIdx.x / NI, part = blockIdx.x % NI;
+  if (NI == 2 && (gridDim.x & 15) == 0) {
+    const int q = (int)blockIdx.x >> 3;
+    part = q & 1;
+    b16 = (q >> 1) * 8 + ((int)blockIdx.x & 7);
+  }
   const int mine = r / RW;                                  // which item of the group this lane works on
   const int rr = RW * part + (r % RW);                      // its row inside the 16-row tile
   const int k = a.k, I = a.I, I_sh = a.I_sh, G = a.G, G_sh = a.G_sh;
@@ -2465,13 +2605,20 @@ static int launch_gemv_route(const GemvArgs &a, int grid, size_t lds, hipStream_
   return moe_check_launch("k_w13_token");
 }
 
-extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, int k, int mode, int H, int I,
+// gate_w != NULL: the launch of phase bit 0 computes the gate logits itself (moe_decode_token_int4_gate)
+static int decode_token_int4_impl(const void *gate_w, const float *gate_bias, int n_gate_rows, void *gate_ws,
+                                  int gate_seq, const void *x, const float *logits, int E, int k, int mode, int H, int I,
                                      int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
                                      float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
                                      void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
                                      int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
+  if (gate_w && (!gate_ws || n_gate_rows < E || n_gate_rows > E + 1 || n_gate_rows > GATE_COPY_WORDS || !(phases & 1))) {
+    moe_set_error("moe_decode_token_int4_gate: needs the gate workspace, E or E + 1 gate rows (%d for E=%d) and "
+                  "phase bit 0", n_gate_rows, E);
+    return MOE_EINVAL;
+  }
   if (!x || !logits || !expert_ptr || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok ||
       !units || !n_active || !active_ids || !h_r || !part_r || !err || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E ||
       mode < 0 || mode > 2 || H <= 0 || H % 128 || I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 ||
@@ -2500,6 +2647,12 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
   a.n_sh_blocks = sh ? I_sh / 16 : 0;
   int grid = a.n_sh_blocks + k * (I / 16) + 1;  // + the publishing workgroup
+  if (gate_w) {  // + the gate workgroups (a wave per row), in front of all others
+    a.g_w = (const uint16_t *)gate_w; a.g_bias = gate_bias; a.g_stamp = (unsigned long long *)gate_ws;
+    a.g_logits_out = (float *)logits; a.g_rows = n_gate_rows; a.g_nbias = E; a.g_nblk = GATE_PARTS * ((n_gate_rows + 3) / 4);
+    a.g_seq = gate_seq;
+    grid += a.g_nblk;
+  }
   {
     const int gpw = (H / 128 + 3) / 4;
     int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
@@ -2550,6 +2703,36 @@ extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, 
   a.kunits_dev = (const KUnit *)unit_ws;
   grid = a.n_sh_blocks + k * (H / 32);
   return launch_gemv_t<false>(a, grid, 1, I_sh > I ? I_sh : I, I / 128, s);
+}
+
+extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, int k, int mode, int H, int I,
+                                     int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                     float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
+                                     int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
+                                     void *h_r, void *h_s, float *part_r, float *part_s, int *err,
+                                     void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
+                                     int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
+  return decode_token_int4_impl(nullptr, nullptr, 0, nullptr, 0, x, logits, E, k, mode, H, I, I_sh, expert_ptr, shared_ptr,
+                                idx, w, counts, offsets, sorted_pair, pos_of_pair, sorted_tok, units, n_active, active_ids,
+                                h_r, h_s, part_r, part_s, err, unit_ws, units_host_out, seq_host_out, seq_value, phases,
+                                shared_gate_logit, y_bf16, stream);
+}
+
+extern "C" int64_t moe_gate_ws_bytes(void) { return (int64_t)GATE_COPIES * GATE_COPY_WORDS * 8; }
+
+extern "C" int moe_decode_token_int4_gate(const void *x, const void *gate_w, const float *gate_bias, int n_gate_rows,
+                                          void *gate_ws, int gate_seq, float *logits, int E, int k, int mode, int H,
+                                          int I, int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                          float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
+                                          int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
+                                          void *h_r, void *h_s, float *part_r, float *part_s, int *err,
+                                          void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
+                                          int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
+  if (!gate_w) { moe_set_error("moe_decode_token_int4_gate: no gate matrix"); return MOE_EINVAL; }
+  return decode_token_int4_impl(gate_w, gate_bias, n_gate_rows, gate_ws, gate_seq, x, logits, E, k, mode, H, I, I_sh,
+                                expert_ptr, shared_ptr, idx, w, counts, offsets, sorted_pair, pos_of_pair, sorted_tok,
+                                units, n_active, active_ids, h_r, h_s, part_r, part_s, err, unit_ws, units_host_out,
+                                seq_host_out, seq_value, phases, shared_gate_logit, y_bf16, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -168,9 +168,24 @@ def experts_decode_int4(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.
     return part_r, part_s, err, h_r, h_s
 
 
+class GateWorkspace:
+    """Hand-over area of the launches that compute the gate logits themselves (moe_decode_token_int4_gate):
+    zeroed once; every call takes the next sequence number."""
+
+    def __init__(self, dev):
+        self.buf = torch.zeros(int(lib.moe_gate_ws_bytes()), dtype=torch.uint8, device=dev)
+        self.seq = 0
+
+    def next_seq(self) -> int:
+        self.seq = self.seq + 1 if self.seq < 0x7fffffff else 1
+        return self.seq
+
+
 def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int, ws=None,
-                      phases: int = 3, unit_ws=None, sg_logit=None, y=None):
-    """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
+                      phases: int = 3, unit_ws=None, sg_logit=None, y=None, gate=None):
+    """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s).
+    gate = (gate_w [rows, H] bf16, bias [E] or None, GateWorkspace): the launch computes the gate logits too and
+    `logits` (rows fp32) is an output."""
     dev = x.device
     if ws is None:
         idx = torch.empty(1, k, dtype=torch.int32, device=dev)
@@ -185,6 +200,17 @@ def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, 
         err = torch.zeros(1, dtype=torch.int32, device=dev)
     else:
         idx, w, d, part_r, part_s, err, h_r, h_s = ws
+    if gate is not None:
+        gw, gb, gws = gate
+        check(lib.moe_decode_token_int4_gate(ptr(_dev(x)), ptr(gw), ptr(gb), gw.shape[0], ptr(gws.buf), gws.next_seq(),
+                                             ptr(logits), E, k, mode, H, I, I_sh if shared is not None else 0,
+                                             ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
+                                             ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                             ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r),
+                                             ptr(part_s), ptr(err), ptr(unit_ws), 0, 0, 0, phases, ptr(sg_logit), ptr(y),
+                                             cur_stream()),
+              "moe_decode_token_int4_gate")
+        return idx, w, d, part_r, part_s, err, h_r, h_s
     check(lib.moe_decode_token_int4(ptr(_dev(x)), ptr(logits), E, k, mode, H, I, I_sh if shared is not None else 0,
                                     ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
                                     ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),

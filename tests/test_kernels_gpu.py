@@ -346,6 +346,59 @@ def test_token_decode_w2_and_combine_in_one_launch(cuda, H, I, E, k, mode, I_sh,
         assert np.abs(a - ref["out"]).max() <= TOL * np.abs(ref["out"]).max()
 
 
+@pytest.mark.parametrize("H,I,E,k,mode,I_sh,zipf,gated", [
+    (2048, 1408, 64, 6, 0, 2816, 1.2, False), (256, 384, 8, 2, 2, 256, None, True), (256, 256, 60, 4, 1, 512, 1.1, True),
+    (512, 128, 200, 8, 0, 0, None, False), (4096, 14336, 4, 2, 2, 0, None, False), (4608, 128, 130, 3, 0, 128, 1.1, True)])
+def test_token_decode_gate_rows_in_the_w13_launch(cuda, H, I, E, k, mode, I_sh, zipf, gated):
+    """One token, two launches: the w13 launch sums the gate rows in its first workgroups and hands the logits to
+    its routing waves.  Logits, routing and y must equal those of gate launch + the same kernels, bit for bit, on
+    successive calls over one hand-over workspace (a word of an earlier call must never pass for a new one)."""
+    from promoe_amd import ops
+    print(f"case token_gate H={H} I={I} E={E} k={k} mode={mode} I_sh={I_sh}", flush=True)
+    layer = Int4Layer(H=H, I=I, E=E, I_sh=I_sh, seed=7, zipf=zipf, shared_gate=gated)
+    slots = [torch.from_numpy(s).to(cuda) for s in layer.slots]
+    table = torch.tensor([s.data_ptr() for s in slots], dtype=torch.int64, device=cuda)
+    shared = torch.from_numpy(layer.shared_img).to(cuda) if I_sh else None
+    wg_np = layer.wg if not gated else np.concatenate([layer.wg, layer.shared_gate[None, :]], axis=0)
+    wg = bf16_dev(wg_np, cuda)
+    bias_e = None if layer.bias is None else torch.from_numpy(layer.bias).to(cuda)     # the routed rows only
+    bias_all = None if layer.bias is None else torch.from_numpy(
+        np.concatenate([layer.bias, np.zeros(wg_np.shape[0] - E, np.float32)])).to(cuda)
+    unit_ws = torch.zeros(32 * k, dtype=torch.uint8, device=cuda)
+    unit_ws2 = torch.zeros(32 * k, dtype=torch.uint8, device=cuda)
+    gws = ops.GateWorkspace(cuda)
+    ws2 = None
+    for seed in range(4):
+        x = O.synth_acts(1, H, seed=seed + 40)
+        if seed == 3:   # constructed ties
+            wg = wg.clone(); wg[3] = wg[1]; wg[E - 1] = wg[1]
+            if bias_e is not None:
+                bias_e = bias_e.clone(); bias_e[3] = bias_e[1]; bias_e[E - 1] = bias_e[1]
+                bias_all = bias_all.clone(); bias_all[3] = bias_all[1]; bias_all[E - 1] = bias_all[1]
+        xd = bf16_dev(x, cuda)
+        logits = ops.gate_logits(xd, wg, bias_all)
+        sg = logits[:, E] if gated else None
+        y_ref = torch.full((1, H), float("nan"), dtype=torch.bfloat16, device=cuda)
+        idx, w, d, _, _, err, h_r, h_s = ops.decode_token_int4(xd, logits, E, k, mode, table, shared, H, I, I_sh,
+                                                                phases=5, unit_ws=unit_ws, sg_logit=sg, y=y_ref)
+        logits2 = torch.full_like(logits, float("nan"))
+        sg2 = logits2[:, E] if gated else None
+        y = torch.full((1, H), float("nan"), dtype=torch.bfloat16, device=cuda)
+        ws2 = ops.decode_token_int4(xd, logits2, E, k, mode, table, shared, H, I, I_sh, ws=ws2, phases=5,
+                                    unit_ws=unit_ws2, sg_logit=sg2, y=y, gate=(wg, bias_e, gws))
+        idx2, w2, d2, _, _, err2, h_r2, h_s2 = ws2
+        torch.cuda.synchronize()
+        assert int(err.cpu()[0]) == 0 and int(err2.cpu()[0]) == 0
+        assert torch.equal(logits.view(torch.int32), logits2.view(torch.int32))
+        assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+        for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active"):
+            assert torch.equal(getattr(d, name), getattr(d2, name)), name
+        assert torch.equal(d.units[:k], d2.units[:k])
+        assert torch.equal(h_r.view(torch.int16), h_r2.view(torch.int16))
+        assert torch.equal(y_ref.view(torch.int16), y.view(torch.int16))
+    assert gws.seq == 4
+
+
 @pytest.mark.parametrize("T,E,k,mode", [(1, 64, 6, 0), (4, 64, 6, 0), (16, 64, 6, 1), (16, 60, 4, 2), (7, 200, 8, 0),
                                         (16, 8, 2, 2), (3, 256, 32, 0), (32, 64, 6, 0), (64, 64, 8, 1), (33, 60, 4, 2)])
 def test_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode):
