@@ -14,6 +14,7 @@ STUB(moe_topk_dispatch)
 STUB(moe_experts_decode_int4)
 STUB(moe_experts_decode_int4_publish)
 STUB(moe_decode_token_int4)
+STUB(moe_decode_token_int4_gate)
 STUB(moe_experts_decode_q4k)
 STUB(moe_experts_prefill)
 STUB(moe_experts_prefill_pieces)
@@ -23,3 +24,4 @@ extern "C" int moe_decode_shared_splits(...) { return 1; }
 extern "C" int moe_prefill_shared_splits(...) { return 1; }
 extern "C" int64_t moe_prefill_workspace_bytes(...) { return 0; }
 extern "C" int64_t moe_dispatch_workspace_bytes(...) { return 0; }
+extern "C" int64_t moe_gate_ws_bytes(...) { return 64; }
