@@ -58,11 +58,14 @@ def timed_steps(pm, xs, L_, steps, torch):
     return time.perf_counter() - t0
 
 
-def launches_timed(torch, launch_n, n):
+def launches_timed(torch, launch_n, n, replay_once=False):
     """Average duration (us) of n launches issued by launch_n(n) on the current stream, between ONE HIP event pair.
     The launches go into a HIP graph first and the graph is replayed between the events: issued one by one from
     Python (a ctypes call costs the host about 10 us) a kernel shorter than that is timed at the host's pace, not at
     its own.  launch_n must only launch kernels (no allocation, no synchronisation, nothing that clears memory).
+    replay_once: the launches carry a sequence number in their arguments that must not come twice (the launches
+    that hand their gate logits over inside the launch): one graph is recorded and replayed untimed, a second one
+    with the following numbers is recorded and its FIRST replay is the timed one.
     Falls back to the plain loop when the capture is refused."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     try:
@@ -74,6 +77,11 @@ def launches_timed(torch, launch_n, n):
                 launch_n(n)
             g.replay()                      # once untimed
             torch.cuda.synchronize()
+            if replay_once:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side, capture_error_mode="thread_local"):
+                    launch_n(n)
+                torch.cuda.synchronize()
             e0.record()
             g.replay()
             e1.record()
@@ -90,46 +98,45 @@ def launches_timed(torch, launch_n, n):
         return e0.elapsed_time(e1) * 1e3 / n, "%d back-to-back launches between one HIP event pair" % n
 
 
-def kernel_times(lib):
-    names = ["gate_logits", "topk", "dispatch", "gemv_w13_swiglu", "gemv_w2", "combine"]
-    out = {}
-    for kid, name in enumerate(names):
-        tot, n = C.c_double(), C.c_int()
-        lib.moe_kernel_timing_read(kid, C.byref(tot), C.byref(n))
-        if n.value:
-            out[name] = {"avg_us": tot.value * 1e3 / n.value, "calls": n.value}
-    return out
+PROFILE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+DECODE_SOURCES = ["promoe_amd/csrc/moe_kernels.hip", "promoe_amd/csrc/moe_device.h"]
+PREFILL_SOURCES = ["promoe_amd/csrc/moe_prefill.hip", "promoe_amd/csrc/moe_device.h"]
 
 
-TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
-                               "hbm_traffic_decode_T1_and_prefill_qwen.md")
-KERNEL_SOURCES = ["promoe_amd/csrc/moe_kernels.hip", "promoe_amd/csrc/moe_device.h"]
-
-
-def kernel_source_hash():
+def source_hash(sources):
     import hashlib
     h = hashlib.sha256()
     root = os.path.dirname(os.path.abspath(__file__))
-    for rel in KERNEL_SOURCES:
+    for rel in sources:
         with open(os.path.join(root, rel), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
 
 
-def recorded_traffic():
-    """HBM bytes per launch of the T=1 w13 kernel as recorded in the committed counter summary (lines
-    `decode_w13_traffic_bytes_per_launch: N` and `decode_kernel_source_sha256_16: H`); None when the summary
-    is missing or was measured on other kernel sources than the ones in the tree."""
+def recorded(fname, key, hash_key, sources):
+    """A figure that cannot be measured in-process (HBM bytes per launch from FETCH_SIZE / WRITE_SIZE counter runs,
+    a kernel's duration inside the timed steps from rocprofv3's kernel trace), read from the committed summary
+    `profiles/<fname>` (a line `<key>: <number>`); None when the summary is missing or was taken on other kernel
+    sources than the ones in the tree (the summary records their hash in the line `<hash_key>: <16 hex digits>`)."""
+    import re
     try:
-        text = open(TRAFFIC_PROFILE).read()
+        text = open(os.path.join(PROFILE_DIR, fname)).read()
     except OSError:
         return None
-    import re
-    m = re.search(r"decode_w13_traffic_bytes_per_launch:\s*(\d+)", text)
-    hsh = re.search(r"decode_kernel_source_sha256_16:\s*([0-9a-f]{16})", text)
-    if not m or not hsh or hsh.group(1) != kernel_source_hash():
+    m = re.search(r"^\s*%s:\s*([0-9.]+)\s*$" % re.escape(key), text, re.M)
+    hsh = re.search(r"^\s*%s:\s*([0-9a-f]{16})\s*$" % re.escape(hash_key), text, re.M)
+    if not m or not hsh or hsh.group(1) != source_hash(sources):
         return None
-    return int(m.group(1))
+    v = float(m.group(1))
+    return int(v) if v == int(v) else v
+
+
+def recorded_decode(key, fname="hbm_traffic_decode_and_prefill.md"):
+    return recorded(fname, key, "decode_kernel_source_sha256_16", DECODE_SOURCES)
+
+
+def recorded_prefill(key, fname="hbm_traffic_decode_and_prefill.md"):
+    return recorded(fname, key, "prefill_kernel_source_sha256_16", PREFILL_SOURCES)
 
 
 def cpu_baseline(T, H, I, E, I_sh, k, threads, budget_s=12.0):
@@ -213,13 +220,16 @@ def prefill_leg(torch, name, T, H, E, I, k, I_sh, fmt, gated, mode, steps=20):
     t_w2 = timed(lambda: ops.experts_prefill(x, d, table, sh, H, I, I_sh, fmt, phases=2, ws=ws), steps)
     flops = 2.0 * T * k * 3 * I * H + 2.0 * T * 3 * I_sh * H
     ach = flops * 2 / 3 / t_w13 / 1e12
+    tag = name.split("-")[0].split(".")[0].lower() + ("_q4k" if fmt == L.FMT_Q4K else ("_bf16" if fmt == L.FMT_BF16 else "_int4"))
     return {"workload": name, "tokens": T, "tokens_per_s": T / t_layer, "ms_per_layer": t_layer * 1e3,
             "expert_flops": flops, "weight_bytes": wbytes,
             "layer_TFLOPs": (flops + 2.0 * T * wg.shape[0] * H) / t_layer / 1e12,
             "roofline": {"bound": "mfma", "kernel": "k_prefill_%s<true> (w13 + SwiGLU, routed + shared in one launch)" %
                          ("gemm" if fmt == L.FMT_BF16 else ("int4<q4_K>" if fmt == L.FMT_Q4K else "int4")),
                          "achieved": ach, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_PEAK_TFLOPS,
-                         "traffic": None, "avg_launch_us": t_w13 * 1e6,
+                         # HBM bytes per launch from the committed FETCH_SIZE / WRITE_SIZE counter summary (null for a
+                         # leg without counters, or when the kernel sources changed since they were taken)
+                         "traffic": recorded_prefill("prefill_%s_w13_traffic_bytes_per_launch" % tag), "avg_launch_us": t_w13 * 1e6,
                          "algorithmic_flops_per_launch": flops * 2 / 3,
                          "method": "%d back-to-back launches (tile-list kernel included) between one HIP event pair" % steps},
             "w2_launch_us": t_w2 * 1e6, "w2_TFLOPs": flops / 3 / t_w2 / 1e12}
@@ -422,15 +432,10 @@ def main():
               "ms_per_step_min": reps[0] / n_timed * 1e3, "ms_per_step_max": reps[-1] / n_timed * 1e3,
               "first_region_of_exactly_steps_ms_per_step": dt_probe / a.steps * 1e3}
 
-    # per-kernel durations (HIP event pairs around every launch), separate short pass; an
-    # event pair adds about 2-3 us to a launch, so these are upper bounds
-    lib.moe_kernel_timing(1)
     xs = stack.acts(T, 8, seed=1)
     d_steps = min(a.steps, 20 * L_)
     act0 = pm.counters()["activated"]
     timed_steps(pm, xs, L_, d_steps, torch)
-    kt = kernel_times(lib)
-    lib.moe_kernel_timing(0)
     # distinct routed experts per step (D) for the algorithmic byte count
     D = (pm.counters()["activated"] - act0) / d_steps
     lay_r, lay_s = LY.int4_layout(H, I), LY.int4_layout(H, I_sh)
@@ -457,8 +462,10 @@ def main():
         def __init__(self, p): self.p = p
         def data_ptr(self): return self.p
 
-    # one token: the timed path runs the w13 GEMV that derives the routing itself; measure that kernel
-    logit_l = [ops.gate_logits(xs[0], stack.gate_w[l], stack.gate_bias[l]) for l in range(L_)]
+    # one token: the timed path runs the w13 GEMV that sums the gate rows in its first workgroups and derives the
+    # routing itself; measure that kernel (launched as moe_forward launches it: the gate logits are an output)
+    logits_out = torch.empty(1, E + 1, dtype=torch.float32, device=dev)
+    gate_ws = ops.GateWorkspace(dev)
     ws_tok = None
 
     def w13_only(n):
@@ -466,32 +473,41 @@ def main():
         for i in range(n):
             l = i % L_
             if T == 1:
-                ws_tok = ops.decode_token_int4(xs[0], logit_l[l], E, k, 0, _Tab(tables[l]), stack.shared[l], H, I, I_sh,
-                                               ws=ws_tok, phases=1)
+                ws_tok = ops.decode_token_int4(xs[i % len(xs)], logits_out, E, k, 0, _Tab(tables[l]), stack.shared[l], H, I,
+                                               I_sh, ws=ws_tok, phases=1, gate=(stack.gate_w[l], stack.gate_bias[l], gate_ws))
             else:
                 ops.experts_decode_int4(xs[0], routed[l], _Tab(tables[l]), stack.shared[l], H, I, I_sh, phases=1, ws=ws)
     w13_only(2 * L_)
     torch.cuda.synchronize()
     n_k = 20 * L_
-    w13_us, w13_method = launches_timed(torch, w13_only, n_k)
+    w13_us, w13_method = launches_timed(torch, w13_only, n_k, replay_once=(T == 1))
     assert int((ws_tok[5] if T == 1 else ws[2]).cpu()[0]) == 0
     D_k = float(np.mean([int(r.n_active.cpu()[0]) for r in routed]))
-    w13_bytes_k = D_k * lay_r["off2_q"] + lay_s["off2_q"] + 2 * T * H
+    gate_bytes = (E * H * 2 + E * 4) if T == 1 else 0          # gate rows + bias, read by the same launch at T = 1
+    w13_bytes_k = D_k * lay_r["off2_q"] + lay_s["off2_q"] + 2 * T * H + gate_bytes
     achieved = w13_bytes_k / (w13_us * 1e-6) / 1e9
-    roofline = {"bound": "hbm", "kernel": ("k_w13_token (w13 + SwiGLU, routing in the kernel)" if T == 1 else "k_gemv_int4_mfma (w13 + SwiGLU)"),
+    # the same kernel inside the timed steps (between the w2 + combine launches of the neighbouring steps), from
+    # the committed rocprofv3 kernel trace of this command; null when the kernel sources changed since
+    in_path_us = recorded_decode("decode_w13_in_path_avg_us", "decode_deepseek_int4_T1_kernel_trace.md") if (T == 1 and L_ == 27) else None
+    roofline = {"bound": "hbm", "kernel": ("k_w13_token (gate rows + routing + w13 + SwiGLU in one launch)" if T == 1 else "k_gemv_int4_mfma (w13 + SwiGLU)"),
                 "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this kernel at this
                 # workload (T=1, 27 layers), scaled by a copy kernel of known size; not measurable in-process:
                 # read from the committed counter summary, null when the kernel sources changed since
-                "traffic": recorded_traffic() if (T == 1 and L_ == 27) else None,
+                "traffic": recorded_decode("decode_w13_traffic_bytes_per_launch") if (T == 1 and L_ == 27) else None,
                 "algorithmic_bytes_per_launch": w13_bytes_k, "avg_launch_us": w13_us,
+                "avg_launch_us_in_timed_steps": in_path_us,
+                "frac_in_timed_steps": (w13_bytes_k / (in_path_us * 1e-6) / 1e9 / HBM_PEAK_GBS) if in_path_us else None,
                 "distinct_routed_experts_per_launch": D_k,
-                "method": w13_method}
-    chain_us = sum(v["avg_us"] for v in kt.values())
-    layer = {"algorithmic_bytes_per_step": layer_bytes, "kernel_chain_us": chain_us,
-             "chain_GBps": layer_bytes / (chain_us * 1e-6) / 1e9,
-             "wall_GBps": layer_bytes / (dt / a.steps) / 1e9}
+                "method": w13_method + "; avg_launch_us_in_timed_steps: rocprofv3 --kernel-trace of this command "
+                                       "(profiles/decode_deepseek_int4_T1_kernel_trace.md)"}
+    step_us = dt / a.steps * 1e6
+    layer = {"algorithmic_bytes_per_step": layer_bytes, "us_per_step": step_us,
+             "wall_GBps": layer_bytes / (dt / a.steps) / 1e9,
+             "frac_of_hbm_peak": layer_bytes / (dt / a.steps) / 1e9 / HBM_PEAK_GBS,
+             "launches_per_step": 2 if T == 1 else 5,
+             "w2_combine_avg_us_in_timed_steps": recorded_decode("decode_w2c_in_path_avg_us", "decode_deepseek_int4_T1_kernel_trace.md") if (T == 1 and L_ == 27) else None}
 
     sweep = {}
     if not a.no_sweep:
@@ -623,6 +639,7 @@ def main():
             # is launched kernel by kernel from Python and runs at the host's pace
             us_layer = Tn / sweep[str(Tn)] * 1e6 if str(Tn) in sweep else leg["us_per_layer"]
             gbps = leg["algorithmic_bytes_per_step"] / us_layer / 1e3
+            leg["roofline"]["traffic"] = recorded_decode("decode_T%d_w13_traffic_bytes_per_launch" % Tn)
             roofline_by_T[str(Tn)] = {"roofline": leg["roofline"], "us_per_layer": us_layer,
                                       "us_per_layer_launched_from_python": leg["us_per_layer"],
                                       "layer_GBps": gbps, "layer_frac_of_hbm_peak": gbps / HBM_PEAK_GBS,
@@ -639,7 +656,7 @@ def main():
                       "weights": "random int4-g128 images (uniform nibbles and zero points, fp16 scales 0.005 to 0.009): "
                                  "the kernels' time does not depend on the values"},
            "timing": timing, "c2_as_configured_tokens_per_s": as_configured,
-           "roofline": roofline, "roofline_by_T": roofline_by_T, "cpu_baseline": cpu, "cpu_baseline_more": cpu_more, "kernels_us": {n: round(v["avg_us"], 2) for n, v in kt.items()},
+           "roofline": roofline, "roofline_by_T": roofline_by_T, "cpu_baseline": cpu, "cpu_baseline_more": cpu_more,
            "layer": layer, "tokens_per_s_by_T": sweep, "cache_run": cache_run, "prefill": prefill, "other_decode_configs": others}
     print(json.dumps(out))
 

@@ -517,11 +517,13 @@ static void resolve_using(moe_engine *eng, Expert *v, std::unique_lock<std::mute
         // does not (the caller stopped, or took another path), an event recorded now proves the same
         const volatile int *sp = v->seq_ptr;
         const int need = v->seq_need;
+        eng->seq_pollers.fetch_add(1, std::memory_order_acq_rel);  // (under the lock: see moe_forward_prepare)
         lk.unlock();
         const auto t0 = std::chrono::steady_clock::now();
         bool reached = false;
         while (!(reached = (int)((unsigned)*sp - (unsigned)need) >= 0) &&
                std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(100)) {}
+        eng->seq_pollers.fetch_sub(1, std::memory_order_acq_rel);  // sp is not read again
         if (!reached) {
           lk.lock();
           if (!eng->proof_event) eng->proof_event = eng->be->event_create();
@@ -642,8 +644,6 @@ moe_engine::~moe_engine() {
   moe_predictor_free(this);
   if (fetch_thread.joinable()) fetch_thread.join();
   if (fw) { moe_forward_free(fw); fw = nullptr; }
-  for (LayerState *old : fw_retired) moe_forward_free(old);
-  fw_retired.clear();
 }
 
 extern "C" int moe_engine_create(const moe_cfg *cfg, int backend, void *compute_stream, moe_engine **out) {

@@ -19,7 +19,6 @@ struct LayerState {
   size_t part_s_elems = 0;  // floats behind part_s
   int *idx = nullptr, *counts = nullptr, *offsets = nullptr, *sorted_pair = nullptr, *pos_of_pair = nullptr,
       *sorted_tok = nullptr, *n_active = nullptr;
-  unsigned *route_counter = nullptr;
   unsigned char *unit_ws = nullptr;  // resolved units of the one-token path (16 bytes each)
   // one-token launches that compute their gate logits themselves: hand-over words (zeroed once) and the number
   // of the last such launch (every launch takes the next one, so no word of an earlier launch passes for a new one)
@@ -37,11 +36,16 @@ struct LayerState {
   // sees them without a copy: one per layer for launches in which that must not happen (checked at the next
   // call and when the engine drains), one for launches that are allowed to meet non-resident experts
   int *err_host = nullptr, *err_loose = nullptr;
-  // error words of the w2 + combine launches that go out before the host knows the routing (one per layer), and
-  // what the host expects of each once it does: 1 = must stay zero (every selected expert was resident at
-  // launch), 2 = may be set (an expert was missing; that launch's output is recomputed), 0 = none outstanding
+  // error words of the w2 + combine launches that go out before the host knows the routing, and what the host
+  // expects of each once it does: 1 = must stay zero (every selected expert was resident at launch), 2 = may be
+  // set (an expert was missing; that launch's output is recomputed), 0 = none outstanding.  Two words per layer,
+  // used in turn: the word a turn re-arms was last written by the launch of two turns ago, and between that
+  // launch and now the host has seen the sequence word of a LATER w13 kernel of the same stream (the one of the
+  // turn in between), so that launch is over and its word final.  With one word per layer and a single layer, the
+  // host could re-arm the word before the previous turn's launch had raised it.
   int *err_spec = nullptr;
   std::vector<char> spec_state;
+  std::vector<unsigned> spec_turn;
   int num_layer = 0;
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
@@ -136,9 +140,15 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
     HIPC(hipStreamSynchronize((hipStream_t)eng->be->compute_stream()));
     if (int rc = moe_forward_check_kernels(eng)) return rc;
     engine_drop_seq_releases(eng);
-    // the fetch thread may still be polling one of the old sequence words (it reads them without the
-    // lock): the old workspace is only freed with the engine, after that thread has been joined
-    eng->fw_retired.push_back(eng->fw);
+    // the fetch thread polls a sequence word without the lock.  No expert points at the old words any more (taken
+    // off under the lock just now, and a poll takes its pointer under the lock), so once the poll that may be in
+    // flight is over (it is bounded: 100 us, then an event of the drained stream) nothing reads the old workspace
+    while (eng->seq_pollers.load(std::memory_order_acquire) != 0) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+    }
+    moe_forward_free(eng->fw);
     eng->fw = nullptr;
   }
   LayerState *s = new LayerState();
@@ -157,7 +167,6 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->pos_of_pair, P);
   rc |= dalloc(s, &s->sorted_tok, P);
   rc |= dalloc(s, &s->n_active, 1);
-  rc |= dalloc(s, &s->route_counter, 1);
   rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
   rc |= dalloc(s, &s->gate_ws, (size_t)moe_gate_ws_bytes());
   rc |= dalloc(s, &s->units, s->max_units);
@@ -183,7 +192,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   s->num_layer = eng->cfg.num_layer;
   rc |= halloc(s, &s->err_host, eng->cfg.num_layer);
   rc |= halloc(s, &s->err_loose, 1);
-  rc |= halloc(s, &s->err_spec, eng->cfg.num_layer);
+  rc |= halloc(s, &s->err_spec, (size_t)2 * eng->cfg.num_layer);
   rc |= halloc(s, &s->opt_seq, 1);
   for (auto &p : s->pend) {
     rc |= halloc(s, &p.units, s->max_units);
@@ -195,9 +204,9 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   if (rc) return MOE_EHIP;
   memset(s->err_host, 0, sizeof(int) * eng->cfg.num_layer);
   *s->err_loose = 0;
-  memset(s->err_spec, 0, sizeof(int) * eng->cfg.num_layer);
-  s->spec_state.assign(eng->cfg.num_layer, 0);
-  HIPC(hipMemset(s->route_counter, 0, sizeof(unsigned)));
+  memset(s->err_spec, 0, sizeof(int) * 2 * eng->cfg.num_layer);
+  s->spec_state.assign((size_t)2 * eng->cfg.num_layer, 0);
+  s->spec_turn.assign(eng->cfg.num_layer, 0);
   HIPC(hipMemset(s->gate_ws, 0, (size_t)moe_gate_ws_bytes()));
   if (s->disp_ws) HIPC(hipMemset(s->disp_ws, 0, 64));
   *s->opt_seq = 0;
@@ -211,7 +220,8 @@ int moe_forward_check_kernels(moe_engine *eng) {
   LayerState *s = eng->fw;
   if (!s) return MOE_OK;
   for (int l = 0; l < s->num_layer; ++l)
-    if (((volatile int *)s->err_host)[l] || (s->spec_state[l] == 1 && ((volatile int *)s->err_spec)[l]))
+    if (((volatile int *)s->err_host)[l] || (s->spec_state[2 * l] == 1 && ((volatile int *)s->err_spec)[2 * l]) ||
+        (s->spec_state[2 * l + 1] == 1 && ((volatile int *)s->err_spec)[2 * l + 1]))
       return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", l);
   return MOE_OK;
 }
@@ -417,15 +427,17 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     // missing expert and raises its own error word, which the host then knows to expect).
     const float *sgo = d.shared_gated ? s->logits + E : nullptr;
     const bool spec_w2c = w2c_fits(d, k);
+    const int sw = 2 * layer + (int)(s->spec_turn[layer] & 1u);   // this turn's word
     if (spec_w2c) {
-      if (s->spec_state[layer] == 1 && ((volatile int *)s->err_spec)[layer])   // the launch of this layer's last turn
+      s->spec_turn[layer]++;
+      if (s->spec_state[sw] == 1 && ((volatile int *)s->err_spec)[sw])   // the launch of two turns ago: final
         return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", layer);
-      s->spec_state[layer] = 0;
-      s->err_spec[layer] = 0;
+      s->spec_state[sw] = 0;
+      s->err_spec[sw] = 0;
       if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                       d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                       s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                      s->h_r, s->h_s, s->part_r, s->part_s, s->err_spec + layer, s->unit_ws,
+                                      s->h_r, s->h_s, s->part_r, s->part_s, s->err_spec + sw, s->unit_ws,
                                       nullptr, nullptr, 0, 4, sgo, y, st)))
         return rc;
     }
@@ -468,7 +480,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     // again without the combine (the w13 kernel is still running) and leaves partial rows for the experts
     // computed below and the combine after them
     const bool w2c = later.empty() && spec_w2c;
-    if (spec_w2c) s->spec_state[layer] = later.empty() ? 1 : 2;
+    if (spec_w2c) s->spec_state[sw] = later.empty() ? 1 : 2;
     if (!w2c &&
         (rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
@@ -540,14 +552,6 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
                                 s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                 max_units, s->units_host, s->n_active_host, s->opt_seq, host_seq, st)))
-      return rc;
-  } else if (T <= 2 && E <= 256 && k <= 32 && T * k <= 512) {
-    // one or two tokens: gate + top-k + dispatch in one launch.  Its routing tail runs in a
-    // single workgroup behind a device-scope counter, which beats two more launches only
-    // while that tail is short (measured: +5 % tokens/s at T=1, -2 % at T=4, -25 % at T=16)
-    if ((rc = moe_route_decode(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, n_gate_rows, ldl, k, d.route_mode,
-                               s->idx, s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair,
-                               s->sorted_tok, s->units, s->n_active, s->active_ids, max_units, s->route_counter, st)))
       return rc;
   } else {
     if (!d.gate_bias) {

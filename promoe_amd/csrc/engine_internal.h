@@ -200,6 +200,7 @@ struct moe_engine {
   std::vector<std::deque<CopyTask>> layer_q;
   CopyTask current;  // the one copy in flight (current.e == nullptr: none)
   std::atomic<unsigned> task_epoch{0};  // bumped with every queued task
+  std::atomic<int> seq_pollers{0};      // fetch thread inside its unlocked poll of a sequence word
   std::thread fetch_thread;
   bool launched = false, exiting = false, slots_ready = false;
   std::string fatal;  // first broken invariant (the reference would have aborted)
@@ -217,7 +218,6 @@ struct moe_engine {
   // fused forward
   std::vector<moe_layer_desc> layer_desc;
   LayerState *fw = nullptr;
-  std::vector<LayerState *> fw_retired;  // workspaces of earlier moe_forward_prepare calls, freed with the engine
   PredictorState *pred = nullptr;
 
   ~moe_engine();

@@ -1372,6 +1372,9 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
     }
     if (scj < 2 * CH) wsc[lane] = sd;
     if (zzj < 2 * CH) wzz[lane] = zd;
+    // (lanes read below what other lanes of the wave stored above: a wave's LDS operations complete in order; the
+    // wave barrier is no instruction, it keeps the compiler from moving the reads in front of the stores)
+    __builtin_amdgcn_wave_barrier();
     // everything the products need besides the tiles is read and converted before the first tile is waited
     // for: what a wave does after its last byte has arrived (all tiles of a wave arrive together) is the tail
     // of the launch, and only the unpacking and the dot products have to be in it
@@ -1402,6 +1405,7 @@ __global__ __launch_bounds__(256, 3) void k_w13_token(const GemvArgs a) {
       accB = fmaf(fsb[j], dB - fzb[j] * xq[j], accB);
       __builtin_amdgcn_sched_barrier(0);
     }
+    __builtin_amdgcn_wave_barrier();  // the next chunk's stores stay behind this chunk's reads
   }
   // reduce the four k-quarters of the wave, then the four waves
   accA += __shfl_xor(accA, 16, 64); accA += __shfl_xor(accA, 32, 64);
@@ -1562,6 +1566,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
         if ((lane & 3) == 0) xsum[(c * NI + lj) * 4 + (lpart >> 2)] = ps;
       }
     }
+    __builtin_amdgcn_wave_barrier();  // (no instruction: the reads below stay behind the stores of other lanes)
     // ---- products: no branch, an absent item has zero weights, a zero scale and zero activations
 #pragma unroll
     for (int c = 0; c < W2C_CHUNK; ++c) {
@@ -1575,6 +1580,7 @@ __global__ __launch_bounds__(64 * W2C_WAVES, 1) void k_w2_combine_token(const W2
       const float fz = 128.f + (float)((zz[c] >> zsh) & 15);
       acc = fmaf(wgt[c] * fs, d - fz * xq, acc);
     }
+    __builtin_amdgcn_wave_barrier();  // the next chunk's stores stay behind this chunk's reads
   }
   // the items of the groups, the four k quarters of the wave, then the waves
 #pragma unroll

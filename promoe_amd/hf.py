@@ -109,10 +109,11 @@ def inject_model(model, device="cuda:0", fmt: str = "bf16", max_tokens: int = 40
         gu, dn = blk.experts.gate_up_proj, blk.experts.down_proj
         if tuple(gu.shape) != (E, 2 * I, H) or tuple(dn.shape) != (E, H, I):
             raise ValueError("block %s differs in shape from the first block" % name)
-        # DeepSeek scales the routed experts' sum by a constant; it goes into their down projections
+        # DeepSeek scales the routed experts' sum by a constant; it goes into their down projections (multiplied in
+        # fp32, before the one rounding to bf16 / the quantisation of the image)
         scale = float(getattr(blk.gate, "routed_scaling_factor", 1.0) or 1.0)
         for e in range(E):
-            img = _expert_image(gu[e, :I], gu[e, I:], dn[e] if scale == 1.0 else dn[e] * scale, H, I, fmt)
+            img = _expert_image(gu[e, :I], gu[e, I:], dn[e] if scale == 1.0 else dn[e].detach().float() * scale, H, I, fmt)
             base = (l * E + e) * total
             stage.array[base: base + total] = img
         sh = _shared_expert(blk)

@@ -248,6 +248,10 @@ def experts_decode_q4k(x, d: Dispatch, expert_ptr: torch.Tensor, shared: torch.T
             # the w2 pass may split the shared expert's reduction: one set of partial rows per split
             part_s = torch.empty(shared_splits(L.FMT_Q4K, T, H, I_sh) * T, H, dtype=torch.float32, device=dev)
         err = torch.zeros(1, dtype=torch.int32, device=dev)
+    if part_s is not None:
+        pieces = shared_splits(L.FMT_Q4K, T, H, I_sh)
+        if part_s.shape[0] != pieces * T:   # a workspace made for another batch size
+            part_s = torch.empty(pieces * T, H, dtype=torch.float32, device=dev)
     check(lib.moe_experts_decode_q4k(ptr(_dev(x)), T, H, I, I_sh if shared is not None else 0, k,
                                      ptr(d.units), d.max_units, ptr(d.sorted_tok), ptr(expert_ptr),
                                      ptr(shared), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
@@ -291,13 +295,22 @@ def shared_splits(fmt: int, T: int, H: int, I_sh: int) -> int:
 
 
 def combine(part_r, part_s, topk_w, pos_of_pair, shared_gate_logit, T: int, H: int, k: int,
-            out: torch.Tensor | None = None):
-    """part_s [S*T, H]: S > 1 when the shared expert's reduction was split (piece s = rows s*T .. s*T+T-1)."""
+            out: torch.Tensor | None = None, pieces: int | None = None):
+    """part_s [S*T, H]: S > 1 when the shared expert's reduction was split (piece s = rows s*T .. s*T+T-1).
+    pieces: S as the expert launch left it (shared_splits / moe_prefill_shared_splits); inferred from the rows of
+    part_s when not given, which is only right for a part_s made for exactly this T."""
     dev = (part_r if part_r is not None else part_s).device
     if out is None:
         out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
     sg_stride = shared_gate_logit.stride(0) if shared_gate_logit is not None else 0
-    n_splits = 1 if part_s is None else max(1, part_s.shape[0] // max(T, 1))
+    if part_s is None:
+        n_splits = 1
+    elif pieces is not None:
+        n_splits = int(pieces)
+        assert part_s.shape[0] >= n_splits * T, "part_s holds fewer rows than pieces x tokens"
+    else:
+        assert part_s.shape[0] % max(T, 1) == 0, "part_s was made for another batch size: pass pieces"
+        n_splits = max(1, part_s.shape[0] // max(T, 1))
     check(lib.moe_combine_splits(ptr(part_r), ptr(part_s), ptr(topk_w), ptr(pos_of_pair),
                                  ptr(shared_gate_logit), sg_stride, ptr(out), T, H, k, n_splits, cur_stream()),
           "moe_combine")

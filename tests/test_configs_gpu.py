@@ -141,6 +141,27 @@ def test_c4_mixtral_layers_through_cache(cuda):
     pm.close()
 
 
+def test_c4_mixtral_prefill_512_tokens_against_the_oracle(cuda):
+    """The int4 tile kernel at Mixtral's reduction lengths (K = 4096 in w13, K = 14336 in w2) against the fp32
+    restatement: 512 tokens, top-2 then softmax, 128 rows per expert (the 4096-token size of the configuration is
+    covered by the size-independent property test; the arithmetic per tile is the same)."""
+    from tests.test_prefill_gpu import run_prefill_gpu
+    print("case C4 mixtral prefill T=512 vs oracle", flush=True)
+    torch.set_num_threads(max(torch.get_num_threads(), 8))
+    H, I, E, k, T = 4096, 14336, 8, 2, 512
+    layer = LazyInt4Layer(H=H, I=I, E=E, seed=82)
+    x = O.synth_acts(T, H, seed=1350)
+    layer.experts_fp32 = None   # (run_prefill_gpu does not read it)
+    got = run_prefill_gpu(layer, x, k, 2, cuda)
+    ref = ref_forward_lazy(layer, x, k, 2)
+    assert got["err"] == 0
+    assert np.array_equal(got["idx"], ref["idx"])
+    err = np.abs(got["y"] - ref["out"]).max() / np.abs(ref["out"]).max()
+    print(f"  max-rel-err {err:.3e}", flush=True)
+    assert err <= TOL
+    layer.drop_cache()
+
+
 @pytest.fixture(scope="module")
 def qwen2_q4k_layer():
     # the layer's real widths; 16 experts instead of 64 keep the host-side quantisation short
@@ -154,6 +175,27 @@ def test_c5_q4k_decode_three_sequences(cuda, qwen2_q4k_layer):
     print("case C5 q4_K decode, shared expert 20480 wide", flush=True)
     for T in (1, 3):
         check_layer(qwen2_q4k_layer, T, 8, 0, cuda, seed=40 + T)
+
+
+def test_c5_q4k_decode_64_experts_top8(cuda, qwen2_q4k_layer):
+    """T = 3 with the configuration's 64 experts and top-8: the 16 quantised experts of the fixture appear four
+    times each under a shuffled numbering (64 slot images at 64 addresses), the gate has 64 rows."""
+    from tests.test_kernels_gpu import check_layer
+    print("case C5 q4_K decode, E=64 k=8", flush=True)
+    base = qwen2_q4k_layer
+
+    rng = np.random.default_rng(5)
+    perm = rng.permutation(64) % 16
+    lay = object.__new__(Q4KLayer)   # (the checks pick the kernels by the layer's class; no quantisation here)
+    lay.H, lay.I, lay.E, lay.I_sh = base.H, base.I, 64, base.I_sh
+    g = torch.Generator().manual_seed(77)
+    lay.wg = O.round_bf16((torch.randn(64, base.H, generator=g) * 0.02).numpy())
+    lay.bias = O.zipf_gate_bias(64, 1.1, seed=2)
+    lay.experts_fp32 = [base.experts_fp32[p] for p in perm]
+    lay.slots = [base.slots[p].copy() for p in perm]
+    lay.shared_fp32, lay.shared_img, lay.shared_gate = base.shared_fp32, base.shared_img, base.shared_gate
+    for T in (1, 3):
+        check_layer(lay, T, 8, 0, cuda, seed=60 + T)
 
 
 def test_c5_q4k_mixed_batch_through_forward(cuda, qwen2_q4k_layer):
@@ -185,10 +227,11 @@ def test_c5_q4k_mixed_batch_through_forward(cuda, qwen2_q4k_layer):
     pm.close()
 
 
-@pytest.mark.parametrize("policy", ["nn", "min", "static-1"])
+@pytest.mark.parametrize("policy", ["nn", "min", "static-1", "static-2", "lru-global", "fifo-global"])
 def test_other_policies_on_the_hip_backend(cuda, policy):
-    """NN, MIN and Static-1 victim selection with real copies underneath: residency and counters against the
-    restated reference policies (cache.hpp:81-126, cache.cpp:340-381, 490-583), outputs against the oracle."""
+    """NN, MIN, Static-1 and Static-2 victim selection with real copies underneath, and one slot group for all
+    layers (per_layer_cache off, cache.hpp:247-259): residency and counters against the restated reference
+    policies (cache.hpp:81-126, cache.cpp:340-381, 490-583), outputs against the oracle."""
     from tests.synth import Int4Layer
     from tests.test_engine_gpu import ref_forward
     print(f"case policy {policy} on the HIP backend", flush=True)
@@ -199,9 +242,11 @@ def test_other_policies_on_the_hip_backend(cuda, policy):
     tokens = (lambda s: 1) if policy == "min" else (lambda s: 1 if s % 4 else 5)
     xs = [[O.synth_acts(tokens(s), H, seed=1500 + s * Lyr + l) for l in range(Lyr)] for s in range(n_steps)]
     refs = [[ref_forward(layers[l], xs[s][l], k, 0) for l in range(Lyr)] for s in range(n_steps)]
-    cfg = dict(cache_rate=0.375, cache_policy=policy, num_predict_expert_per_layer=0)
+    per_layer = not policy.endswith("-global")
+    policy = policy.split("-global")[0]
+    cfg = dict(cache_rate=0.375, cache_policy=policy, num_predict_expert_per_layer=0, per_layer_cache=per_layer)
     pm = build_engine(layers, k, cuda, **cfg)
-    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy=policy, num_predict=0)
+    sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy=policy, num_predict=0, per_layer_cache=per_layer)
     if policy == "min":
         dec = np.array([[np.unique(refs[s][l]["idx"]) for l in range(Lyr)] for s in range(n_steps)], np.int32)
         em = np.stack([np.zeros(n_steps, np.int64), np.arange(n_steps)], 1)

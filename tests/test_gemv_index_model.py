@@ -13,14 +13,62 @@ descriptors of a load lies inside the image / the h vector, and that items past 
 outside the descriptor (they read zeros).  Any index outside its buffer fails the sweep.
 """
 import itertools
+import os
+import re
 
 import pytest
 
 from promoe_amd import layout as LY
 
+# The model's constants come out of the kernel source, and the rules it restates (launcher choices, block order,
+# workgroup -> rows mapping) are checked to stand in the source word for word: a change there fails this file
+# until the model follows.
+_SRC = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "promoe_amd", "csrc",
+                         "moe_kernels.hip")).read()
+
+
+def _define(name):
+    m = re.search(r"^#define %s(\([a-z]+\))? +(.+?)(?: *//.*)?$" % name, _SRC, re.M)
+    assert m, "no #define %s in moe_kernels.hip" % name
+    return m.group(2).strip()
+
+
+def _source_has(*lines):
+    flat = " ".join(_SRC.split())
+    for ln in lines:
+        assert " ".join(ln.split()) in flat, "moe_kernels.hip no longer contains: " + ln
+
+
+_W13T_WAVE_DW = _define("W13T_WAVE_DW")          # an expression in (ch)
+W2C_WAVES = int(_define("W2C_WAVES"))
+GATE_PARTS = int(_define("GATE_PARTS"))
+GATE_COPY_WORDS = int(_define("GATE_COPY_WORDS"))
+
+
+def test_restated_rules_stand_in_the_source():
+    _source_has(
+        # launcher: tiles in flight per wave of k_w13_token, its LDS size, its grid
+        "int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;",
+        "static size_t w13_token_lds(int ch) { return (size_t)4 * W13T_WAVE_DW(ch) * 4 + 4 * 2 * 16 * 4; }",
+        "int grid = a.n_sh_blocks + k * (I / 16) + 1;",
+        "a.g_nblk = GATE_PARTS * ((n_gate_rows + 3) / 4);",
+        # block order of k_w13_token: gate workgroups, routed, publisher, shared
+        "if ((int)blockIdx.x < a.g_nblk) {",
+        "const int n_rt = k * a.cls[1].nblk + 1;",
+        "const bool publisher = !sh && rr == k * wk.c.nblk;",
+        "const int e = ((int)blockIdx.x >> 3) * 4 + w;",
+        # launcher of k_w2_combine_token and its workgroup -> rows mapping
+        "const int loads_per_wave = (k * ((c.G + 1) / 2) + (c.G_sh + 1) / 2 + W2C_WAVES - 1) / W2C_WAVES;",
+        "if (loads_per_wave <= 3) hipLaunchKernelGGL((k_w2_combine_token<2, 3>), dim3(H / 8)",
+        "else if (H / 16 >= 256)",
+        "if (NI == 2 && (gridDim.x & 15) == 0) {",
+        "b16 = (q >> 1) * 8 + ((int)blockIdx.x & 7);",
+        "extern \"C\" int64_t moe_gate_ws_bytes(void) { return (int64_t)GATE_COPIES * GATE_COPY_WORDS * 8; }",
+        "#define GATE_COPIES (GATE_PARTS + 1)")
+
 
 def w13_wave_dw(ch):
-    return ch * 64 + ch * 4 + ch * 16 + ch * 4
+    return int(eval(_W13T_WAVE_DW, {"ch": ch}))
 
 
 def w13_token_lds(ch):
@@ -77,6 +125,21 @@ def model_route_launch(E, k, H, I, I_sh):
                     assert ((half + g) * 8 + 7) * 4 + 4 <= 2 * G * 32
                     assert ((half + g) * 2 + 1) * 4 + 4 <= 2 * G * 8
                     assert 63 * 16 + (half + g) * 1024 + 16 <= 2 * G * 1024
+    # gate workgroups in front of the grid (launches that sum the gate rows themselves): eight per block of four
+    # rows; a wave writes word e of one of GATE_PARTS + 1 copies of GATE_COPY_WORDS words
+    for rows in (E, E + 1):
+        g_nblk = GATE_PARTS * ((rows + 3) // 4)
+        covered = set()
+        for bxg in range(g_nblk):
+            for w in range(4):
+                e = (bxg >> 3) * 4 + w
+                if e < rows:
+                    covered.add((bxg & 7, e))
+                    assert e < GATE_COPY_WORDS
+                    for copy in range(GATE_PARTS + 1):
+                        assert (copy * GATE_COPY_WORDS + e) * 8 + 8 <= (GATE_PARTS + 1) * GATE_COPY_WORDS * 8
+        # with workgroup i on part i mod 8 of the chip, every part sums every row
+        assert covered == {(p_, e) for p_ in range(GATE_PARTS) for e in range(rows)}
     n_checked = 0
     n_pub = 0
     for bx in range(grid):
@@ -113,7 +176,13 @@ def model_route_launch(E, k, H, I, I_sh):
     return n_checked
 
 
-W2C_WAVES = 16
+def w2c_rows_of(bx, grid, NI):
+    """(b16, part) of workgroup bx (k_w2_combine_token): pairs that share a tile get indices equal mod 8."""
+    b16, part = bx // NI, bx % NI
+    if NI == 2 and grid % 16 == 0:
+        q = bx >> 3
+        part, b16 = q & 1, (q >> 1) * 8 + (bx & 7)
+    return b16, part
 
 
 def launcher_w2c(k, H, I, I_sh):
@@ -205,10 +274,13 @@ def model_w2_combine_launch(k, H, I, I_sh, NI=2, CHUNK=3):
     for u in range(k):
         assert u * I + G * 128 <= k * I
     assert G_sh * 128 <= max(I_sh, 0)
-    # output rows
+    # output rows: every (tile, part) exactly once
+    seen_rows = set()
     for bx in range(grid):
-        b16, part = bx // NI, bx % NI
-        assert b16 < H // 16 and b16 * 16 + RW * part + RW - 1 < H
+        b16, part = w2c_rows_of(bx, grid, NI)
+        assert 0 <= part < NI and 0 <= b16 < H // 16 and b16 * 16 + RW * part + RW - 1 < H
+        seen_rows.add((b16, part))
+    assert len(seen_rows) == grid == (H // 16) * NI
     return grid
 
 

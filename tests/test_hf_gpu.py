@@ -94,17 +94,19 @@ def test_mixtral_model_through_the_engine_int4(cuda):
     _compare(model, cuda, "int4", 3e-2, cache_rate=1.0)
 
 
-def test_deepseek_model_through_the_engine(cuda):
+@pytest.mark.parametrize("scaling", [1.0, 2.5])
+def test_deepseek_model_through_the_engine(cuda, scaling):
     """DeepSeek family (stock transformers DeepseekV2): a dense first layer, then sparse blocks with greedy
-    softmax top-k routing and a plain shared expert of two experts' width; half of the experts resident."""
-    print("case hf_deepseek", flush=True)
+    softmax top-k routing and a plain shared expert of two experts' width; half of the experts resident.
+    scaling: routed_scaling_factor (it goes into the routed experts' down projections; 2.5 is no power of two)."""
+    print(f"case hf_deepseek scaling={scaling}", flush=True)
     from transformers import DeepseekV2Config, DeepseekV2ForCausalLM
     from promoe_amd import hf
     cfg = DeepseekV2Config(vocab_size=128, hidden_size=256, intermediate_size=512, moe_intermediate_size=128,
                            num_hidden_layers=3, num_attention_heads=4, num_key_value_heads=4, n_shared_experts=2,
                            n_routed_experts=8, num_experts_per_tok=2, first_k_dense_replace=1, kv_lora_rank=32,
                            q_lora_rank=None, qk_rope_head_dim=16, qk_nope_head_dim=32, v_head_dim=32, head_dim=16,
-                           topk_method="greedy", routed_scaling_factor=1.0, max_position_embeddings=128)
+                           topk_method="greedy", routed_scaling_factor=scaling, max_position_embeddings=128)
     torch.manual_seed(3)
     model = DeepseekV2ForCausalLM(cfg)
     names = [n for n, _ in hf.find_moe_blocks(model)]
