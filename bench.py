@@ -523,11 +523,13 @@ def main():
     cache_run = None
     as_configured = None
     if not a.no_cache_run:
-        def cache_leg(Tn, predict=None):
+        def cache_leg(Tn, predict=None, min_precision=0.0):
             """predict: None (demand fetching only), "exact" (every layer of a token sees one hidden state, so the
             gate-as-predictor is always right: what prefetching can hide at best) or "drifting" (the hidden state
             of a token drifts from layer to layer, x_l+1 = x_l + 0.5 noise: predictions made from an earlier
-            layer's input are sometimes wrong, as with a real model)."""
+            layer's input are sometimes wrong, as with a real model).  min_precision: requests for a layer whose
+            predictions were lately right for less than this share go out empty (0: all go out, as in the
+            reference)."""
             cfg = dict(cache_rate=0.375, cache_policy="lru", reorder_experts=True, early_preempt=True,
                        num_predict_expert_per_layer=k if predict else 0)
             if predict:
@@ -538,6 +540,8 @@ def main():
                 for src, (f0, f1) in enumerate(pm2.predictor_windows()):
                     for dst in range(f0, f1):
                         pm2.set_predictor_model(src, dst, stack.gate_w[dst], stack.gate_bias[dst])
+                if min_precision > 0:
+                    pm2.set_predictor_min_precision(min_precision)
                 pm2.start_predictor()
             n_tok = 64
             base = stack.acts(Tn, n_tok, seed=3)
@@ -566,6 +570,7 @@ def main():
             torch.cuda.synchronize()
             d3 = time.perf_counter() - t0
             c2 = pm2.counters()
+            withheld = pm2.predictor_precision()[1] if predict else None
             pm2.close()
             dl = {kk: c2[kk] - c0[kk] for kk in ("hit", "miss", "prefetch_hit", "prefetch_miss", "ready", "unready",
                                                  "wait_us", "h2d_bytes")}
@@ -575,11 +580,15 @@ def main():
                     "h2d_GBps": dl["h2d_bytes"] / d3 / 1e9, "steps": n2, "misses": dl["miss"],
                     "wait_us_per_miss": dl["wait_us"] / max(dl["miss"], 1) if not predict else None,
                     "prefetch_hits": dl["prefetch_hit"], "prefetch_copies": dl["prefetch_miss"],
-                    "ready_rate": dl["ready"] / max(dl["ready"] + dl["unready"], 1), "wait_us_total": dl["wait_us"]}
+                    "ready_rate": dl["ready"] / max(dl["ready"] + dl["unready"], 1), "wait_us_total": dl["wait_us"],
+                    "predictor_min_precision": min_precision if predict else None, "requests_sent_empty": withheld}
         cache_run = cache_leg(T)
         if T == 1:
             cache_run["with_predictor"] = cache_leg(T, "exact")
-            cache_run["with_predictor_drifting_hidden_state"] = cache_leg(T, "drifting")
+            # mispredictions cost copies that evict useful experts: with the predictor's precision feedback on
+            # (requests for layers it lately got wrong go out empty) and with every request sent as ranked
+            cache_run["with_predictor_drifting_hidden_state"] = cache_leg(T, "drifting", min_precision=0.5)
+            cache_run["with_predictor_drifting_hidden_state_every_request_sent"] = cache_leg(T, "drifting")
         # the decode configuration as configured (cache rate 0.375, LRU, demand fetching): T = 1, 4, 16
         as_configured = {}
         for Tn in (1, 4, 16):

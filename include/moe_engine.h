@@ -166,6 +166,16 @@ int moe_predictor_stats(moe_engine *eng, uint64_t *n_jobs, uint64_t *n_requests)
  * moment); 0 = idle, 1 = still busy after timeout_ms (it may be waiting for the run-ahead budget, which only
  * further layers release).  No counterpart in the reference, whose worker is joined at exit only. */
 int moe_predictor_wait_idle(moe_engine *eng, int timeout_ms);
+/* Requests scored against what the layers then route to.  Every decode step's routing of a layer
+ * (moe_report_one_layer) is compared with the ranking the predictor made for that turn; the share of the
+ * ranked experts that were routed to is kept as a moving average per destination layer (0.8 old + 0.2 new,
+ * starting at 1).  moe_predictor_set_min_precision(t), t in (0, 1]: a request for a layer whose average is below t
+ * goes out EMPTY (as a prefill step's does: the layer's progress count stays in step and nothing is copied)
+ * until the average has recovered; the ranking is still made and scored.  t = 0 (the default): every request
+ * goes out as ranked, as in the reference (worker.cpp:41-68), whose PredictWorker has no such feedback.
+ * moe_predictor_precision: the averages (num_layer floats) and the number of requests sent empty so far. */
+int moe_predictor_set_min_precision(moe_engine *eng, float min_precision);
+int moe_predictor_precision(moe_engine *eng, float *precision, uint64_t *n_withheld);
 
 /* ---- Belady policy hooks: CacheOracle / set_cur_seq (adapter.cpp:62-70, cache.cpp:592-644) ---- */
 int moe_oracle_load(moe_engine *eng, const int64_t *entry_metas, int64_t n_entries,

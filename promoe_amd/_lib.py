@@ -66,6 +66,8 @@ _sig("moe_predictor_windows", [vp, vp, vp])
 _sig("moe_predictor_set_model", [vp, i32, i32, vp, vp, i32])
 _sig("moe_predictor_start", [vp])
 _sig("moe_predictor_stats", [vp, vp, vp])
+_sig("moe_predictor_set_min_precision", [vp, C.c_float])
+_sig("moe_predictor_precision", [vp, vp, vp])
 _sig("moe_predictor_wait_idle", [vp, C.c_int])
 _sig("moe_q4k_layout_make", [i32, i32, C.POINTER(Int4Layout)])
 _sig("moe_experts_decode_q4k", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp])

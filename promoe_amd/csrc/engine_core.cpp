@@ -900,6 +900,9 @@ static int report_one_layer_locked(moe_engine *eng, int layer, int64_t *ids, int
   if (eng->predictor_attached) {  // consume_prefetch_layer_progress (worker.hpp:312-314)
     eng->cv_sem.wait(lk, [&] { return eng->progress > 0 || eng->exiting; });
     if (eng->progress > 0) eng->progress--;
+    // the layer's request for this turn has been issued: a decode step (prefetcher.cpp:467: at most top-k ids)
+    // tells the built-in predictor what the layer routed to, before the hooks reorder the ids
+    if (n > 0 && n <= std::max(eng->cfg.num_expert_per_token, 1)) moe_predictor_observe(eng, layer, ids, n);
   }
   // PreemptTask (prefetcher.cpp:521-537)
   if (eng->cfg.reorder_experts) reorder_experts(eng, layer, ids, n);

@@ -229,6 +229,8 @@ void moe_predictor_free(moe_engine *eng);
 int moe_predictor_on_logits(moe_engine *eng, int layer, const void *hidden, int B, int S, int H);
 bool moe_predictor_fused_rows(moe_engine *eng, int layer, int H, const void **w, const float **bias, float **out, int *rows);
 int moe_predictor_scores_pending(moe_engine *eng, int layer, const int *seq_word, int seq_value);
+// the routing of a decode step at `layer` (before the hooks reorder it): what the layer's last prediction is scored against
+void moe_predictor_observe(moe_engine *eng, int layer, const int64_t *ids, int64_t n);
 // moe_report_layer_logits without the predictor's part (the caller runs that part itself)
 int moe_report_layer_logits_bookkeeping(moe_engine *eng, int layer, int S);
 // launching -> using without an event: the experts count as in use until *seq_ptr reaches seq_need

@@ -50,6 +50,15 @@ struct PredictorState {
   bool exit = false, started = false, host_math = false;
   uint64_t n_jobs = 0, n_requests = 0;
   std::string error;                                     // first failure on the thread
+  // How good the requests for each destination layer have been (optional; off = every request goes out as
+  // ranked, which is what the reference does): the share of a request's experts that the layer then routed to,
+  // as a moving average per destination layer.  A request for a layer whose average is below min_precision goes
+  // out empty (the layer's progress count stays in step, nothing is copied): a wrong prefetch costs a copy on the
+  // host link and evicts an expert that may be needed, so below about one half it loses more than it hides.
+  float min_precision = 0.f;
+  std::vector<float> precision;                          // [L], starts at 1
+  std::vector<std::vector<int64_t>> last_pred;           // [L]: the ranking made for the layer's next turn
+  uint64_t n_withheld = 0;
 };
 
 // predictor.cpp:8-46
@@ -76,6 +85,8 @@ static PredictorState *state_of(moe_engine *eng) {
     auto *p = new PredictorState();
     p->window = layer_windows(eng->cfg);
     for (auto &w : p->window) p->max_win = std::max(p->max_win, w.second - w.first);
+    p->precision.assign(eng->cfg.num_layer, 1.f);
+    p->last_pred.assign(eng->cfg.num_layer, {});
     eng->pred = p;
   }
   return eng->pred;
@@ -169,6 +180,9 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
         std::partial_sort(order.begin(), order.begin() + n, order.end(),
                           [&](int a, int b) { return s[a] > s[b] || (s[a] == s[b] && a < b); });
         ids.assign(order.begin(), order.begin() + n);
+        std::lock_guard<std::mutex> lk(p->mu);
+        p->last_pred[dst] = ids;                     // scored when the layer reports its routing
+        if (p->min_precision > 0.f && p->precision[dst] < p->min_precision) { n = 0; p->n_withheld++; }
       }
       {  // a copy of this layer still in flight is a leftover of the layer's previous turn and normally over
          // in a moment: give it that moment, so that the new tasks do not queue behind it for nothing
@@ -319,6 +333,37 @@ int moe_predictor_scores_pending(moe_engine *eng, int layer, const int *seq_word
     p->q.push_back(j);
   }
   p->cv.notify_all();
+  return MOE_OK;
+}
+
+void moe_predictor_observe(moe_engine *eng, int layer, const int64_t *ids, int64_t n) {
+  PredictorState *p = eng->pred;
+  if (!p || !p->started || layer < 0 || layer >= (int)p->last_pred.size()) return;
+  std::lock_guard<std::mutex> lk(p->mu);
+  std::vector<int64_t> &pred = p->last_pred[layer];
+  if (pred.empty()) return;
+  int hit = 0;
+  for (int64_t e : pred)
+    for (int64_t i = 0; i < n; ++i)
+      if (ids[i] == e) { ++hit; break; }
+  p->precision[layer] = 0.8f * p->precision[layer] + 0.2f * (float)hit / (float)pred.size();
+  pred.clear();
+}
+
+extern "C" int moe_predictor_set_min_precision(moe_engine *eng, float min_precision) {
+  if (!eng || !(min_precision >= 0.f && min_precision <= 1.f)) { moe_set_error("moe_predictor_set_min_precision: bad argument"); return MOE_EINVAL; }
+  PredictorState *p = state_of(eng);
+  std::lock_guard<std::mutex> lk(p->mu);
+  p->min_precision = min_precision;
+  return MOE_OK;
+}
+
+extern "C" int moe_predictor_precision(moe_engine *eng, float *precision, uint64_t *n_withheld) {
+  if (!eng || !eng->pred) { moe_set_error("moe_predictor_precision: no predictor"); return MOE_ESTATE; }
+  PredictorState *p = eng->pred;
+  std::lock_guard<std::mutex> lk(p->mu);
+  if (precision) for (size_t l = 0; l < p->precision.size(); ++l) precision[l] = p->precision[l];
+  if (n_withheld) *n_withheld = p->n_withheld;
   return MOE_OK;
 }
 

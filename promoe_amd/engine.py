@@ -231,6 +231,18 @@ class PrefetchMngr:
         check(lib.moe_predictor_stats(self._h, C.byref(a), C.byref(b)), "predictor_stats")
         return {"jobs": a.value, "requests": b.value}
 
+    def set_predictor_min_precision(self, t: float):
+        """Requests for a layer whose predictions have lately been right for less than the share t go out empty
+        (0 = never: the reference's behaviour)."""
+        check(lib.moe_predictor_set_min_precision(self._h, float(t)), "set_predictor_min_precision")
+
+    def predictor_precision(self):
+        """(moving average of the predictions' precision per destination layer, requests sent empty so far)"""
+        p = np.zeros(int(self.metas.num_layer), np.float32)
+        n = C.c_uint64()
+        check(lib.moe_predictor_precision(self._h, p.ctypes.data, C.byref(n)), "predictor_precision")
+        return p, n.value
+
     def update_priority(self, p: np.ndarray, starting_layer: int = 0):
         p = np.ascontiguousarray(p, dtype=np.float32)
         check(lib.moe_update_priority(self._h, p.ctypes.data, p.shape[0], starting_layer), "update_priority")
