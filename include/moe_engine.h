@@ -167,9 +167,10 @@ int moe_predictor_stats(moe_engine *eng, uint64_t *n_jobs, uint64_t *n_requests)
  * further layers release).  No counterpart in the reference, whose worker is joined at exit only. */
 int moe_predictor_wait_idle(moe_engine *eng, int timeout_ms);
 /* Requests scored against what the layers then route to.  Every decode step's routing of a layer
- * (moe_report_one_layer) is compared with the ranking the predictor made for that turn; the share of the
- * ranked experts that were routed to is kept as a moving average per destination layer (0.8 old + 0.2 new,
- * starting at 1).  moe_predictor_set_min_precision(t), t in (0, 1]: a request for a layer whose average is below t
+ * (moe_report_one_layer) is compared with the ranking the predictor made for that turn: of the ranked experts
+ * that were not resident when the request was made (the ones it has to copy; a turn whose ranked experts were
+ * all resident is not scored), the share that was routed to, kept as a moving average per destination layer
+ * (0.8 old + 0.2 new, starting at 1).  moe_predictor_set_min_precision(t), t in (0, 1]: a request for a layer whose average is below t
  * goes out EMPTY (as a prefill step's does: the layer's progress count stays in step and nothing is copied)
  * until the average has recovered; the ranking is still made and scored.  t = 0 (the default): every request
  * goes out as ranked, as in the reference (worker.cpp:41-68), whose PredictWorker has no such feedback.

@@ -51,8 +51,8 @@ struct PredictorState {
   uint64_t n_jobs = 0, n_requests = 0;
   std::string error;                                     // first failure on the thread
   // How good the requests for each destination layer have been (optional; off = every request goes out as
-  // ranked, which is what the reference does): the share of a request's experts that the layer then routed to,
-  // as a moving average per destination layer.  A request for a layer whose average is below min_precision goes
+  // ranked, which is what the reference does): of the experts a request would have to copy (ranked, not resident),
+  // the share that the layer then routed to, as a moving average per destination layer.  A request for a layer whose average is below min_precision goes
   // out empty (the layer's progress count stays in step, nothing is copied): a wrong prefetch costs a copy on the
   // host link and evicts an expert that may be needed, so below about one half it loses more than it hides.
   float min_precision = 0.f;
@@ -180,9 +180,18 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
         std::partial_sort(order.begin(), order.begin() + n, order.end(),
                           [&](int a, int b) { return s[a] > s[b] || (s[a] == s[b] && a < b); });
         ids.assign(order.begin(), order.begin() + n);
+        // what this request would copy: the ranked experts that are not resident now.  They are what a wrong
+        // prediction costs (the resident ones cost nothing either way), so they are what the layer's routing is
+        // scored against - the ranking as a whole looks good whenever the popular experts are resident.
+        std::vector<int64_t> would_copy;
+        {
+          std::lock_guard<std::mutex> lk(eng->mu);
+          for (int64_t e : ids)
+            if (!eng->resident.count(eng->ex(dst, (int)e))) would_copy.push_back(e);
+        }
         std::lock_guard<std::mutex> lk(p->mu);
-        p->last_pred[dst] = ids;                     // scored when the layer reports its routing
-        if (p->min_precision > 0.f && p->precision[dst] < p->min_precision) { n = 0; p->n_withheld++; }
+        p->last_pred[dst] = would_copy;              // scored when the layer reports its routing
+        if (p->min_precision > 0.f && p->precision[dst] < p->min_precision && !would_copy.empty()) { n = 0; p->n_withheld++; }
       }
       {  // a copy of this layer still in flight is a leftover of the layer's previous turn and normally over
          // in a moment: give it that moment, so that the new tasks do not queue behind it for nothing
