@@ -203,6 +203,15 @@ int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k,
                           void *y_bf16, void *stream);
 
 
+/* One token, an expert whose copy landed after the step's routing launch (moe_decode_token_int4 with phase bit
+ * 0 skipped it and published its unit with slot address 0): w13 + SwiGLU of that one unit, h_r row `pos` (the
+ * unit's position in the step's unit list), and the unit's slot address written into unit_ws[pos], so that a
+ * following moe_decode_token_int4 with phase bit 2 (w2 + combine over all units) finds it.  The cache's
+ * counterpart in the reference: the per-expert forward between report_one_expert and one_expert_done
+ * (utils/__init__.py:89-95). */
+int moe_decode_token_late_expert_int4(const void *x_bf16, int H, int I, uint64_t slot_addr, int pos, void *h_r,
+                                      void *unit_ws, int *err, void *stream);
+
 /* k1a + k1b + k2 + k3 for ONE token: moe_decode_token_int4 whose launch of phase bit 0 also computes the gate
  * logits, so a decode step is two launches (this one, then w2 + combine) instead of three.  The first
  * ceil(n_gate_rows / 4) workgroups sum the gate rows (a wave per row, the summation order of moe_gate_logits:

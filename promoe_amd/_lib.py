@@ -60,6 +60,7 @@ _sig("moe_noalloc_scratch_bytes", [], i64)
 _sig("moe_decode_token_int4_noalloc", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp])
 _sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])
 _sig("moe_gate_ws_bytes", [], i64)
+_sig("moe_decode_token_late_expert_int4", [vp, i32, i32, u64, i32, vp, vp, vp, vp])
 _sig("moe_decode_token_int4_gate", [vp, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 +
      [vp, vp, vp, i32, i32, vp, vp, vp])
 _sig("moe_predictor_windows", [vp, vp, vp])

@@ -476,12 +476,21 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       eng->ctr.ready += (uint64_t)now_ids.size();
     }
     guard.release();
-    // with every selected expert resident the launch above was the whole layer; otherwise the w2 pass goes out
-    // again without the combine (the w13 kernel is still running) and leaves partial rows for the experts
-    // computed below and the combine after them
+    // With every selected expert resident the launch above was the whole layer.  Otherwise the late experts
+    // follow as their copies land: each one's w13 launch alone (it also writes the expert's slot address into the
+    // step's published unit list), then w2 over ALL units with the combine in one launch, which overwrites what the
+    // speculative launch left in y.  That needs every late expert in a slot of its own until the last launch
+    // (they stay `launching` till then): only when the layer's slot group has room for that; else the w2 pass
+    // goes out again without the combine, every late expert runs w13 and w2 and is released at once, and the
+    // combine closes the layer (three more launches per step instead of one per late expert plus one).
     const bool w2c = later.empty() && spec_w2c;
     if (spec_w2c) s->spec_state[sw] = later.empty() ? 1 : 2;
-    if (!w2c &&
+    bool late_w13_only = false;
+    if (!w2c && spec_w2c) {
+      std::lock_guard<std::mutex> lk(eng->mu);
+      late_w13_only = later.size() + now_ids.size() <= eng->group_of(layer).full_len;
+    }
+    if (!w2c && !late_w13_only &&
         (rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
@@ -496,6 +505,17 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     s->sub_cursor = 0;
     for (int64_t id : later) {
       if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
+      if (late_w13_only) {
+        uint64_t addr = 0;
+        {
+          std::lock_guard<std::mutex> lk(eng->mu);
+          addr = eng->h_table[(size_t)layer * E + id];
+        }
+        if ((rc = moe_decode_token_late_expert_int4(x, d.H, d.I, addr, unit_of[(int)id].row0, s->h_r, s->unit_ws,
+                                                    s->err_host + layer, st)))
+          return rc;
+        continue;   // still `launching`: the w2 + combine launch below reads its slot too
+      }
       moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
       *slot_h = unit_of[(int)id];
       // (an int4 decode launch of one unit takes the unit and its slot address in the kernel arguments: no device
@@ -505,8 +525,17 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       s->sub_cursor++;
       if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
     }
-    if (!w2c &&
-        (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
+    if (late_w13_only) {
+      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+                                      d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
+                                      s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                                      s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws,
+                                      nullptr, nullptr, 0, 4, sgo, y, st)))
+        return rc;
+      for (int64_t id : later)
+        if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
+    } else if (!w2c &&
+               (rc = moe_combine(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, st)))
       return rc;
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);

@@ -1099,6 +1099,10 @@ __global__ __launch_bounds__(256, (TMAX == 1 ? 3 : 2)) void k_gemv_int4(const Ge
     if (tid == 0 && wk.b == 0) moe_raise_err(a.err);  // one store per missing unit (the word may be host memory)
     return;
   }
+  // a unit that travels by value and arrived late (its copy landed after the step's routing launch had published
+  // the unit list with slot address 0): its address goes into the published list, for the w2 + combine launch
+  if (!DEVUNITS && SWIGLU && a.r_kunits && blockIdx.x == (unsigned)a.n_sh_blocks && tid == 0)
+    a.r_kunits[row0].base = (unsigned long long)base;
   // Gt groups per row block in memory; this workgroup reduces over the window [g0, g0 + G) of them (the whole
   // row unless the class is split: then `split` of c.ksplit workgroups share a block pair)
   const int Gt = c.G;
@@ -2601,6 +2605,25 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
     if (rc) return rc;
   }
   return MOE_OK;
+}
+
+extern "C" int moe_decode_token_late_expert_int4(const void *x, int H, int I, uint64_t slot_addr, int pos, void *h_r,
+                                                 void *unit_ws, int *err, void *stream) {
+  if (!x || !h_r || !unit_ws || !err || !slot_addr || pos < 0 || H <= 0 || H % 128 || I <= 0 || I % 128) {
+    moe_set_error("moe_decode_token_late_expert_int4: bad argument (H=%d I=%d pos=%d)", H, I, pos);
+    return MOE_EINVAL;
+  }
+  moe_int4_layout lr;
+  if (moe_int4_layout_make(H, I, &lr)) return MOE_EINVAL;
+  GemvArgs a;
+  memset(&a, 0, sizeof a);
+  a.T = 1; a.err = err;
+  a.ku[0].base = slot_addr; a.ku[0].m = 1; a.ku[0].row0 = pos;
+  a.r_kunits = (KUnit *)unit_ws;
+  a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, nullptr, 0, 0, 0, H, H / 128, 0, 0, 0, 0};
+  a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, 0, I, I / 16, 0};
+  a.n_sh_blocks = 0;
+  return launch_gemv_t<true>(a, I / 16, 1, H, H / 128, (hipStream_t)stream);
 }
 
 template <int CH>

@@ -15,6 +15,7 @@ STUB(moe_experts_decode_int4)
 STUB(moe_experts_decode_int4_publish)
 STUB(moe_decode_token_int4)
 STUB(moe_decode_token_int4_gate)
+STUB(moe_decode_token_late_expert_int4)
 STUB(moe_experts_decode_q4k)
 STUB(moe_experts_prefill)
 STUB(moe_experts_prefill_pieces)
