@@ -111,7 +111,10 @@ typedef __amdgpu_buffer_rsrc_t pf_rsrc_t;
 // their global address accordingly; the LDS side of the transfer is fixed (lane l writes 16 bytes at 16 l).
 // All addresses are buffer addresses (lane offset in a register that never changes, slab offset in a scalar):
 // with one wave per SIMD every vector instruction that is not a product is issue time taken from the products.
-template <int NB>
+// NTW: the weight fragments are read with the non-temporal hint (a routed expert's tile is the only reader of
+// its fragments: they only pass through the caches); the shared expert's row tiles all read the same fragments
+// and those are requested with plain loads, so that the second-level cache keeps them for the next row tile
+template <int NB, bool NTW>
 static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsigned lds_base, const pf_i32x4_t ra_rsrc,
                                                     const int (&a_voff)[8], const pf_rsrc_t rb, int b_delta1, int nk, int rot0,
                                                     int rot1, int tid) {
@@ -171,8 +174,8 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsign
       for (int n = 0; n < NL; ++n)
         if (n * NS / NL == g) {  // request n of this step goes out behind product group g
           if (n < NB) dma(n, kt + 3, (S + 3) % PF4_RING);
-          else if (n - NB < 4) far[0][n - NB] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB), sb0, 2);
-          else far[1][n - NB - 4] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB - 4), sb1, 2);
+          else if (n - NB < 4) far[0][n - NB] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB), sb0, NTW ? 2 : 0);
+          else far[1][n - NB - 4] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * (n - NB - 4), sb1, NTW ? 2 : 0);
         }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -184,9 +187,9 @@ static __device__ __forceinline__ void pf_mainloop(f32x16_t (&acc)[8][2], unsign
   auto gloadB = [&](u32x4_t(&b)[2][4], int kt) {
     const int sb0 = bslab(kt, rot0), sb1 = bslab(kt, rot1) + b_delta1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[0][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb0, 2);
+    for (int j = 0; j < 4; ++j) b[0][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb0, NTW ? 2 : 0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) b[1][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb1, 2);
+    for (int j = 0; j < 4; ++j) b[1][j] = __builtin_amdgcn_raw_buffer_load_b128(rb, b_voff + 1024 * j, sb1, NTW ? 2 : 0);
   };
 #pragma unroll
   for (int t = 0; t < 3; ++t) {
@@ -274,16 +277,19 @@ __global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
   const int rot0 = (int)((unsigned)(G0 * c.slab_step) % (unsigned)nk), rot1 = (int)((unsigned)(G1 * c.slab_step) % (unsigned)nk);
   const int nb = (tile.rows + 31) >> 5;  // live row blocks (uniform for the workgroup)
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint16_t *)As;
-  switch (nb) {
-    case 1: pf_mainloop<1>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 2: pf_mainloop<2>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 3: pf_mainloop<3>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 4: pf_mainloop<4>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 5: pf_mainloop<5>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 6: pf_mainloop<6>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    case 7: pf_mainloop<7>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
-    default: pf_mainloop<8>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break;
+#define PF_LOOPS(NTW_)                                                                                          \
+  switch (nb) {                                                                                             \
+    case 1: pf_mainloop<1, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 2: pf_mainloop<2, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 3: pf_mainloop<3, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 4: pf_mainloop<4, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 5: pf_mainloop<5, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 6: pf_mainloop<6, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    case 7: pf_mainloop<7, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
+    default: pf_mainloop<8, NTW_>(acc, lds_base, ra_rsrc, a_voff, rb, b_delta1, nk, rot0, rot1, tid); break; \
   }
+  if (c.m_fastest) { PF_LOOPS(false) } else { PF_LOOPS(true) }   // (m_fastest: the shared expert's class)
+#undef PF_LOOPS
   // epilogue.  acc element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l%32
   const int col = 32 * w + (lane & 31);
 #pragma unroll
