@@ -1846,8 +1846,12 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 //     are in flight while the current ones are worked on;
 //   * NT = 2: two 16-token column blocks per pass share every dequantised weight tile.
 // ---------------------------------------------------------------------------
-template <bool SWIGLU, bool DEVUNITS, int NT, int CG, int KS>
-__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
+// One pass of the chunked-K form: rows row_first .. row_first + mc - 1 (mc <= 16 NT) of one unit against the block
+// pair b of its matrix.  Every thread of the workgroup takes part (barriers inside).
+template <bool SWIGLU, int NT, int CG, int KS>
+static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char *smem, const rsrc_t rq, const rsrc_t rs,
+                                               const rsrc_t rz, const rsrc_t rx, const int b, const int row_first,
+                                               const int mc, const Q4Consts &q4c) {
   constexpr int NB = 2;                // 16-row blocks per wave
   constexpr int GW = CG / KS;          // groups per wave and chunk
   constexpr int WS = GW < 4 ? GW : 4;  // groups per weight step
@@ -1860,131 +1864,139 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   constexpr int NSD = (NSE + 63) / 64;
   static_assert(CG % KS == 0 && GW >= 1 && GW == SPC * WS && (SPC == 1 || SPC == 2) && NPC >= 1, "chunk shape");
   static_assert(4 * NB * NT * 4 * 64 * 4 <= 2 * TBK * XSC, "the partial sums reuse the activation buffers");
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // the thread index is made opaque per pass: what a pass shape derives from it (staging addresses, scale
+  // indices) would otherwise be hoisted out of the caller's loop over passes, for all shapes at once, and
+  // the registers that holds spill
+  int tid_ = threadIdx.x;
+  asm volatile("" : "+v"(tid_));
+  const int tid = tid_, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, qd = lane >> 4;
-  const Q4Consts q4c = q4_consts();
   const int kh = w % KS;  // which part of every chunk this wave takes
-
-  // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
-  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
-  if (publishes && blockIdx.x == 0) {
-    gemv_publish_units(a);
-    return;
-  }
-  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
-  const GemvClass &c = wk.c;
-  const int m = wk.m, row0 = wk.row0;
-  const unsigned char *base = wk.base;
-  if (m <= 0) return;
-  if (base == nullptr) {
-    if (tid == 0) moe_raise_err(a.err);
-    return;
-  }
   const int K = c.K, G = c.G;
   unsigned char *xs = smem;                                   // [2][TBK][XSC]
   float *xsum = (float *)(smem + (size_t)2 * TBK * XSC);      // [2][TBK][CG]
   float *sfw = xsum + 2 * TBK * CG + w * (NB * CG * 32);      // this wave's [NB][GW][16 rows][2]
-
-  const int b = wk.b * (4 / KS) + w / KS;  // the wave's block pair
-  const int rbA = 2 * b;
-  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
-  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
-  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
-  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
   const int NCH = (G + CG - 1) / CG;  // activation chunks
   // first group of this wave's weight step i (steps past the end of the reduction are empty;
   // the non-empty ones are a prefix)
   auto step_group = [&](const int i) { return (i / SPC) * CG + kh * GW + (i % SPC) * WS; };
 
-  for (int t0 = 0; t0 < m; t0 += TBK) {
-    const int mc = (m - t0) < TBK ? (m - t0) : TBK;
-    const int row_first = row0 + t0;
-    // byte offset of the activation row behind each of this thread's vectors (rows past the
-    // last token repeat it; they are staged but never read)
-    int xoff[NPC];
+  // byte offset of the activation row behind each of this thread's vectors (rows past the
+  // last token repeat it; they are staged but never read)
+  int xoff[NPC];
+#pragma unroll
+  for (int i = 0; i < NPC; ++i) {
+    const int row = (tid + 256 * i) / XV;
+    const int gr = row_first + (row < mc ? row : mc - 1);
+    xoff[i] = (c.gather ? c.gather[gr] : gr) * c.act_stride * 2;
+  }
+  uint4 xr[NPC];
+  u32 scr[NSD], zr[NSD];
+  // loads of one chunk: activations, this wave's scale dwords and the zero dwords that hold their
+  // nibbles (groups past the end of the reduction: zero activations, zero scales)
+  auto load_chunk = [&](const int ch) {
 #pragma unroll
     for (int i = 0; i < NPC; ++i) {
-      const int row = (tid + 256 * i) / XV;
-      const int gr = row_first + (row < mc ? row : mc - 1);
-      xoff[i] = (c.gather ? c.gather[gr] : gr) * c.act_stride * 2;
+      const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
+      // columns past K: any valid address; chunk_begin zeroes them (a select here would wait for the load)
+      xr[i] = bload16(rx, xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
     }
-    uint4 xr[NPC];
-    u32 scr[NSD], zr[NSD];
-    // loads of one chunk: activations, this wave's scale dwords and the zero dwords that hold their
-    // nibbles (groups past the end of the reduction: zero activations, zero scales)
-    auto load_chunk = [&](const int ch) {
 #pragma unroll
-      for (int i = 0; i < NPC; ++i) {
-        const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
-        // columns past K: any valid address; chunk_begin zeroes them (a select here would wait for the load)
-        xr[i] = bload16(rx, xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
-      }
+    for (int i = 0; i < NSD; ++i) {
+      const int e = lane + 64 * i;
+      const int n = e / (GW * 8), g = ch * CG + kh * GW + ((e % (GW * 8)) >> 3), j = e & 7;
+      const bool ok = e < NSE && g < G;
+      scr[i] = bload4(rs, ok ? ((n * G + g) * 8 + j) * 4 : 0x7ffffff0, 0);
+      zr[i] = bload4(rz, ok ? (n * G + g) * 8 + (j >> 2) * 4 : 0x7ffffff0, 0);
+    }
+  };
+  auto load_w = [&](const int i, uint4 (&wt_)[WS][NB]) {
+    const int g0 = step_group(i);
 #pragma unroll
-      for (int i = 0; i < NSD; ++i) {
-        const int e = lane + 64 * i;
-        const int n = e / (GW * 8), g = ch * CG + kh * GW + ((e % (GW * 8)) >> 3), j = e & 7;
-        const bool ok = e < NSE && g < G;
-        scr[i] = bload4(rs, ok ? ((n * G + g) * 8 + j) * 4 : 0x7ffffff0, 0);
-        zr[i] = bload4(rz, ok ? (n * G + g) * 8 + (j >> 2) * 4 : 0x7ffffff0, 0);
-      }
-    };
-    auto load_w = [&](const int i, uint4 (&wt_)[WS][NB]) {
-      const int g0 = step_group(i);
+    for (int j = 0; j < WS; ++j) {
+      const int g = g0 + j < G ? g0 + j : G - 1;
 #pragma unroll
-      for (int j = 0; j < WS; ++j) {
-        const int g = g0 + j < G ? g0 + j : G - 1;
+      // (plain loads here: popular experts take several passes at 32 and 64 tokens and find their tiles in the caches;
+      // marked non-temporal, a 64-token step took 128.8 instead of 126.9 us)
+      for (int n = 0; n < NB; ++n) wt_[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
+    }
+  };
+  f32x4_t acc[NB][NT];
 #pragma unroll
-        // (plain loads here: popular experts take several passes at 32 and 64 tokens and find their tiles in the caches;
-        // marked non-temporal, a 64-token step took 128.8 instead of 126.9 us)
-        for (int n = 0; n < NB; ++n) wt_[j][n] = bload16(rq, lane * 16, (n * G + g) * 1024);
-      }
-    };
-    f32x4_t acc[NB][NT];
+  for (int n = 0; n < NB; ++n)
 #pragma unroll
-    for (int n = 0; n < NB; ++n)
+    for (int t = 0; t < NT; ++t) acc[n][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  int tokl[NT];  // lanes past the last token repeat it (their columns are not stored)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) acc[n][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    int tokl[NT];  // lanes past the last token repeat it (their columns are not stored)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) tokl[t] = 16 * t + r < mc ? 16 * t + r : mc - 1;
+  for (int t = 0; t < NT; ++t) tokl[t] = 16 * t + r < mc ? 16 * t + r : mc - 1;
 
-    // registers -> LDS for chunk ch, barrier, then the next chunk's loads
-    auto chunk_begin = [&](const int ch) {
-      const int cb = ch & 1;
+  // registers -> LDS for chunk ch, barrier, then the next chunk's loads
+  auto chunk_begin = [&](const int ch) {
+    const int cb = ch & 1;
 #pragma unroll
-      for (int i = 0; i < NPC; ++i) {
-        const int p = tid + 256 * i;
-        const int row = p / XV, v = p & (XV - 1);
-        const uint4 xq = (ch * XV + v) * 8 < K ? xr[i] : make_uint4(0u, 0u, 0u, 0u);
-        float ps = sum8_bf16(xq);
-        ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
-        ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
-        *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xq;
-        if ((tid & 15) == 0) xsum[(cb * TBK + row) * CG + (v >> 4)] = ps;
-      }
+    for (int i = 0; i < NPC; ++i) {
+      const int p = tid + 256 * i;
+      const int row = p / XV, v = p & (XV - 1);
+      const uint4 xq = (ch * XV + v) * 8 < K ? xr[i] : make_uint4(0u, 0u, 0u, 0u);
+      float ps = sum8_bf16(xq);
+      ps += __shfl_xor(ps, 1, 64); ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64); ps += __shfl_xor(ps, 8, 64);
+      *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xq;
+      if ((tid & 15) == 0) xsum[(cb * TBK + row) * CG + (v >> 4)] = ps;
+    }
 #pragma unroll
-      for (int i = 0; i < NSD; ++i) {
-        const int e = lane + 64 * i;
-        if (e < NSE) ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
-      }
-      __syncthreads();
-      // unconditional (past the end: clamped addresses, zero scales), so that every iteration issues the
-      // same number of loads and the waits for the prefetched registers can be exact
-      load_chunk(ch + 1);
-    };
-    // this wave's weight step i on the tiles in cur; the next step's tiles go to nxt first
-    auto step = [&](const int i, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
-      const int g0 = step_group(i);
-      load_w(i + 1, nxt);  // unconditional, clamped: see chunk_begin
-      if (g0 >= G) return;
-      const int cb = (i / SPC) & 1;
+    for (int i = 0; i < NSD; ++i) {
+      const int e = lane + 64 * i;
+      if (e < NSE) ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
+    }
+    __syncthreads();
+    // unconditional (past the end: clamped addresses, zero scales), so that every iteration issues the
+    // same number of loads and the waits for the prefetched registers can be exact
+    load_chunk(ch + 1);
+  };
+  // this wave's weight step i on the tiles in cur; the next step's tiles go to nxt first
+  auto step = [&](const int i, uint4 (&cur)[WS][NB], uint4 (&nxt)[WS][NB]) {
+    const int g0 = step_group(i);
+    load_w(i + 1, nxt);  // unconditional, clamped: see chunk_begin
+    if (g0 >= G) return;
+    const int cb = (i / SPC) & 1;
 #pragma unroll
-      for (int j = 0; j < WS; ++j) {
-        if (g0 + j < G) {  // uniform
-          const int gl = (i % SPC) * WS + j;  // group within this wave's part of the chunk
-          const int gq = kh * GW + gl;        // and within the chunk
+    for (int j = 0; j < WS; ++j) {
+      if (g0 + j < G) {  // uniform
+        const int gl = (i % SPC) * WS + j;  // group within this wave's part of the chunk
+        const int gq = kh * GW + gl;        // and within the chunk
+        if constexpr (NT >= 4) {
+          // wide passes: the dequantised tiles of both blocks stay in registers and the token blocks pass by
+          // (32 + 16 registers live, where activations-first holds 16 NT + 16)
+          bf16x8_t wd[NB][4];
+          float4 f0[NB], f1[NB];
+#pragma unroll
+          for (int n = 0; n < NB; ++n) {
+            wd[n][0] = deq8_bf16(cur[j][n].x, q4c); wd[n][1] = deq8_bf16(cur[j][n].y, q4c);
+            wd[n][2] = deq8_bf16(cur[j][n].z, q4c); wd[n][3] = deq8_bf16(cur[j][n].w, q4c);
+            const float4 *sf = (const float4 *)(sfw + ((n * GW + gl) * 16 + 4 * qd) * 2);
+            f0[n] = sf[0]; f1[n] = sf[1];
+          }
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const uint4 *xp = (const uint4 *)(xs + ((size_t)cb * TBK + tokl[t]) * XSC + gq * 256 + qd * 64);
+            const bf16x8_t x0 = as_bf16x8(xp[0]), x1 = as_bf16x8(xp[1]), x2 = as_bf16x8(xp[2]), x3 = as_bf16x8(xp[3]);
+            const float xg = xsum[(cb * TBK + tokl[t]) * CG + gq];
+#pragma unroll
+            for (int n = 0; n < NB; ++n) {
+              f32x4_t d = f32x4_t{0.f, 0.f, 0.f, 0.f};
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[n][0], x0, d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[n][1], x1, d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[n][2], x2, d, 0, 0, 0);
+              d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wd[n][3], x3, d, 0, 0, 0);
+              acc[n][t][0] = fmaf(f0[n].x, d[0], fmaf(f0[n].y, xg, acc[n][t][0]));
+              acc[n][t][1] = fmaf(f0[n].z, d[1], fmaf(f0[n].w, xg, acc[n][t][1]));
+              acc[n][t][2] = fmaf(f1[n].x, d[2], fmaf(f1[n].y, xg, acc[n][t][2]));
+              acc[n][t][3] = fmaf(f1[n].z, d[3], fmaf(f1[n].w, xg, acc[n][t][3]));
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);  // keeps the next group's dequantisation out of this one's registers
+        } else {
           bf16x8_t xv[NT][4];
           float xg[NT];
 #pragma unroll
@@ -2016,77 +2028,129 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
           }
         }
       }
-    };
+    }
+  };
 
-    uint4 wA[WS][NB], wB[WS][NB];
-    load_chunk(0);
-    load_w(0, wA);
-    if constexpr (SPC == 2) {
-      for (int ch = 0; ch < NCH; ++ch) {
-        chunk_begin(ch);
-        step(2 * ch, wA, wB);
-        step(2 * ch + 1, wB, wA);
-      }
-    } else {
-      for (int ch = 0; ch < NCH; ch += 2) {
-        chunk_begin(ch);
-        step(ch, wA, wB);
-        if (ch + 1 < NCH) {
-          chunk_begin(ch + 1);
-          step(ch + 1, wB, wA);
-        }
+  uint4 wA[WS][NB], wB[WS][NB];
+  load_chunk(0);
+  load_w(0, wA);
+  if constexpr (SPC == 2) {
+    for (int ch = 0; ch < NCH; ++ch) {
+      chunk_begin(ch);
+      step(2 * ch, wA, wB);
+      step(2 * ch + 1, wB, wA);
+    }
+  } else {
+    for (int ch = 0; ch < NCH; ch += 2) {
+      chunk_begin(ch);
+      step(ch, wA, wB);
+      if (ch + 1 < NCH) {
+        chunk_begin(ch + 1);
+        step(ch + 1, wB, wA);
       }
     }
-    if constexpr (KS > 1) {
-      // the sums of a pair's waves meet in the activation buffers (free once every wave is done with them)
-      __syncthreads();
-      float *red = (float *)smem;  // [4 waves][NB][NT][4][64 lanes]
-      if (kh != 0) {
+  }
+  if constexpr (KS > 1) {
+    // the sums of a pair's waves meet in the activation buffers (free once every wave is done with them)
+    __syncthreads();
+    float *red = (float *)smem;  // [4 waves][NB][NT][4][64 lanes]
+    if (kh != 0) {
+#pragma unroll
+      for (int n = 0; n < NB; ++n)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) red[((w * NB + n) * NT + t) * 256 + i * 64 + lane] = acc[n][t][i];
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int q = 1; q < KS; ++q)
 #pragma unroll
         for (int n = 0; n < NB; ++n)
 #pragma unroll
           for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[((w * NB + n) * NT + t) * 256 + i * 64 + lane] = acc[n][t][i];
-      }
-      __syncthreads();
-      if (kh == 0) {
+            for (int i = 0; i < 4; ++i) acc[n][t][i] += red[(((w + q) * NB + n) * NT + t) * 256 + i * 64 + lane];
+    }
+  }
+  // every lane holds 4 consecutive rows of both blocks for one token per column block
+  if (kh == 0) {
 #pragma unroll
-        for (int q = 1; q < KS; ++q)
+    for (int t = 0; t < NT; ++t) {
+      if (16 * t + r < mc) {
+        const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
+        if (SWIGLU) {
+          u32 h[2];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
+            const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
+            const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
+            h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
+          }
+          *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
+        } else {
 #pragma unroll
           for (int n = 0; n < NB; ++n)
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) acc[n][t][i] += red[(((w + q) * NB + n) * NT + t) * 256 + i * 64 + lane];
-      }
-    }
-    // every lane holds 4 consecutive rows of both blocks for one token per column block
-    if (kh == 0) {
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        if (16 * t + r < mc) {
-          const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
-          if (SWIGLU) {
-            u32 h[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-              const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
-              const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
-              const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
-              h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
-            }
-            *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
-          } else {
-#pragma unroll
-            for (int n = 0; n < NB; ++n)
-              *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
-                  make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
-          }
+            *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
+                make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
         }
       }
     }
-    if (t0 + TBK < m) __syncthreads();  // the next pass restages chunk buffer 0
+  }
+}
+
+// The kernel: a workgroup walks the rows of its unit in passes and picks every pass's width by the rows that are
+// left: 64 rows (NT = 4, chunks of 2 groups) when more than 32 remain, 32 rows (NT = 2, chunks of 4) when more
+// than 16 remain, else 16 rows (chunks of 8), as far as NTMAX allows.  The three shapes stage the same number of
+// activation bytes per chunk, so the LDS footprint is that of the 16-row shape.  A unit's weights are streamed and
+// dequantised once per pass, so a popular expert (and the shared expert, which sees every token) costs one stream
+// where 16-row passes cost up to four.
+template <bool SWIGLU, bool DEVUNITS, int NTMAX, int KS>
+__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
+  constexpr int NB = 2;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const Q4Consts q4c = q4_consts();
+
+  // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
+  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
+  if (publishes && blockIdx.x == 0) {
+    gemv_publish_units(a);
+    return;
+  }
+  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
+  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
+  const GemvClass &c = wk.c;
+  const int m = wk.m, row0 = wk.row0;
+  const unsigned char *base = wk.base;
+  if (m <= 0) return;
+  if (base == nullptr) {
+    if (tid == 0) moe_raise_err(a.err);
+    return;
+  }
+  const int G = c.G;
+  const int b = wk.b * (4 / KS) + w / KS;  // the wave's block pair
+  const int rbA = 2 * b;
+  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
+  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
+  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
+
+  for (int t0 = 0; t0 < m;) {
+    const int left = m - t0;
+    if (NTMAX >= 4 && left > 32) {
+      kc_pass<SWIGLU, 4, 2, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 64 ? left : 64, q4c);
+      t0 += 64;
+    } else if (NTMAX >= 2 && left > 16) {
+      kc_pass<SWIGLU, 2, 4, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 32 ? left : 32, q4c);
+      t0 += 32;
+    } else {
+      kc_pass<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 16 ? left : 16, q4c);
+      t0 += 16;
+    }
+    if (t0 < m) __syncthreads();  // the next pass restages chunk buffer 0
   }
 }
 
@@ -2431,7 +2495,7 @@ static size_t gemv_mfma_kc_lds(int nt, int cg) {
 
 // chunked-K form: a workgroup takes 4 / KS block pairs of a unit (both classes' pair counts are
 // multiples of four: I and H are multiples of 128)
-template <bool SW, int NT, int CG, int KS>
+template <bool SW, int NTMAX, int KS>
 static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t s) {
   constexpr int PW = 4 / KS;
   GemvArgs a = a_in;
@@ -2443,13 +2507,15 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
   a.cls[1].nblk /= PW;
   const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
-  const size_t lds = gemv_mfma_kc_lds(NT, CG);
+  size_t lds = gemv_mfma_kc_lds(1, 8);  // the widest of the pass shapes the kernel may pick
+  if (NTMAX >= 2 && gemv_mfma_kc_lds(2, 4) > lds) lds = gemv_mfma_kc_lds(2, 4);
+  if (NTMAX >= 4 && gemv_mfma_kc_lds(4, 2) > lds) lds = gemv_mfma_kc_lds(4, 2);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NT, CG, KS>,
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NTMAX, KS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NT, CG, KS>,
+      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NTMAX, KS>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
@@ -2458,8 +2524,8 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NT, CG, KS>), dim3(grid), dim3(256), lds, s, a);
-  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NT, CG, KS>), dim3(grid), dim3(256), lds, s, a);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NTMAX, KS>), dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NTMAX, KS>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4_mfma_kc");
 }
@@ -2468,10 +2534,10 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
 // unit slot in use; the unit list is made on the device, the host only knows its capacity), else one.
 // Measured: 256 workgroups (4096 x 14336 w2, 8 units) 101 us with one wave per pair, 77 us with two; 484
 // workgroups (2048 x 1408 w13, 20 units) 19.5 us against 25.7 us.  Four never paid.
-template <bool SW, int NT, int CG>
+template <bool SW, int NTMAX>
 static int launch_gemv_mfma_kc(const GemvArgs &a, int grid, hipStream_t s) {
-  if (grid / 4 >= 384) return launch_gemv_mfma_kc_ks<SW, NT, CG, 1>(a, grid, s);
-  return launch_gemv_mfma_kc_ks<SW, NT, CG, 2>(a, grid, s);
+  if (grid / 4 >= 384) return launch_gemv_mfma_kc_ks<SW, NTMAX, 1>(a, grid, s);
+  return launch_gemv_mfma_kc_ks<SW, NTMAX, 2>(a, grid, s);
 }
 
 template <bool SW>
@@ -2491,8 +2557,9 @@ static int launch_gemv_t(const GemvArgs &a, int grid, int T, int Kmax, int G_rou
     // above 48 tokens - at 40 and 48 they tie on the first shape and lose 128 to 85 us on the second -,
     // the w13 pass only under skewed routing)
     if (T >= 16 || !whole_rows_fit) {
-      if (!SW && T > 48) return launch_gemv_mfma_kc<SW, 2, 4>(a, grid, s);
-      return launch_gemv_mfma_kc<SW, 1, 8>(a, grid, s);
+      if (T > 32) return launch_gemv_mfma_kc<SW, 4>(a, grid, s);
+      if (T > 16) return launch_gemv_mfma_kc<SW, 2>(a, grid, s);
+      return launch_gemv_mfma_kc<SW, 1>(a, grid, s);
     }
     int tb = 1;
     while (tb < T && tb < 16) tb <<= 1;

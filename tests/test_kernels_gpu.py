@@ -195,11 +195,13 @@ def test_decode_layer_small_variants(cuda):
     check_layer(Int4Layer(H=384, I=640, E=4, I_sh=128, seed=6), 3, 2, 0, cuda)
 
 
-@pytest.mark.parametrize("T", [3, 16, 20, 40, 64, 70])
+@pytest.mark.parametrize("T", [3, 16, 20, 33, 40, 50, 64, 70])
 def test_decode_layer_long_reduction(cuda, T):
     """Reductions longer than 2048 and batches of more than 16 tokens take the chunked-K GEMV: group counts
-    that leave a partial last chunk and an odd number of weight steps (G = 18, 17, 20), units with more rows
-    than one pass holds (E = 4, k = 2: about T / 2 rows per unit), 32-token passes in w2 above 48 tokens."""
+    that leave a partial last chunk and an odd number of weight steps (G = 18, 17, 20) in chunks of 8, 4 and
+    2 groups; passes of 16, 32 and 64 rows picked per unit by the rows it has left (E = 4, k = 2: about T / 2
+    rows per routed unit, T rows for the shared expert: 33 = one partial 64-row pass, 70 = a 64-row pass and
+    a 16-row pass, 20 and 40 = partial 32-row passes)."""
     print(f"case decode_long_reduction T={T}", flush=True)
     layer = Int4Layer(H=2304, I=2176, E=4, I_sh=2560, seed=8)
     check_layer(layer, T, 2, 0, cuda)
