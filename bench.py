@@ -332,7 +332,7 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
             "us_per_layer": t_layer * 1e6, "distinct_routed_experts_per_step": D,
             "algorithmic_bytes_per_step": step_bytes, "layer_GBps": step_bytes / t_layer / 1e9,
             "roofline": {"bound": "hbm", "kernel": ("k_prefill_int4 (w13 + SwiGLU)" if tiles else
-                                                    "k_gemv_int4%s (w13 + SwiGLU)" % ("<q4_K>" if q4k else ("_mfma_kc" if (T > 16 or H > 2048) and T > 1 else ("_mfma" if T > 1 else "")))),
+                                                    "k_gemv_int4%s (w13 + SwiGLU)" % (("_mfma_kc<q4_K>" if T > 1 else "<q4_K>") if q4k else ("_mfma_kc" if (T > 16 or H > 2048) and T > 1 else ("_mfma" if T > 1 else "")))),
                          "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
                          "algorithmic_bytes_per_launch": w13_bytes, "avg_launch_us": t_w13 * 1e6,
                          "method": w13_method}}
@@ -348,6 +348,8 @@ def other_configs(torch):
                               steps=60 if T == 1 else 20))
     out.append(decode_leg(torch, "Qwen2-57B-A14B-shaped layer, q4_K experts, decode T=3 (three sequences), all "
                           "resident, Zipf(1.1)", L.FMT_Q4K, 3, 3584, 64, 2560, 8, 20480, True, 0, 3, 1.1, steps=60))
+    out.append(decode_leg(torch, "Qwen2-57B-A14B-shaped layer, q4_K experts, decode T=32, all resident, Zipf(1.1)",
+                          L.FMT_Q4K, 32, 3584, 64, 2560, 8, 20480, True, 0, 3, 1.1, steps=30))
     return out
 
 

@@ -175,12 +175,14 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, (uint16_t **)&s->h_r, P * I);
   rc |= dalloc(s, (uint16_t **)&s->h_s, (size_t)T * I_sh);
   rc |= dalloc(s, &s->part_r, P * H);
-  // q4_K decode batches (at most 16 tokens) may leave the shared expert's partial rows in up to 8 pieces, and so
+  // q4_K decode batches (at most 64 tokens) may leave the shared expert's partial rows in up to 8 pieces, and so
   // may a prefill batch of a nibble format whose shared expert is wide (pieces x tokens rows, largest over the
   // batch sizes the workspace admits)
   size_t rows_s = T > 128 ? T : 128;
-  for (int t = 1; t <= T; ++t)
+  for (int t = 1; t <= T; ++t) {
     rows_s = std::max(rows_s, (size_t)t * (size_t)moe_prefill_shared_splits(MOE_FMT_Q4K, t, H, I_sh));
+    if (t <= 64) rows_s = std::max(rows_s, (size_t)t * (size_t)moe_decode_shared_splits(MOE_FMT_Q4K, t, H, I_sh));
+  }
   rc |= dalloc(s, &s->part_s, rows_s * H);
   s->part_s_elems = rows_s * H;
   rc |= dalloc(s, (unsigned char **)&s->tiles_ws, (size_t)moe_prefill_workspace_bytes(T, k, s->max_units));
@@ -254,11 +256,11 @@ int moe_forward_harvest(moe_engine *eng, bool wait) {
 // go to the matrix-core tile kernels, decode batches to the bandwidth-bound GEMV kernels.
 static bool use_prefill(const moe_layer_desc &d, int T) {
   if (d.fmt == MOE_FMT_BF16) return true;
-  // int4-g128: up to 64 tokens the grouped launch is bound by the weight stream and the GEMV kernels
-  // (operand 128 + q, scale and zero applied after the products) stream it faster than the tile kernels,
-  // which dequantise every weight completely (measured on the 2048 x 1408 and 4096 x 14336 shapes)
-  const int gemv_tmax = d.fmt == MOE_FMT_INT4_G128 ? 64 : 16;
-  return T > gemv_tmax && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
+  // nibble formats: up to 64 tokens the grouped launch is bound by the weight stream, and the decode kernels
+  // (a workgroup streams four block pairs of a unit over the whole reduction, 16 to 64 token rows per pass)
+  // stream it faster than the tile kernels, whose tiles are short at these batch sizes (measured on the
+  // 2048 x 1408 and 4096 x 14336 int4 shapes and the 3584 x 2560 q4_K shape)
+  return T > 64 && d.H % 256 == 0 && d.I % 128 == 0 && d.I_sh % 128 == 0;
 }
 
 static int shared_pieces(const moe_layer_desc &d, int T, const LayerState *s);

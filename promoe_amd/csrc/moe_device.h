@@ -119,3 +119,46 @@ static __device__ __forceinline__ u32 bload1(rsrc_t r, int voff, int soff) {
   return (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(r, voff, soff, 0);
 }
 
+// ---------------------------------------------------------------------------
+// fp16 operands for the matrix cores from nibble formats (int4-g128 and q4_K tile kernels, q4_K decode)
+// ---------------------------------------------------------------------------
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+static __device__ __forceinline__ u32 bf16x2_to_f16x2(u32 d) {
+  // both halves are bf16; fp16 has more mantissa bits, so round-to-zero conversion is exact
+  auto h = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(d << 16), __uint_as_float(d & 0xffff0000u));
+  return __builtin_bit_cast(u32, h);
+}
+// Dequantisation of 8 nibbles of a dword into 8 fp16 weights with ONE packed fma per pair: a nibble is masked into
+// mantissa bits 6..9 of an fp16 with the exponent of 1.0, which makes the exact value h = 1 + q/16; with S = 16 s and
+// C = -(16 + zero) s (int4) or C = -(16 s + m) (q4_K), both prepared once per group and row, h S + C = (q - zero) s
+// or q s - m.  The product is exact inside the fma; C carries the one extra rounding (2^-11 of at most 31 s, i.e.
+// 0.015 of a quantisation step, a bias common to the 128 weights of a group row).  The form before this one
+// ((h - (1024 + zero)) s with h = 1024 + q) was exact up to the final rounding and cost a packed subtract and
+// a packed multiply per pair (three operations for q4_K), in kernels that are bound by these operations.
+// Mask and exponent pattern are held in vector registers, made once per kernel: (x & M) | C is then ONE
+// v_and_or_b32 (a VOP3 instruction takes no literal and one scalar operand on this target).
+struct DeqF16Consts { u32 M, C; };
+static __device__ __forceinline__ DeqF16Consts deq_f16_consts() {
+  DeqF16Consts q{0x03c003c0u, 0x3c003c00u};
+  asm volatile("" : "+v"(q.M), "+v"(q.C));
+  return q;
+}
+// s2 / c2: fp16 bit patterns of S and C replicated in both halves
+static __device__ __forceinline__ f16x8_t deq8_f16(u32 d, u32 s2, u32 c2, const DeqF16Consts &q) {
+  const u32 M = q.M, C = q.C;
+  u32x4_t v;
+  v.x = ((d << 6) & M) | C; v.y = ((d << 2) & M) | C; v.z = ((d >> 2) & M) | C; v.w = ((d >> 6) & M) | C;
+  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1 + q/16, exact
+  const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
+  const f16x8_t c8 = __builtin_bit_cast(f16x8_t, u32x4_t{c2, c2, c2, c2});
+  return __builtin_elementwise_fma(h, s8, c8);
+}
+
+static __device__ __forceinline__ u32 h2f_bits(u32 hbits) {  // fp16 bits -> fp32 bits
+  const _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)hbits);
+  return __builtin_bit_cast(u32, (float)h);
+}
+static __device__ __forceinline__ u32 f2h_bits(float f) {  // fp32 -> fp16 bits (round to nearest)
+  return (u32)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+

@@ -1846,6 +1846,11 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 //     are in flight while the current ones are worked on;
 //   * NT = 2: two 16-token column blocks per pass share every dequantised weight tile.
 // ---------------------------------------------------------------------------
+// Length of the activations' buffer resource in the chunked-K kernels, and the offset that stands for "no row": the
+// first byte past it, so that such a load is out of range by any reading of the range rule (first byte or last
+// byte of the access, no 32-bit wrap) and returns zeros without a memory request.
+#define KC_NO_ROW 0x7fffff00u
+
 // One pass of the chunked-K form: rows row_first .. row_first + mc - 1 (mc <= 16 NT) of one unit against the block
 // pair b of its matrix.  Every thread of the workgroup takes part (barriers inside).
 template <bool SWIGLU, int NT, int CG, int KS>
@@ -1881,14 +1886,15 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
   // the non-empty ones are a prefix)
   auto step_group = [&](const int i) { return (i / SPC) * CG + kh * GW + (i % SPC) * WS; };
 
-  // byte offset of the activation row behind each of this thread's vectors (rows past the
-  // last token repeat it; they are staged but never read)
+  // byte offset of the activation row behind each of this thread's vectors (rows past the last token: -1, their
+  // loads go past the end of the buffer resource, which returns zeros and asks the memory for nothing; they are
+  // staged but never read)
   int xoff[NPC];
 #pragma unroll
   for (int i = 0; i < NPC; ++i) {
     const int row = (tid + 256 * i) / XV;
     const int gr = row_first + (row < mc ? row : mc - 1);
-    xoff[i] = (c.gather ? c.gather[gr] : gr) * c.act_stride * 2;
+    xoff[i] = row < mc ? (c.gather ? c.gather[gr] : gr) * c.act_stride * 2 : -1;
   }
   uint4 xr[NPC];
   u32 scr[NSD], zr[NSD];
@@ -1899,7 +1905,7 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
     for (int i = 0; i < NPC; ++i) {
       const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
       // columns past K: any valid address; chunk_begin zeroes them (a select here would wait for the load)
-      xr[i] = bload16(rx, xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
+      xr[i] = bload16(rx, xoff[i] < 0 ? (int)KC_NO_ROW : xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
     }
 #pragma unroll
     for (int i = 0; i < NSD; ++i) {
@@ -2101,18 +2107,227 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
   }
 }
 
+// The same pass over q4_K tiles.  A lane's 32 weights of a tile are one 32-wide sub-block of its row, with its own
+// 6-bit (scale, min) pair under the (d, dmin) of the row's 256-wide super-block, so nothing can be factored out
+// of a group's products: every weight is dequantised completely (d sc q - dmin m, one packed fp16 fma per pair, the
+// arithmetic of the tile kernels for longer batches) and the products accumulate on the matrix cores in fp32.  The
+// activations are staged as fp16 (exact from bf16); no sums of activations are needed.  The (scale, min) pair and
+// the (d, dmin) pair of a tile travel with it, one 2-byte and one 4-byte load per lane.
+// Gt: groups per row block in memory; the pass reduces over the window of G groups that the resources start at.
+template <bool SWIGLU, int NT, int CG, int KS>
+static __device__ __forceinline__ void kc_pass_q4k(const GemvClass &c, unsigned char *smem, const rsrc_t rq,
+                                                   const rsrc_t rs, const rsrc_t rz, const rsrc_t rx, const int Gt,
+                                                   const int G, const int b, const size_t out_row0, const int row_first,
+                                                   const int mc, const DeqF16Consts &dqc) {
+  constexpr int NB = 2, GW = CG / KS, WS = GW < 4 ? GW : 4, SPC = GW / WS, TBK = 16 * NT;
+  constexpr int XSC = CG * 256 + 16, XV = CG * 16, NPC = TBK * XV / 256;
+  static_assert(CG % KS == 0 && GW >= 1 && GW == SPC * WS && (SPC == 1 || SPC == 2) && NPC >= 1, "chunk shape");
+  static_assert(4 * NB * NT * 4 * 64 * 4 <= 2 * TBK * XSC, "the partial sums reuse the activation buffers");
+  int tid_ = threadIdx.x;
+  asm volatile("" : "+v"(tid_));  // see kc_pass
+  const int tid = tid_, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, qd = lane >> 4;
+  const int kh = w % KS;
+  const int K = G * 128;
+  unsigned char *xs = smem;  // [2][TBK][XSC] fp16
+  const int NCH = (G + CG - 1) / CG;
+  auto step_group = [&](const int i) { return (i / SPC) * CG + kh * GW + (i % SPC) * WS; };
+
+  int xoff[NPC];
+#pragma unroll
+  for (int i = 0; i < NPC; ++i) {
+    const int row = (tid + 256 * i) / XV;
+    const int gr = row_first + (row < mc ? row : mc - 1);
+    xoff[i] = row < mc ? (c.gather ? c.gather[gr] : gr) * c.act_stride * 2 : -1;
+  }
+  uint4 xr[NPC];
+  auto load_chunk = [&](const int ch) {
+#pragma unroll
+    for (int i = 0; i < NPC; ++i) {
+      const int kv = ch * XV + ((tid + 256 * i) & (XV - 1));
+      xr[i] = bload16(rx, xoff[i] < 0 ? (int)KC_NO_ROW : xoff[i] + (kv * 8 < K ? kv * 16 : 0), 0);
+    }
+  };
+  struct Tiles { uint4 q[WS][NB]; u32 sm[WS][NB], dd[WS][NB]; };
+  auto load_w = [&](const int i, Tiles &t_) {
+    const int g0 = step_group(i);
+#pragma unroll
+    for (int j = 0; j < WS; ++j) {
+      const int g = g0 + j < G ? g0 + j : G - 1;
+#pragma unroll
+      for (int n = 0; n < NB; ++n) {
+        const int tile = n * Gt + g;
+        t_.q[j][n] = bload16_nt(rq, lane * 16, tile * 1024);
+        t_.sm[j][n] = bload2(rs, lane * 2, tile * 128);
+        t_.dd[j][n] = bload4(rz, r * 4, (tile >> 1) * 64);
+      }
+    }
+  };
+  f32x4_t acc[NB][NT];
+#pragma unroll
+  for (int n = 0; n < NB; ++n)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[n][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  int tokl[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) tokl[t] = 16 * t + r < mc ? 16 * t + r : mc - 1;
+
+  auto chunk_begin = [&](const int ch) {
+    const int cb = ch & 1;
+#pragma unroll
+    for (int i = 0; i < NPC; ++i) {
+      const int p = tid + 256 * i;
+      const int row = p / XV, v = p & (XV - 1);
+      const bool in = (ch * XV + v) * 8 < K;
+      uint4 xq;
+      xq.x = in ? bf16x2_to_f16x2(xr[i].x) : 0u; xq.y = in ? bf16x2_to_f16x2(xr[i].y) : 0u;
+      xq.z = in ? bf16x2_to_f16x2(xr[i].z) : 0u; xq.w = in ? bf16x2_to_f16x2(xr[i].w) : 0u;
+      *(uint4 *)(xs + ((size_t)cb * TBK + row) * XSC + (size_t)v * 16) = xq;
+    }
+    __syncthreads();
+    load_chunk(ch + 1);  // unconditional: see kc_pass
+  };
+  // the 8 fp16 weights behind each dword of a lane's tile row
+  auto deq_tile = [&](const uint4 &q, const u32 sm, const u32 dd, f16x8_t (&wd)[4]) {
+    const float s16 = 16.f * half_bits_to_f32((uint16_t)dd) * (float)(sm & 0xffu);
+    const float cz = -s16 - half_bits_to_f32((uint16_t)(dd >> 16)) * (float)(sm >> 8);
+    const u32 sb = f2h_bits(s16), cb = f2h_bits(cz);
+    const u32 s2 = sb | (sb << 16), c2 = cb | (cb << 16);
+    wd[0] = deq8_f16(q.x, s2, c2, dqc); wd[1] = deq8_f16(q.y, s2, c2, dqc);
+    wd[2] = deq8_f16(q.z, s2, c2, dqc); wd[3] = deq8_f16(q.w, s2, c2, dqc);
+  };
+  auto step = [&](const int i, const Tiles &cur, Tiles &nxt) {
+    const int g0 = step_group(i);
+    load_w(i + 1, nxt);
+    if (g0 >= G) return;
+    const int cb = (i / SPC) & 1;
+#pragma unroll
+    for (int j = 0; j < WS; ++j) {
+      if (g0 + j < G) {  // uniform
+        const int gq = kh * GW + (i % SPC) * WS + j;  // group within the chunk
+        if constexpr (NT >= 4) {
+          f16x8_t wd[NB][4];
+#pragma unroll
+          for (int n = 0; n < NB; ++n) deq_tile(cur.q[j][n], cur.sm[j][n], cur.dd[j][n], wd[n]);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const f16x8_t *xp = (const f16x8_t *)(xs + ((size_t)cb * TBK + tokl[t]) * XSC + gq * 256 + qd * 64);
+            const f16x8_t x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+#pragma unroll
+            for (int n = 0; n < NB; ++n) {
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[n][0], x0, acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[n][1], x1, acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[n][2], x2, acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[n][3], x3, acc[n][t], 0, 0, 0);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          f16x8_t xv[NT][4];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const f16x8_t *xp = (const f16x8_t *)(xs + ((size_t)cb * TBK + tokl[t]) * XSC + gq * 256 + qd * 64);
+            xv[t][0] = xp[0]; xv[t][1] = xp[1]; xv[t][2] = xp[2]; xv[t][3] = xp[3];
+          }
+#pragma unroll
+          for (int n = 0; n < NB; ++n) {
+            f16x8_t wd[4];
+            deq_tile(cur.q[j][n], cur.sm[j][n], cur.dd[j][n], wd);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[0], xv[t][0], acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[1], xv[t][1], acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[2], xv[t][2], acc[n][t], 0, 0, 0);
+              acc[n][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wd[3], xv[t][3], acc[n][t], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+  };
+
+  Tiles wA, wB;
+  load_chunk(0);
+  load_w(0, wA);
+  if constexpr (SPC == 2) {
+    for (int ch = 0; ch < NCH; ++ch) {
+      chunk_begin(ch);
+      step(2 * ch, wA, wB);
+      step(2 * ch + 1, wB, wA);
+    }
+  } else {
+    for (int ch = 0; ch < NCH; ch += 2) {
+      chunk_begin(ch);
+      step(ch, wA, wB);
+      if (ch + 1 < NCH) {
+        chunk_begin(ch + 1);
+        step(ch + 1, wB, wA);
+      }
+    }
+  }
+  if constexpr (KS > 1) {
+    __syncthreads();
+    float *red = (float *)smem;  // [4 waves][NB][NT][4][64 lanes]
+    if (kh != 0) {
+#pragma unroll
+      for (int n = 0; n < NB; ++n)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) red[((w * NB + n) * NT + t) * 256 + i * 64 + lane] = acc[n][t][i];
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int q = 1; q < KS; ++q)
+#pragma unroll
+        for (int n = 0; n < NB; ++n)
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[n][t][i] += red[(((w + q) * NB + n) * NT + t) * 256 + i * 64 + lane];
+    }
+  }
+  if (kh == 0) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (16 * t + r < mc) {
+        if (SWIGLU) {
+          const size_t orow = (size_t)(row_first + 16 * t + r) * c.out_stride;
+          u32 h[2];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const float g0 = acc[0][t][2 * i], g1 = acc[0][t][2 * i + 1];
+            const float h0 = g0 / (1.f + expf(-g0)) * acc[1][t][2 * i];
+            const float h1 = g1 / (1.f + expf(-g1)) * acc[1][t][2 * i + 1];
+            h[i] = (u32)f32_to_bf16(h0) | ((u32)f32_to_bf16(h1) << 16);
+          }
+          *(uint2 *)((uint16_t *)c.out + orow + b * 16 + 4 * qd) = make_uint2(h[0], h[1]);
+        } else {
+          const size_t orow = (out_row0 + (size_t)(row_first + 16 * t + r)) * c.out_stride;
+#pragma unroll
+          for (int n = 0; n < NB; ++n)
+            *(float4 *)((float *)c.out + orow + (2 * b + n) * 16 + 4 * qd) =
+                make_float4(acc[n][t][0], acc[n][t][1], acc[n][t][2], acc[n][t][3]);
+        }
+      }
+    }
+  }
+}
+
 // The kernel: a workgroup walks the rows of its unit in passes and picks every pass's width by the rows that are
 // left: 64 rows (NT = 4, chunks of 2 groups) when more than 32 remain, 32 rows (NT = 2, chunks of 4) when more
 // than 16 remain, else 16 rows (chunks of 8), as far as NTMAX allows.  The three shapes stage the same number of
 // activation bytes per chunk, so the LDS footprint is that of the 16-row shape.  A unit's weights are streamed and
 // dequantised once per pass, so a popular expert (and the shared expert, which sees every token) costs one stream
 // where 16-row passes cost up to four.
-template <bool SWIGLU, bool DEVUNITS, int NTMAX, int KS>
+// q4_K: the shared expert's w2 class may be split (c.ksplit workgroups per group of block pairs, each over 1 / ksplit
+// of the reduction, partial rows to their own copy of the output: see k_gemv_int4).
+template <bool SWIGLU, bool DEVUNITS, int NTMAX, int KS, bool Q4K = false>
 __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
   constexpr int NB = 2;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const Q4Consts q4c = q4_consts();
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
   const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
@@ -2130,24 +2345,37 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
     if (tid == 0) moe_raise_err(a.err);
     return;
   }
-  const int G = c.G;
-  const int b = wk.b * (4 / KS) + w / KS;  // the wave's block pair
+  const int Gt = c.G;
+  const int nsp = (Q4K && c.ksplit > 1) ? c.ksplit : 1;
+  const int split = nsp > 1 ? wk.b % nsp : 0;
+  const int G = Gt / nsp, g0 = split * G;   // this workgroup's window of the reduction
+  const int b = (nsp > 1 ? wk.b / nsp : wk.b) * (4 / KS) + w / KS;  // the wave's block pair
   const int rbA = 2 * b;
-  const rsrc_t rq = make_rsrc(base + c.off_q + (size_t)rbA * G * 1024, (u32)NB * G * 1024u);
-  const rsrc_t rs = make_rsrc(base + c.off_s + (size_t)rbA * G * 32, (u32)NB * G * 32u);
-  const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
-  const rsrc_t rx = make_rsrc(c.act, 0x7fffffffu);
+  constexpr int SCB = Q4K ? 128 : 32, ZZB = Q4K ? 32 : 8;  // bytes of section s / z per tile
+  const rsrc_t rq = make_rsrc(base + c.off_q + ((size_t)rbA * Gt + g0) * 1024, (u32)(Gt + G) * 1024u);
+  const rsrc_t rs = make_rsrc(base + c.off_s + ((size_t)rbA * Gt + g0) * SCB, (u32)(Gt + G) * SCB);
+  const rsrc_t rz = make_rsrc(base + c.off_z + ((size_t)rbA * Gt + g0) * ZZB, (u32)(Gt + G) * ZZB);
+  const rsrc_t rx = make_rsrc((const unsigned char *)c.act + (size_t)g0 * 256, KC_NO_ROW);
+  const Q4Consts q4c = q4_consts();
+  const DeqF16Consts dqc = deq_f16_consts();
+  const size_t orow0 = (size_t)split * a.T;
 
   for (int t0 = 0; t0 < m;) {
     const int left = m - t0;
     if (NTMAX >= 4 && left > 32) {
-      kc_pass<SWIGLU, 4, 2, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 64 ? left : 64, q4c);
+      const int mc = left < 64 ? left : 64;
+      if constexpr (Q4K) kc_pass_q4k<SWIGLU, 4, 2, KS>(c, smem, rq, rs, rz, rx, Gt, G, b, orow0, row0 + t0, mc, dqc);
+      else kc_pass<SWIGLU, 4, 2, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c);
       t0 += 64;
     } else if (NTMAX >= 2 && left > 16) {
-      kc_pass<SWIGLU, 2, 4, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 32 ? left : 32, q4c);
+      const int mc = left < 32 ? left : 32;
+      if constexpr (Q4K) kc_pass_q4k<SWIGLU, 2, 4, KS>(c, smem, rq, rs, rz, rx, Gt, G, b, orow0, row0 + t0, mc, dqc);
+      else kc_pass<SWIGLU, 2, 4, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c);
       t0 += 32;
     } else {
-      kc_pass<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, left < 16 ? left : 16, q4c);
+      const int mc = left < 16 ? left : 16;
+      if constexpr (Q4K) kc_pass_q4k<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, Gt, G, b, orow0, row0 + t0, mc, dqc);
+      else kc_pass<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c);
       t0 += 16;
     }
     if (t0 < m) __syncthreads();  // the next pass restages chunk buffer 0
@@ -2428,6 +2656,11 @@ static int launch_gemv_q4k_t(const GemvArgs &a, int grid, size_t lds, hipStream_
 
 template <bool SW>
 static int launch_gemv_q4k(const GemvArgs &a, int grid, int T, int Kmax, hipStream_t s) {
+  if (T > 1) {  // matrix-core form, passes of 16, 32 or 64 rows per unit
+    if (T > 32) return launch_gemv_mfma_kc<SW, 4, true>(a, grid, s);
+    if (T > 16) return launch_gemv_mfma_kc<SW, 2, true>(a, grid, s);
+    return launch_gemv_mfma_kc<SW, 1, true>(a, grid, s);
+  }
   // rows per pass: the smallest power of two >= T (at most 16) whose activations fit LDS; a unit with more
   // rows than that streams its weights once per pass (three tokens against a 20480-column reduction: two
   // rows per pass, two passes)
@@ -2495,13 +2728,19 @@ static size_t gemv_mfma_kc_lds(int nt, int cg) {
 
 // chunked-K form: a workgroup takes 4 / KS block pairs of a unit (both classes' pair counts are
 // multiples of four: I and H are multiples of 128)
-template <bool SW, int NTMAX, int KS>
+template <bool SW, int NTMAX, int KS, bool Q4K = false>
 static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t s) {
   constexpr int PW = 4 / KS;
   GemvArgs a = a_in;
   const int units = a.cls[1].nblk > 0 ? (grid_in - a.n_sh_blocks) / a.cls[1].nblk : 0;
-  if ((a.n_sh_blocks > 0 && a.cls[0].nblk % 4) || (units > 0 && a.cls[1].nblk % 4)) {
+  // q4_K, shared expert's w2 class: nblk counts ksplit workgroups per block pair
+  const int nsp = (Q4K && a.n_sh_blocks > 0 && a.cls[0].ksplit > 1) ? a.cls[0].ksplit : 1;
+  if ((a.n_sh_blocks > 0 && (a.cls[0].nblk % nsp || (a.cls[0].nblk / nsp) % 4)) || (units > 0 && a.cls[1].nblk % 4)) {
     moe_set_error("k_gemv_int4_mfma_kc: block pairs per unit not a multiple of 4");
+    return MOE_EINVAL;
+  }
+  if (Q4K && ((a.n_sh_blocks > 0 && (a.cls[0].G % (2 * nsp))) || (units > 0 && a.cls[1].G % 2))) {
+    moe_set_error("k_gemv_int4_mfma_kc<q4_K>: a reduction window must hold whole 256-wide super-blocks");
     return MOE_EINVAL;
   }
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
@@ -2512,10 +2751,10 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   if (NTMAX >= 4 && gemv_mfma_kc_lds(4, 2) > lds) lds = gemv_mfma_kc_lds(4, 2);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NTMAX, KS>,
+    hipError_t e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, true, NTMAX, KS, Q4K>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NTMAX, KS>,
+      e = hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<SW, false, NTMAX, KS, Q4K>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       moe_set_error("hipFuncSetAttribute(max dynamic LDS): %s", hipGetErrorString(e));
@@ -2524,8 +2763,8 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
     attr_set = true;
   }
   moe_ktimer_begin(SW ? MOE_K_W13 : MOE_K_W2, s);
-  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NTMAX, KS>), dim3(grid), dim3(256), lds, s, a);
-  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NTMAX, KS>), dim3(grid), dim3(256), lds, s, a);
+  if (a.units) hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, true, NTMAX, KS, Q4K>), dim3(grid), dim3(256), lds, s, a);
+  else hipLaunchKernelGGL((k_gemv_int4_mfma_kc<SW, false, NTMAX, KS, Q4K>), dim3(grid), dim3(256), lds, s, a);
   moe_ktimer_end(SW ? MOE_K_W13 : MOE_K_W2, s);
   return moe_check_launch("k_gemv_int4_mfma_kc");
 }
@@ -2534,10 +2773,10 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
 // unit slot in use; the unit list is made on the device, the host only knows its capacity), else one.
 // Measured: 256 workgroups (4096 x 14336 w2, 8 units) 101 us with one wave per pair, 77 us with two; 484
 // workgroups (2048 x 1408 w13, 20 units) 19.5 us against 25.7 us.  Four never paid.
-template <bool SW, int NTMAX>
+template <bool SW, int NTMAX, bool Q4K = false>
 static int launch_gemv_mfma_kc(const GemvArgs &a, int grid, hipStream_t s) {
-  if (grid / 4 >= 384) return launch_gemv_mfma_kc_ks<SW, NTMAX, 1>(a, grid, s);
-  return launch_gemv_mfma_kc_ks<SW, NTMAX, 2>(a, grid, s);
+  if (grid / 4 >= 384) return launch_gemv_mfma_kc_ks<SW, NTMAX, 1, Q4K>(a, grid, s);
+  return launch_gemv_mfma_kc_ks<SW, NTMAX, 2, Q4K>(a, grid, s);
 }
 
 template <bool SW>

@@ -17,12 +17,10 @@
 
 #include "moe_common.h"
 #include "moe_kernels.h"
+#include "moe_device.h"
 
-typedef unsigned int u32;
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(1))) const u32x4_t g_uint4;
 
 #define PF_BM 256     // most rows of one tile (8 blocks of 32)
 #define PF_BM_SHARED 256     // rows per tile of the dense shared expert in the w13 pass
@@ -316,12 +314,11 @@ __global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
 // v_mfma_f32_16x16x32_f16 (lane = row l&15, k quarter l>>4, dword j = 8 consecutive k), so a
 // wave loads them straight into registers and dequantises there: a nibble pair is shifted and masked
 // into the mantissas of two fp16 values 1 + q/16 and one packed fma per pair applies scale and zero
-// (pf_deq8 below).  gfx950 has packed fp16 arithmetic
+// (deq8_f16 below).  gfx950 has packed fp16 arithmetic
 // but no packed bf16 arithmetic, hence fp16 operands: activations are converted bf16 -> fp16
 // while they are staged into LDS (exact for |x| < 65504 outside the fp16 subnormal range); the h rows
 // between the two passes are written as fp16 by the w13 epilogue, so the w2 pass stages them as they are.
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const uint16_t g_u16;
 typedef __attribute__((address_space(1))) const unsigned char g_u8;
@@ -329,38 +326,6 @@ typedef __attribute__((address_space(1))) const unsigned char g_u8;
 #define PI_LDK 136  // LDS row stride in fp16 (128 + 8 pad = 272 bytes)
 #define PI_BM 192   // most rows of one tile: 6 blocks of 32 (96 accumulator registers per wave)
 
-static __device__ __forceinline__ u32 pf_bf16x2_to_f16x2(u32 d) {
-  // both halves are bf16; fp16 has more mantissa bits, so round-to-zero conversion is exact
-  auto h = __builtin_amdgcn_cvt_pkrtz(__uint_as_float(d << 16), __uint_as_float(d & 0xffff0000u));
-  return __builtin_bit_cast(u32, h);
-}
-// Dequantisation of 8 nibbles of a dword into 8 fp16 weights with ONE packed fma per pair: a nibble is masked into
-// mantissa bits 6..9 of an fp16 with the exponent of 1.0, which makes the exact value h = 1 + q/16; with S = 16 s and
-// C = -(16 + zero) s (int4) or C = -(16 s + m) (q4_K), both prepared once per group and row, h S + C = (q - zero) s
-// or q s - m.  The product is exact inside the fma; C carries the one extra rounding (2^-11 of at most 31 s, i.e.
-// 0.015 of a quantisation step, a bias common to the 128 weights of a group row).  The form before this one
-// ((h - (1024 + zero)) s with h = 1024 + q) was exact up to the final rounding and cost a packed subtract and
-// a packed multiply per pair (three operations for q4_K), in kernels that are bound by these operations.
-// Mask and exponent pattern are held in vector registers, made once per kernel: (x & M) | C is then ONE
-// v_and_or_b32 (a VOP3 instruction takes no literal and one scalar operand on this target).
-struct PfDeqConsts { u32 M, C; };
-static __device__ __forceinline__ PfDeqConsts pf_deq_consts() {
-  PfDeqConsts q{0x03c003c0u, 0x3c003c00u};
-  asm volatile("" : "+v"(q.M), "+v"(q.C));
-  return q;
-}
-// s2 / c2: fp16 bit patterns of S and C replicated in both halves
-static __device__ __forceinline__ f16x8_t pf_deq8(u32 d, u32 s2, u32 c2, const PfDeqConsts &q) {
-  const u32 M = q.M, C = q.C;
-  u32x4_t v;
-  v.x = ((d << 6) & M) | C; v.y = ((d << 2) & M) | C; v.z = ((d >> 2) & M) | C; v.w = ((d >> 6) & M) | C;
-  const f16x8_t h = __builtin_bit_cast(f16x8_t, v);   // 1 + q/16, exact
-  const f16x8_t s8 = __builtin_bit_cast(f16x8_t, u32x4_t{s2, s2, s2, s2});
-  const f16x8_t c8 = __builtin_bit_cast(f16x8_t, u32x4_t{c2, c2, c2, c2});
-  return __builtin_elementwise_fma(h, s8, c8);
-}
-
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
 // buffer resource over [p, p+bytes): loads past the end return 0 instead of faulting
 static __device__ __forceinline__ rsrc_t pf_rsrc(const void *p, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, (int)bytes, 0x00020000);
@@ -369,14 +334,6 @@ static __device__ __forceinline__ const unsigned char *pf_uniform(const unsigned
   const unsigned long long v = (unsigned long long)p;
   const u32 lo = __builtin_amdgcn_readfirstlane((u32)v), hi = __builtin_amdgcn_readfirstlane((u32)(v >> 32));
   return (const unsigned char *)(((unsigned long long)hi << 32) | lo);
-}
-
-static __device__ __forceinline__ u32 pf_h2f(u32 hbits) {  // fp16 bits -> fp32 bits
-  const _Float16 h = __builtin_bit_cast(_Float16, (uint16_t)hbits);
-  return __builtin_bit_cast(u32, (float)h);
-}
-static __device__ __forceinline__ u32 pf_f2h(float f) {  // fp32 -> fp16 bits (round to nearest)
-  return (u32)__builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
 struct PiMeta { u32 sc[4]; u32 zz[4]; };  // raw fp16 scale bits / zero nibble of the lane's row in the 4 tiles
@@ -391,7 +348,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
   const int lane = tid & 63, g = tid >> 8;
   const int r = lane & 15, qd = lane >> 4;
   const int ch = tid & 15, r0 = tid >> 4;  // staging: row r0 + 32 i (block i), 16-byte chunk ch of the 128-k group
-  const PfDeqConsts dqc = pf_deq_consts();
+  const DeqF16Consts dqc = deq_f16_consts();
   u32x4_t ra[3], wA[4], wB[4];
   PiMeta mA, mB;
   // activations of the next group travel in two halves (row blocks 0..2, then 3..5) through
@@ -408,8 +365,8 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
       if (3 * half + i < nb) {
         u32x4_t v = ra[i];
         if (!ACT16) {
-          v.x = pf_bf16x2_to_f16x2(ra[i].x); v.y = pf_bf16x2_to_f16x2(ra[i].y);
-          v.z = pf_bf16x2_to_f16x2(ra[i].z); v.w = pf_bf16x2_to_f16x2(ra[i].w);
+          v.x = bf16x2_to_f16x2(ra[i].x); v.y = bf16x2_to_f16x2(ra[i].y);
+          v.z = bf16x2_to_f16x2(ra[i].z); v.w = bf16x2_to_f16x2(ra[i].w);
         }
         *(u32x4_t *)(A_ + (r0 + 32 * (3 * half + i)) * PI_LDK + ch * 8) = v;
       }
@@ -428,21 +385,21 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
       }
     }
   };
-  // S = 16 s and C of pf_deq8 for the lane's row in the 4 tiles of a group, once per group
+  // S = 16 s and C of deq8_f16 for the lane's row in the 4 tiles of a group, once per group
   auto prep = [&](const PiMeta &m, u32 (&s2)[4], u32 (&c2)[4]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       float s16, cz;
       if (Q4K) {
-        s16 = 16.f * __builtin_bit_cast(float, pf_h2f(m.zz[t] & 0xffffu)) * (float)(m.sc[t] & 0xffu);
-        const float dmn = __builtin_bit_cast(float, pf_h2f(m.zz[t] >> 16)) * (float)((m.sc[t] >> 8) & 0xffu);
+        s16 = 16.f * __builtin_bit_cast(float, h2f_bits(m.zz[t] & 0xffffu)) * (float)(m.sc[t] & 0xffu);
+        const float dmn = __builtin_bit_cast(float, h2f_bits(m.zz[t] >> 16)) * (float)((m.sc[t] >> 8) & 0xffu);
         cz = -s16 - dmn;
       } else {
-        const float sf = __builtin_bit_cast(float, pf_h2f(m.sc[t] & 0xffffu));
+        const float sf = __builtin_bit_cast(float, h2f_bits(m.sc[t] & 0xffffu));
         s16 = 16.f * sf;
         cz = -(16.f + (float)((m.zz[t] >> (4 * (r & 1))) & 15u)) * sf;
       }
-      const u32 sb = pf_f2h(s16), cb = pf_f2h(cz);
+      const u32 sb = f2h_bits(s16), cb = f2h_bits(cz);
       s2[t] = sb | (sb << 16);
       c2[t] = cb | (cb << 16);
     }
@@ -454,7 +411,7 @@ static __device__ __forceinline__ void pi_mainloop(f32x4_t (&acc)[4][6], uint16_
       const int j = j0 + jj;
       f16x8_t wd[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) wd[t] = pf_deq8(wq[t][j], s2[t], z2[t], dqc);
+      for (int t = 0; t < 4; ++t) wd[t] = deq8_f16(wq[t][j], s2[t], z2[t], dqc);
 #pragma unroll
       for (int tb = 0; tb < 2 * NBW; ++tb) {
         const f16x8_t xa = *(const f16x8_t *)(A_ + (64 * (tb >> 1) + 16 * (tb & 1)) * PI_LDK + 8 * j);

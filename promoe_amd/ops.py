@@ -14,7 +14,7 @@ from ._lib import lib, ptr, cur_stream, check
 def gemv_max_tokens(fmt: int) -> int:
     """Largest token group moe_forward sends to the GEMV kernels; larger ones (and every bf16 layer) take
     the matrix-core tile kernels."""
-    return 64 if fmt == L.FMT_INT4_G128 else 16
+    return 0 if fmt == L.FMT_BF16 else 64
 
 
 def _dev(t):

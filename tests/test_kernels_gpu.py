@@ -246,10 +246,23 @@ def test_fused_route_equals_separate_kernels(cuda, T, H, E, k, mode, extra):
     assert torch.equal(d.units, d_ref.units) and torch.equal(d.active_ids, d_ref.active_ids)
 
 
-@pytest.mark.parametrize("T", [1, 3, 4, 16, 21])
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 16, 21, 33, 40, 64])
 def test_decode_q4k_layer_small(cuda, T):
+    """One token: the dot-product GEMV; more: the chunked-K matrix-core form with passes of 16, 32 and 64 rows
+    (E = 8, k = 2: the shared expert has T rows, a routed unit about T / 4)."""
     print(f"case decode_q4k_small T={T}", flush=True)
     check_layer(Q4KLayer(H=256, I=512, E=8, I_sh=256, seed=3), T, 2, 0, cuda)
+
+
+@pytest.mark.parametrize("T", [3, 20, 48])
+def test_decode_q4k_long_reduction_split_shared_expert(cuda, T):
+    """A shared expert wide enough that its w2 reduction is split over workgroups (I_sh = 8192: 64 groups in 2 or
+    4 windows, each window a whole number of super-blocks), group counts that leave partial chunks (I = 768: 6
+    groups against chunks of 8 and 4), few experts with many rows each."""
+    from promoe_amd import ops, _lib as L
+    print(f"case decode_q4k_split T={T}", flush=True)
+    assert ops.shared_splits(L.FMT_Q4K, T, 512, 8192) > 1
+    check_layer(Q4KLayer(H=512, I=768, E=4, I_sh=8192, seed=11), T, 2, 0, cuda)
 
 
 def test_decode_q4k_qwen2_shape(cuda):
