@@ -744,6 +744,7 @@ struct GemvArgs {
   // (value, g_seq) pair; g_nblk = 0: the logits come from an earlier launch (r_logits)
   const uint16_t *g_w; const float *g_bias; unsigned long long *g_stamp; float *g_logits_out;
   int g_rows, g_nbias, g_nblk, g_seq;
+  int unit_slots;               // chunked-K launches of more than 16 tokens: slots of `units` when at most 64, else 0
 };
 
 // Gate logits handed over inside a launch.  A logit travels as one 8-byte word (value, sequence number of the
@@ -831,8 +832,12 @@ static __device__ __forceinline__ void gemv_publish_units(const GemvArgs &a) {
 }
 
 // bx: the workgroup's index among the working ones (launches with a publishing workgroup put that one first)
-template <bool DEVUNITS>
-static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const int bx) {
+// BY_ROWS (device-built unit list of at most 64 slots, a.unit_slots > 0): position u of the grid takes the unit of
+// rank u when the units are ordered by the passes they need (more than 32 rows, 17 to 32, 1 to 16, none; list
+// order inside a class).  The workgroups of the units with the most rows then start first and those of the unused
+// slots last, instead of a popular expert starting when the first round of workgroups has finished.
+template <bool DEVUNITS, bool BY_ROWS = false>
+static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const int bx, const int lane = 0) {
   GemvWork wk;
   const GemvClass c0 = a.cls[0], c1 = a.cls[1];
   const int n_sh = a.n_sh_blocks;
@@ -853,6 +858,23 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
         const KUnit kd = a.kunits_dev[u];
         wk.m = kd.m; wk.row0 = kd.row0;
         wk.base = (const unsigned char *)kd.base;
+      } else if (BY_ROWS && a.unit_slots > 0) {
+        const rsrc_t ru = make_rsrc(a.units, (u32)a.unit_slots * 16u);
+        const u32x4_t ul = __builtin_amdgcn_raw_buffer_load_b128(ru, lane * 16, 0, 0);  // past the list: zeros
+        const int ml = (int)ul.y;
+        const unsigned long long c3 = __ballot(ml > 32), c2 = __ballot(ml > 16 && ml <= 32),
+                                 c1 = __ballot(ml > 0 && ml <= 16), c0 = ~(c3 | c2 | c1);
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const int n3 = __popcll(c3), n2 = __popcll(c2), n1 = __popcll(c1);
+        const int rank = ml > 32 ? __popcll(c3 & below)
+                         : ml > 16 ? n3 + __popcll(c2 & below)
+                         : ml > 0 ? n3 + n2 + __popcll(c1 & below) : n3 + n2 + n1 + __popcll(c0 & below);
+        const unsigned long long hit = __ballot(rank == u);
+        const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)hit) - 1);  // u < 64: exactly one lane
+        const int ue = __builtin_amdgcn_readlane((int)ul.x, src);
+        wk.m = __builtin_amdgcn_readlane(ml, src);
+        wk.row0 = __builtin_amdgcn_readlane((int)ul.z, src);
+        wk.base = wk.m > 0 ? (const unsigned char *)a.expert_ptr[ue] : nullptr;
       } else {
         const moe_unit ud = a.units[u];
         wk.m = ud.m; wk.row0 = ud.row0;
@@ -1850,6 +1872,16 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 // first byte past it, so that such a load is out of range by any reading of the range rule (first byte or last
 // byte of the access, no 32-bit wrap) and returns zeros without a memory request.
 #define KC_NO_ROW 0x7fffff00u
+#ifdef MOE_STAMPS
+#ifndef KC_STAMP_SW
+#define KC_STAMP_SW true
+#endif
+#define KC_STAMP(i) do { if (SWIGLU == KC_STAMP_SW) STAMP(i); } while (0)
+#define KC_STAMPV(i, v) do { if (SWIGLU == KC_STAMP_SW) STAMPV(i, v); } while (0)
+#else
+#define KC_STAMP(i)
+#define KC_STAMPV(i, v)
+#endif
 
 // One pass of the chunked-K form: rows row_first .. row_first + mc - 1 (mc <= 16 NT) of one unit against the block
 // pair b of its matrix.  Every thread of the workgroup takes part (barriers inside).
@@ -1956,6 +1988,7 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
       if (e < NSE) ((float4 *)sfw)[e] = scale_zero_pair(scr[i], zr[i] >> (8 * (e & 3)));
     }
     __syncthreads();
+    if (ch == 0) KC_STAMP(2);
     // unconditional (past the end: clamped addresses, zero scales), so that every iteration issues the
     // same number of loads and the waits for the prefetched registers can be exact
     load_chunk(ch + 1);
@@ -2056,6 +2089,7 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
       }
     }
   }
+  KC_STAMP(3);
   if constexpr (KS > 1) {
     // the sums of a pair's waves meet in the activation buffers (free once every wave is done with them)
     __syncthreads();
@@ -2328,6 +2362,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   constexpr int NB = 2;
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  KC_STAMP(0);
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
   const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
@@ -2336,15 +2372,17 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
     return;
   }
   const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
+  const GemvWork wk = gemv_resolve<DEVUNITS, (NTMAX > 1)>(a, bx, lane);
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
+  KC_STAMPV(5, (unsigned long long)(m + 1));
   if (m <= 0) return;
   if (base == nullptr) {
     if (tid == 0) moe_raise_err(a.err);
     return;
   }
+  KC_STAMP(1);
   const int Gt = c.G;
   const int nsp = (Q4K && c.ksplit > 1) ? c.ksplit : 1;
   const int split = nsp > 1 ? wk.b % nsp : 0;
@@ -2380,6 +2418,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
     }
     if (t0 < m) __syncthreads();  // the next pass restages chunk buffer 0
   }
+  KC_STAMP(4);
 }
 
 // ---------------------------------------------------------------------------
@@ -2745,6 +2784,7 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   }
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
   a.cls[1].nblk /= PW;
+  a.unit_slots = (NTMAX > 1 && a.units && units <= 64) ? units : 0;
   const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
   size_t lds = gemv_mfma_kc_lds(1, 8);  // the widest of the pass shapes the kernel may pick
   if (NTMAX >= 2 && gemv_mfma_kc_lds(2, 4) > lds) lds = gemv_mfma_kc_lds(2, 4);
