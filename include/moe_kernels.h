@@ -249,7 +249,11 @@ int moe_decode_token_int4_noalloc(const void *x_bf16, const float *logits, int E
                                   const float *shared_gate_logit, void *y_bf16, int *err, void *stream);
 
 /* k3 for q4_K experts: same buffers as moe_experts_decode_int4, device-side unit list only.
- * Exception: part_s.  With few output rows and a long reduction (H / 32 block pairs, I_sh columns: Qwen2-57B's
+ * One token: dot products on the vector ALU in bf16 x (128 + q), scales applied per sub-block in fp32.  Two tokens
+ * and more (any T; moe_forward sends up to 64): the chunked-K matrix-core kernel, every weight dequantised to fp16
+ * (d sc q - dmin m, the arithmetic of moe_experts_prefill for this format) against fp16 activations, fp32
+ * accumulation; activations must stay below 65504 in magnitude there.
+ * Exception to "same buffers": part_s.  With few output rows and a long reduction (H / 32 block pairs, I_sh columns: Qwen2-57B's
  * shared expert is 112 block pairs over 20480 columns) the w2 pass splits the shared expert's reduction over
  * moe_decode_shared_splits(MOE_FMT_Q4K, T, H, I_sh) = S workgroups per block pair; split s writes its partial
  * rows to part_s + s*T*H, so part_s must hold S*T*H floats and the combine must be told
