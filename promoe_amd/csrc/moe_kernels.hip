@@ -745,6 +745,9 @@ struct GemvArgs {
   const uint16_t *g_w; const float *g_bias; unsigned long long *g_stamp; float *g_logits_out;
   int g_rows, g_nbias, g_nblk, g_seq;
   int unit_slots;               // chunked-K launches of more than 16 tokens: slots of `units` when at most 64, else 0
+  int pairs;                    // T k of the step (0: unknown)
+  int row_split;                // w2 launches of more than 32 tokens: a unit of more than 32 rows has two workgroups
+                                // per group of block pairs, rows 0..31 and 32.., and so has the shared expert
 };
 
 // Gate logits handed over inside a launch.  A logit travels as one 8-byte word (value, sequence number of the
@@ -813,6 +816,7 @@ struct GemvWork {
   GemvClass c;
   const unsigned char *base;
   int m, row0, b;
+  int half;  // row_split: which half of the unit's rows
 };
 // The publishing workgroup of a w13 launch (the last one of its grid): the unit list of the step goes from device
 // memory to the host's pinned copy while the other workgroups stream weights, then the sequence word the host
@@ -850,6 +854,11 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
   const int rr = sh ? bx : bx - n_sh;
   const int u = sh ? 0 : rr / c.nblk;
   wk.b = rr - u * c.nblk;
+  wk.half = 0;
+  if (BY_ROWS && sh && a.row_split) {  // the shared expert's workgroups come twice, one set per half of the rows
+    wk.half = bx >= (n_sh >> 1) ? 1 : 0;
+    wk.b = bx - (wk.half ? (n_sh >> 1) : 0);
+  }
   if (DEVUNITS) {
     if (sh) {
       wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
@@ -869,12 +878,22 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
         const int rank = ml > 32 ? __popcll(c3 & below)
                          : ml > 16 ? n3 + __popcll(c2 & below)
                          : ml > 0 ? n3 + n2 + __popcll(c1 & below) : n3 + n2 + n1 + __popcll(c0 & below);
-        const unsigned long long hit = __ballot(rank == u);
-        const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)hit) - 1);  // u < 64: exactly one lane
-        const int ue = __builtin_amdgcn_readlane((int)ul.x, src);
-        wk.m = __builtin_amdgcn_readlane(ml, src);
-        wk.row0 = __builtin_amdgcn_readlane((int)ul.z, src);
-        wk.base = wk.m > 0 ? (const unsigned char *)a.expert_ptr[ue] : nullptr;
+        // row_split: the n3 units of more than 32 rows take two positions each (rows 0..31, rows 32..)
+        int ur = u;
+        if (a.row_split) {
+          if (u < 2 * n3) { wk.half = u & 1; ur = u >> 1; }
+          else ur = u - n3;
+        }
+        const unsigned long long hit = __ballot(rank == ur);
+        if (hit == 0ull) {  // a position past the list
+          wk.m = 0; wk.row0 = 0; wk.base = nullptr;
+        } else {
+          const int src = __builtin_amdgcn_readfirstlane(__ffsll((long long)hit) - 1);  // exactly one lane
+          const int ue = __builtin_amdgcn_readlane((int)ul.x, src);
+          wk.m = __builtin_amdgcn_readlane(ml, src);
+          wk.row0 = __builtin_amdgcn_readlane((int)ul.z, src);
+          wk.base = wk.m > 0 ? (const unsigned char *)a.expert_ptr[ue] : nullptr;
+        }
       } else {
         const moe_unit ud = a.units[u];
         wk.m = ud.m; wk.row0 = ud.row0;
@@ -2398,8 +2417,14 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
   const DeqF16Consts dqc = deq_f16_consts();
   const size_t orow0 = (size_t)split * a.T;
 
-  for (int t0 = 0; t0 < m;) {
-    const int left = m - t0;
+  // rows of this workgroup: all of the unit's, or one half of a unit of more than 32 rows (row_split)
+  int r_lo = 0, r_hi = m;
+  if (NTMAX > 1 && a.row_split) {
+    if (m > 32) { r_lo = wk.half ? 32 : 0; r_hi = wk.half ? m : 32; }
+    else if (wk.half) return;
+  }
+  for (int t0 = r_lo; t0 < r_hi;) {
+    const int left = r_hi - t0;
     if (NTMAX >= 4 && left > 32) {
       const int mc = left < 64 ? left : 64;
       if constexpr (Q4K) kc_pass_q4k<SWIGLU, 4, 2, KS>(c, smem, rq, rs, rz, rx, Gt, G, b, orow0, row0 + t0, mc, dqc);
@@ -2416,7 +2441,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
       else kc_pass<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c);
       t0 += 16;
     }
-    if (t0 < m) __syncthreads();  // the next pass restages chunk buffer 0
+    if (t0 < r_hi) __syncthreads();  // the next pass restages chunk buffer 0
   }
   KC_STAMP(4);
 }
@@ -2785,7 +2810,38 @@ static int launch_gemv_mfma_kc_ks(const GemvArgs &a_in, int grid_in, hipStream_t
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
   a.cls[1].nblk /= PW;
   a.unit_slots = (NTMAX > 1 && a.units && units <= 64) ? units : 0;
-  const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
+  // w2 pass above 32 tokens: its launch ends with the workgroups of the units that have the most rows (the shared
+  // expert's above all: every token's row against the longest reduction), and the chip has room beside them, so
+  // those units get a second workgroup per group of block pairs for the rows from 32 on.  At most pairs / 33 units
+  // can have more than 32 rows.  The weights of such a unit are streamed twice (few units, from the caches the
+  // second time).
+  int units_grid = units;
+  if (!SW && NTMAX >= 4 && a.unit_slots > 0 && a.pairs > 0 && !a.kunits_dev) {
+    a.row_split = 1;
+    const int extra = a.pairs / 33 < units ? a.pairs / 33 : units;
+    units_grid = units + extra;
+    a.n_sh_blocks *= 2;
+  } else if (!SW && NTMAX >= 4 && !a.units && !a.kunits_dev && units > 0 && units <= GEMV_MAX_KUNITS) {
+    // the same split for units that travel by value: the halves become entries of their own, most rows first
+    int heavy = 0;
+    for (int u = 0; u < units; ++u) heavy += a.ku[u].m > 32;
+    if (units + heavy <= GEMV_MAX_KUNITS) {
+      KUnit out[GEMV_MAX_KUNITS];
+      int n = 0;
+      for (int u = 0; u < units; ++u)
+        if (a.ku[u].m > 32) {
+          out[n++] = KUnit{a.ku[u].base, 32, a.ku[u].row0};
+          out[n++] = KUnit{a.ku[u].base, a.ku[u].m - 32, a.ku[u].row0 + 32};
+        }
+      for (int u = 0; u < units; ++u)
+        if (a.ku[u].m <= 32) out[n++] = a.ku[u];
+      for (int u = 0; u < n; ++u) a.ku[u] = out[u];
+      a.row_split = 1;
+      units_grid = n;
+      a.n_sh_blocks *= 2;
+    }
+  }
+  const int grid = a.n_sh_blocks + units_grid * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
   size_t lds = gemv_mfma_kc_lds(1, 8);  // the widest of the pass shapes the kernel may pick
   if (NTMAX >= 2 && gemv_mfma_kc_lds(2, 4) > lds) lds = gemv_mfma_kc_lds(2, 4);
   if (NTMAX >= 4 && gemv_mfma_kc_lds(4, 2) > lds) lds = gemv_mfma_kc_lds(4, 2);
@@ -2903,7 +2959,6 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
     moe_set_error("moe_experts_decode_int4: bad argument (T=%d H=%d I=%d I_sh=%d)", T, H, I, I_sh);
     return MOE_EINVAL;
   }
-  (void)k;
   moe_int4_layout lr, ls;
   memset(&lr, 0, sizeof lr); memset(&ls, 0, sizeof ls);
   if (max_units > 0 && moe_int4_layout_make(H, I, &lr)) return MOE_EINVAL;
@@ -2915,6 +2970,7 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
   memset(&a, 0, sizeof a);
   a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
   a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err;
+  a.pairs = k > 0 ? T * k : 0;
   if (units_host && expert_ptr_host && max_units <= GEMV_MAX_KUNITS) {
     a.units = nullptr;
     for (int u = 0; u < max_units; ++u) {
@@ -3214,7 +3270,6 @@ extern "C" int moe_experts_decode_q4k(const void *x, int T, int H, int I, int I_
     moe_set_error("moe_experts_decode_q4k: bad argument (T=%d H=%d I=%d I_sh=%d)", T, H, I, I_sh);
     return MOE_EINVAL;
   }
-  (void)k;
   moe_int4_layout lr, ls;
   memset(&lr, 0, sizeof lr); memset(&ls, 0, sizeof ls);
   if (max_units > 0 && moe_q4k_layout_make(H, I, &lr)) return MOE_EINVAL;
@@ -3225,6 +3280,7 @@ extern "C" int moe_experts_decode_q4k(const void *x, int T, int H, int I, int I_
   memset(&a, 0, sizeof a);
   a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
   a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err;
+  a.pairs = k > 0 ? T * k : 0;
   a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z,
                        H, H / 128, T == 1 ? 0 : H, I_sh, I_sh / 16, 0};
   a.cls[1] = GemvClass{(const uint16_t *)x, T == 1 ? nullptr : sorted_tok, h_r, lr.off13_q, lr.off13_s,
