@@ -149,6 +149,25 @@ int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int k, int mod
                       moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
                       void *stream);
 
+/* k1a + k1b + k2 in one launch for decode batches (2 <= T <= 32, E <= 256, T*k <= 512): same results, bit for
+ * bit, as moe_gate_logits + moe_topk_dispatch (reference: the gate's linear layer, the top-k and the expert
+ * grouping of the patched sparse block, utils/__init__.py:84-141).  Workgroup 0 routes; the other workgroups sum
+ * the gate rows (a wave per (token, row)) and hand every logit to it through gate_ws as a (value, gate_seq) word,
+ * which it polls (bounded: on a time-out *err |= 1); the logits also land in logits[t*ldl + e].
+ *   E_rows = E, or E+1 when row E of wg is the shared expert's gate vector; bias covers rows 0 .. n_bias-1.
+ *   gate_ws: moe_gate_route_ws_bytes(T, E_rows) of device memory, zeroed once (the area of
+ *   moe_decode_token_int4_gate may be shared when it is that large); gate_seq: nonzero, never used before on gate_ws.
+ *   parts: 8 = every gate row is summed once per part of the chip and travels through that part's second-level
+ *   cache (plus one device-scope copy as the fallback), 1 = summed once and handed over at device scope.
+ *   units_host_out .. seq_value: as in moe_topk_dispatch. */
+int64_t moe_gate_route_ws_bytes(int T, int E_rows);
+int moe_gate_topk_dispatch(const void *x_bf16, const void *wg_bf16, const float *bias, int n_bias, float *logits,
+                           int T, int H, int E, int E_rows, int ldl, int k, int mode, int *idx, float *w,
+                           int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
+                           moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
+                           moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
+                           void *gate_ws, int gate_seq, int parts, int *err, void *stream);
+
 /* k3 (decode): int4 grouped SwiGLU expert product through the slot table.
  *   expert_ptr[e] : device address of expert e's slot (0 = not resident -> *err |= 1)
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL

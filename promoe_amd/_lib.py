@@ -56,6 +56,9 @@ _sig("moe_experts_decode_int4", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, v
 _sig("moe_experts_decode_int4_publish", [vp, i32, i32, i32, i32, i32, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32,
                                           vp, vp, vp, vp, i32, vp])
 _sig("moe_topk_dispatch", [vp, i32, i32, i32, i32, i32] + [vp] * 10 + [i32, vp, vp, vp, i32, vp])
+_sig("moe_gate_route_ws_bytes", [i32, i32], i64)
+_sig("moe_gate_topk_dispatch", [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 10 +
+     [i32, vp, vp, vp, i32, vp, i32, i32, vp, vp])
 _sig("moe_noalloc_scratch_bytes", [], i64)
 _sig("moe_decode_token_int4_noalloc", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp])
 _sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])

@@ -23,6 +23,7 @@ struct LayerState {
   // one-token launches that compute their gate logits themselves: hand-over words (zeroed once) and the number
   // of the last such launch (every launch takes the next one, so no word of an earlier launch passes for a new one)
   unsigned char *gate_ws = nullptr;
+  size_t gate_ws_bytes = 0;
   int gate_seq = 0;
   moe_unit *units = nullptr, *units_sub = nullptr;
   int64_t *active_ids = nullptr;
@@ -168,7 +169,8 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->sorted_tok, P);
   rc |= dalloc(s, &s->n_active, 1);
   rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
-  rc |= dalloc(s, &s->gate_ws, (size_t)moe_gate_ws_bytes());
+  s->gate_ws_bytes = (size_t)std::max<int64_t>(moe_gate_ws_bytes(), moe_gate_route_ws_bytes(std::min(T, 32), E + 1));
+  rc |= dalloc(s, &s->gate_ws, s->gate_ws_bytes);
   rc |= dalloc(s, &s->units, s->max_units);
   rc |= dalloc(s, &s->units_sub, (size_t)s->max_units * 2);
   rc |= dalloc(s, &s->active_ids, s->max_units);
@@ -209,7 +211,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   memset(s->err_spec, 0, sizeof(int) * 2 * eng->cfg.num_layer);
   s->spec_state.assign((size_t)2 * eng->cfg.num_layer, 0);
   s->spec_turn.assign(eng->cfg.num_layer, 0);
-  HIPC(hipMemset(s->gate_ws, 0, (size_t)moe_gate_ws_bytes()));
+  HIPC(hipMemset(s->gate_ws, 0, s->gate_ws_bytes));
   if (s->disp_ws) HIPC(hipMemset(s->disp_ws, 0, 64));
   *s->opt_seq = 0;
   HIPC(hipEventCreateWithFlags(&s->ev, hipEventDisableTiming));
@@ -306,6 +308,40 @@ static int shared_pieces(const moe_layer_desc &d, int T, const LayerState *s) {
 // what the one-token w2 + combine kernel asks of a layer (its waves stage what they need themselves, so the
 // widths of the experts do not matter; a lane per unit holds the unit's address)
 static bool w2c_fits(const moe_layer_desc &d, int k) { return d.H % 16 == 0 && k < 64; }
+
+
+// Gate logits, top-k and dispatch of a decode batch of 2 to 32 tokens: one launch (the gate rows' workgroups hand
+// the logits to the routing workgroup inside it), or the gate launch(es) and the routing launch
+static int gate_parts_env() {
+  static const int v = [] { const char *e = getenv("MOE_GATE_ROUTE"); return e ? atoi(e) : 1; }();
+  return v;
+}
+static int route_batch(const moe_layer_desc &d, LayerState *s, const void *x, int T, int E, int k, int n_gate_rows, int ldl,
+                       int max_units, int layer, moe_unit *host_units, int *host_n, int *host_seq, int seq_val,
+                       hipStream_t st) {
+  int rc;
+  const int parts = gate_parts_env();
+  if (T >= 2 && d.H % 8 == 0 && (parts == 1 || parts == 8) &&
+      moe_gate_route_ws_bytes(T, n_gate_rows) <= (int64_t)s->gate_ws_bytes) {
+    s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
+    return moe_gate_topk_dispatch(x, d.gate_w, d.gate_bias, d.gate_bias ? E : 0, s->logits, T, d.H, E, n_gate_rows, ldl, k,
+                                  d.route_mode, s->idx, s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair,
+                                  s->sorted_tok, s->units, s->n_active, s->active_ids, max_units, host_units, host_n,
+                                  host_seq, seq_val, s->gate_ws, s->gate_seq, parts, s->err_host + layer, st);
+  }
+  if (!d.gate_bias) {
+    if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
+  } else {
+    // the bias covers the routed experts only; the shared-gate row (row E) has none
+    if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
+    if (d.shared_gated &&
+        (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
+      return rc;
+  }
+  return moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
+                           s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
+                           max_units, host_units, host_n, host_seq, seq_val, st);
+}
 
 extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
   if (!eng) { moe_set_error("null engine"); return MOE_EINVAL; }
@@ -547,42 +583,23 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   if (all_resident && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory
-    if (!d.gate_bias) {
-      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
-    } else {
-      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
-      if (d.shared_gated &&
-          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
-        return rc;
-    }
     LayerState::Pending &pn = s->pend[s->pend_head];
     if (pn.busy && (rc = moe_forward_harvest(eng, true))) return rc;
     tail_seq = ++s->seq_counter;
     // the unit list reaches the host from the w13 launch where that one can carry it (its stores to pinned memory
     // hold the routing launch for about 2 us, and nothing in the w13 launch waits for them), else from here
     w13_publishes = decode_publishes(d, T, max_units);
-    if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
-                                s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                max_units, w13_publishes ? nullptr : pn.units, w13_publishes ? nullptr : pn.n_active,
-                                w13_publishes ? nullptr : pn.seq, tail_seq, st)))
+    if ((rc = route_batch(d, s, x, T, E, k, n_gate_rows, ldl, max_units, layer, w13_publishes ? nullptr : pn.units,
+                          w13_publishes ? nullptr : pn.n_active, w13_publishes ? nullptr : pn.seq, tail_seq, st)))
       return rc;
     routed_by_tail = true;
   } else if (T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch whose routing the host has to see before it can go on (experts may be missing): logits, then
     // top-k + dispatch in one launch that stores the unit list into pinned host memory and, behind it, a sequence
     // word; the host polls the word below.  Two copies, an event and a blocking wait for it took 15-20 us per step.
-    if (!d.gate_bias) {
-      if ((rc = moe_gate_logits(x, d.gate_w, nullptr, s->logits, T, d.H, n_gate_rows, ldl, st))) return rc;
-    } else {
-      if ((rc = moe_gate_logits(x, d.gate_w, d.gate_bias, s->logits, T, d.H, E, ldl, st))) return rc;
-      if (d.shared_gated &&
-          (rc = moe_gate_logits(x, (const uint16_t *)d.gate_w + (size_t)E * d.H, nullptr, s->logits + E, T, d.H, 1, ldl, st)))
-        return rc;
-    }
     host_seq = ++s->seq_counter;
-    if ((rc = moe_topk_dispatch(s->logits, T, E, ldl, k, d.route_mode, s->idx, s->topk_w, s->counts, s->offsets,
-                                s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
-                                max_units, s->units_host, s->n_active_host, s->opt_seq, host_seq, st)))
+    if ((rc = route_batch(d, s, x, T, E, k, n_gate_rows, ldl, max_units, layer, s->units_host, s->n_active_host, s->opt_seq,
+                          host_seq, st)))
       return rc;
   } else {
     if (!d.gate_bias) {

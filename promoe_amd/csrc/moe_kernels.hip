@@ -544,6 +544,11 @@ struct RouteArgs {
   moe_unit *units; int *n_active; long long *active_ids;
   unsigned *counter;
   moe_unit *host_units; int *host_n_active; int *host_seq; int host_seq_val, pad_;
+  // k_gate_route: bias rows, the hand-over area of the gate rows (copies of g_copy_words words: one per part of the
+  // chip and a device-scope one), the launch's sequence number, and the word raised when the hand-over times out
+  int n_bias, g_seq, g_copy_words, g_parts;  // g_parts: 8 = every item once per part of the chip, 1 = once
+  unsigned long long *g_stamp;
+  int *err;
 };
 
 // top-k (one wave per token) and stable dispatch by ONE workgroup of NW waves; the bodies of
@@ -806,6 +811,84 @@ static __device__ __forceinline__ void gate_rows_stamped(const GemvArgs &a, cons
 #ifdef MOE_STAMPS
   if (w == 0) { asm volatile("" ::: "memory"); STAMP(1); asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); STAMP(2); }
 #endif
+}
+
+// k1a + k1b + k2 in one launch for decode batches (2 to 32 tokens): workgroup 0 is the routing workgroup of
+// k_topk_dispatch, the others sum the gate rows and hand every logit to it as a (value, sequence number) word, the
+// way the one-token launch does (see gate_rows_stamped): each work item (a token and NW gate rows, a wave per row,
+// the summation order of k_gate_logits) is done by eight workgroups in a row, one per part of the chip in the
+// usual placement; each writes the copy of the part it finds itself on through that part's second-level cache,
+// the first of the eight also a device-scope copy and the plain logits for the kernels behind this launch.  The
+// routing workgroup polls the copy of its own part (a thread per word, loads past the first-level cache) and
+// after GATE_LOCAL_SPINS rounds the device-scope copy, keeps the logits in LDS and goes on as k_topk_dispatch.
+// A word that never arrives raises *err after GATE_POLL_LIMIT rounds instead of holding the launch.
+#define GROUTE_MAX_ROWS 264  // LDS row stride of the logits: E <= 256 and a shared-gate row, padded
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void k_gate_route(const RouteArgs a) {
+  __shared__ int s_idx[ROUTE_MAXP];
+  __shared__ unsigned long long s_mask[ROUTE_MAXT * 4];
+  __shared__ int s_off[257];
+  __shared__ int s_wsum[NW], s_wact[NW], s_tot;
+  __shared__ float s_logits[(NW == 4 ? 4 : 32) * GROUTE_MAX_ROWS];
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int T = a.T, Erows = a.Erows, H = a.H;
+  if (blockIdx.x > 0) {
+    const int q = (int)blockIdx.x - 1;
+    const bool per_part = a.g_parts == GATE_PARTS;
+    const int item = per_part ? q >> 3 : q;
+    const int nrb = (Erows + NW - 1) / NW;
+    const int t = item / nrb, e = (item - t * nrb) * NW + w;
+    if (e >= Erows) return;
+    const bool biased = a.bias && e < a.n_bias;
+    const float bias_e = biased ? a.bias[e] : 0.f;
+    asm volatile("" :: "v"(bias_e));  // requested in front of the row
+    const float acc = gate_row_sum(a.x + (size_t)t * H, a.wg + (size_t)e * H, H, lane);
+    const float val = biased ? acc + bias_e : acc;
+    const u32x2_t word = {__float_as_uint(val), (u32)a.g_seq};
+    const int wi = t * Erows + e;
+    if (per_part && lane == 0)
+      __builtin_amdgcn_raw_buffer_store_b64(word, make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words,
+                                                            (u32)a.g_copy_words * 8u), wi * 8, 0, 1 /* sc0 */);
+    if (!per_part || (q & 7) == 0) {
+      const unsigned long long word64 = ((unsigned long long)word.y << 32) | word.x;
+      if (lane == 1)
+        __hip_atomic_store(a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words + wi, word64, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) a.logits[(size_t)t * a.ldl + e] = val;
+    }
+    return;
+  }
+  // the routing workgroup: collect the logits
+  {
+    const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
+    const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
+    const int nw = T * Erows;
+    const unsigned local_spins = a.g_parts == GATE_PARTS ? GATE_LOCAL_SPINS : 0u;
+    bool timeout = false;
+    for (int wi = tid; wi < nw; wi += 64 * NW) {
+      unsigned spins = 0;
+      u32x2_t word;
+      for (;;) {
+        if (spins < local_spins) {
+          word = __builtin_amdgcn_raw_buffer_load_b64(rl, wi * 8, 0, 16 /* sc1: past the first-level cache */);
+        } else {
+          const unsigned long long w64 = __hip_atomic_load(cg + wi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+        }
+        if ((int)word.y == a.g_seq) break;
+        if (++spins >= GATE_POLL_LIMIT) { timeout = true; break; }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const int t = wi / Erows;
+      s_logits[t * GROUTE_MAX_ROWS + (wi - t * Erows)] = __uint_as_float(word.x);
+    }
+    if (timeout && a.err) moe_raise_err(a.err);
+  }
+  __syncthreads();
+  RouteArgs b = a;
+  b.logits = s_logits;  // (generic loads from LDS)
+  b.ldl = GROUTE_MAX_ROWS;
+  route_tail<NW, false>(b, s_idx, s_mask, s_off, s_wsum, s_wact, s_tot);
 }
 
 // Work item of a GEMV workgroup, resolved from the kernel arguments without dependent
@@ -3354,6 +3437,53 @@ extern "C" int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int
   else hipLaunchKernelGGL(k_topk_dispatch<16>, dim3(1), dim3(1024), 0, (hipStream_t)stream, a);
   moe_ktimer_end(MOE_K_TOPK, (hipStream_t)stream);
   return moe_check_launch("k_topk_dispatch");
+}
+
+// Bytes of the hand-over area of moe_gate_topk_dispatch for batches of up to T tokens over Erows gate rows
+// (zeroed once by the caller; also large enough for moe_decode_token_int4_gate on the same area)
+extern "C" int64_t moe_gate_route_ws_bytes(int T, int Erows) {
+  if (T < 1 || Erows < 1) return 0;
+  const int64_t words = (int64_t)T * Erows > GATE_COPY_WORDS ? (int64_t)T * Erows : GATE_COPY_WORDS;
+  return (int64_t)GATE_COPIES * words * 8;
+}
+
+extern "C" int moe_gate_topk_dispatch(const void *x, const void *wg, const float *bias, int n_bias, float *logits, int T,
+                                      int H, int E, int Erows, int ldl, int k, int mode, int *idx, float *w, int *counts,
+                                      int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok, moe_unit *units,
+                                      int *n_active, int64_t *active_ids, int max_units, moe_unit *units_host_out,
+                                      int *n_active_host_out, int *seq_host_out, int seq_value, void *gate_ws,
+                                      int gate_seq, int parts, int *err, void *stream) {
+  if (!x || !wg || !logits || !idx || !w || !counts || !offsets || !sorted_pair || !pos_of_pair || !sorted_tok || !units ||
+      !n_active || !active_ids || !gate_ws || !err || T < 2 || T > 32 || H <= 0 || H % 8 || E <= 0 || E > 256 ||
+      Erows < E || Erows > E + 1 || ldl < Erows || k <= 0 || k > 32 || k > E || T * k > ROUTE_MAXP || mode < 0 || mode > 2 ||
+      max_units < 0 || n_bias < 0 || n_bias > Erows || gate_seq == 0 || (parts != 1 && parts != GATE_PARTS) ||
+      (units_host_out && (!n_active_host_out || !seq_host_out))) {
+    moe_set_error("moe_gate_topk_dispatch: bad argument (T=%d H=%d E=%d rows=%d k=%d)", T, H, E, Erows, k);
+    return MOE_EINVAL;
+  }
+  RouteArgs a;
+  memset(&a, 0, sizeof a);
+  a.x = (const uint16_t *)x; a.wg = (const uint16_t *)wg; a.bias = bias; a.n_bias = bias ? n_bias : 0;
+  a.logits = logits; a.T = T; a.H = H; a.E = E; a.Erows = Erows; a.ldl = ldl; a.k = k; a.mode = mode;
+  while ((1 << a.nbits) < E) ++a.nbits;
+  a.max_units = max_units; a.idx = idx; a.w = w; a.counts = counts; a.offsets = offsets;
+  a.sorted_pair = sorted_pair; a.pos_of_pair = pos_of_pair; a.sorted_tok = sorted_tok;
+  a.units = units; a.n_active = n_active; a.active_ids = (long long *)active_ids;
+  a.host_units = units_host_out; a.host_n_active = n_active_host_out; a.host_seq = seq_host_out; a.host_seq_val = seq_value;
+  a.g_stamp = (unsigned long long *)gate_ws; a.g_seq = gate_seq; a.err = err;
+  a.g_copy_words = T * Erows > GATE_COPY_WORDS ? T * Erows : GATE_COPY_WORDS;
+  a.g_parts = parts;
+  hipStream_t s = (hipStream_t)stream;
+  moe_ktimer_begin(MOE_K_TOPK, s);
+  if (T <= 4) {
+    const int items = T * ((Erows + 3) / 4);
+    hipLaunchKernelGGL(k_gate_route<4>, dim3(1 + parts * items), dim3(256), 0, s, a);
+  } else {
+    const int items = T * ((Erows + 15) / 16);
+    hipLaunchKernelGGL(k_gate_route<16>, dim3(1 + parts * items), dim3(1024), 0, s, a);
+  }
+  moe_ktimer_end(MOE_K_TOPK, s);
+  return moe_check_launch("k_gate_route");
 }
 
 extern "C" int moe_combine_splits(const float *part_r, const float *part_s, const float *topk_w,

@@ -120,6 +120,29 @@ def topk_dispatch(logits: torch.Tensor, k: int, E: int, mode: int = L.ROUTE_SOFT
     return idx, w, d
 
 
+def gate_topk_dispatch(x, wg, bias, E: int, k: int, mode: int, gws: "GateWorkspace", parts: int = 1):
+    """Gate logits, top-k and dispatch in one launch for 2 <= T <= 32.  wg may carry one extra row (shared gate,
+    no bias).  Returns (logits [T, rows], idx, w, Dispatch, err int32[1])."""
+    T, H = x.shape
+    rows = wg.shape[0]
+    dev = x.device
+    need = int(lib.moe_gate_route_ws_bytes(T, rows))
+    if gws.buf.numel() < need:
+        raise L.MoeError("gate workspace of %d bytes, %d needed" % (gws.buf.numel(), need))
+    logits = torch.empty(T, rows, dtype=torch.float32, device=dev)
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    w = torch.empty(T, k, dtype=torch.float32, device=dev)
+    d = Dispatch(T, k, E, min(E, T * k), dev)
+    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    check(lib.moe_gate_topk_dispatch(ptr(_dev(x)), ptr(_dev(wg)), ptr(bias), E if bias is not None else 0, ptr(logits),
+                                     T, H, E, rows, rows, k, mode, ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
+                                     ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                     ptr(d.n_active), ptr(d.active_ids), d.max_units, 0, 0, 0, 0, ptr(gws.buf),
+                                     gws.next_seq(), parts, ptr(err), cur_stream()),
+          "moe_gate_topk_dispatch")
+    return logits, idx, w, d, err
+
+
 _route_counter = {}
 
 
@@ -172,8 +195,9 @@ class GateWorkspace:
     """Hand-over area of the launches that compute the gate logits themselves (moe_decode_token_int4_gate):
     zeroed once; every call takes the next sequence number."""
 
-    def __init__(self, dev):
-        self.buf = torch.zeros(int(lib.moe_gate_ws_bytes()), dtype=torch.uint8, device=dev)
+    def __init__(self, dev, T: int = 1, rows: int = 1):
+        nbytes = max(int(lib.moe_gate_ws_bytes()), int(lib.moe_gate_route_ws_bytes(T, rows)))
+        self.buf = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         self.seq = 0
 
     def next_seq(self) -> int:

@@ -430,3 +430,40 @@ def test_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode
     assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
     for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active", "units", "active_ids"):
         assert torch.equal(getattr(d, name), getattr(d2, name)), name
+
+
+@pytest.mark.parametrize("parts", [1, 8])
+@pytest.mark.parametrize("T,E,k,mode,H,rows_extra,with_bias",
+                         [(2, 64, 6, 0, 2048, 0, False), (4, 64, 6, 0, 2048, 0, False), (16, 64, 6, 1, 2048, 1, True),
+                          (16, 60, 4, 2, 2048, 1, False), (7, 200, 8, 0, 1024, 0, True), (5, 8, 2, 2, 4096, 0, False),
+                          (3, 256, 32, 0, 520, 1, True), (32, 64, 6, 0, 2048, 0, False), (32, 16, 8, 1, 3584, 1, False)])
+def test_gate_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k, mode, H, rows_extra, with_bias, parts):
+    """The launch that sums the gate rows and routes (workgroup 0 polls the logits the others hand over) against
+    the gate launch followed by the routing launch: same bits everywhere, on three calls that share a workspace."""
+    from promoe_amd import ops
+    print(f"case gate_topk_dispatch T={T} E={E} k={k} mode={mode} H={H} rows={E + rows_extra} bias={with_bias} parts={parts}",
+          flush=True)
+    rng = np.random.default_rng(T * 977 + E * 31 + k + H)
+    rows = E + rows_extra
+    wg = torch.from_numpy(rng.normal(0, 0.05, (rows, H)).astype(np.float32)).to(cuda).to(torch.bfloat16)
+    wg[E // 2] = wg[1]          # ties
+    bias = torch.from_numpy(rng.normal(0, 0.3, E).astype(np.float32)).to(cuda) if with_bias else None
+    if bias is not None:
+        bias[E // 2] = bias[1]
+    gws = ops.GateWorkspace(cuda, 32, 257)
+    for rep in range(3):
+        x = torch.from_numpy(rng.normal(0, 1, (T, H)).astype(np.float32)).to(cuda).to(torch.bfloat16)
+        lg = torch.empty(T, rows, dtype=torch.float32, device=cuda)
+        lg_e = ops.gate_logits(x, wg[:E].contiguous(), bias)
+        lg[:, :E] = lg_e
+        if rows_extra:
+            lg[:, E:] = ops.gate_logits(x, wg[E:].contiguous(), None)
+        idx, w, d = ops.topk_dispatch(lg, k, E, mode)
+        lg2, idx2, w2, d2, err = ops.gate_topk_dispatch(x, wg, bias, E, k, mode, gws, parts=parts)
+        torch.cuda.synchronize()
+        assert int(err.item()) == 0
+        assert torch.equal(lg.view(torch.int32), lg2.view(torch.int32))
+        assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+        for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active", "units", "active_ids"):
+            assert torch.equal(getattr(d, name), getattr(d2, name)), name
+    assert gws.seq == 3
