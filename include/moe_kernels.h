@@ -168,6 +168,24 @@ int moe_gate_topk_dispatch(const void *x_bf16, const void *wg_bf16, const float 
                            moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
                            void *gate_ws, int gate_seq, int parts, int *err, void *stream);
 
+/* k1a + k1b + k2 + the w13 half of k3 in ONE launch for decode batches of 2 to 8 tokens (reference: the gate's
+ * linear layer, top-k, expert grouping and the experts' first two projections of the patched sparse block,
+ * utils/__init__.py:84-141): the launch sums the gate rows in its first workgroups, every workgroup of a unit slot
+ * derives the routing itself from the handed-over logits, and one workgroup publishes the routing (all arrays of
+ * moe_topk_dispatch, bit for bit, and the optional host copy).  Results equal moe_gate_topk_dispatch followed by
+ * moe_experts_decode_int4, bit for bit.  phases: bit 0 = that launch, bit 1 = the w2 launch over the published
+ * unit list.  max_units must be min(E, T k); gate_ws / gate_seq as in moe_gate_topk_dispatch
+ * (moe_gate_route_ws_bytes(T, n_gate_rows) bytes).  moe_decode_batch_int4_gate_fits says whether a shape is taken. */
+int moe_decode_batch_int4_gate_fits(int T, int E, int k, int H, int I, int I_sh, int n_gate_rows);
+int moe_decode_batch_int4_gate(const void *x_bf16, int T, const void *gate_w_bf16, const float *gate_bias,
+                               int n_gate_rows, void *gate_ws, int gate_seq, float *logits, int ldl, int E, int k,
+                               int mode, int H, int I, int I_sh, const uint64_t *expert_ptr, const void *shared_ptr,
+                               int *idx, float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
+                               int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
+                               void *h_r, void *h_s, float *part_r, float *part_s, int *err,
+                               moe_unit *units_host_out, int *n_active_host_out, int *seq_host_out, int seq_value,
+                               int phases, void *stream);
+
 /* k3 (decode): int4 grouped SwiGLU expert product through the slot table.
  *   expert_ptr[e] : device address of expert e's slot (0 = not resident -> *err |= 1)
  *   shared_ptr    : resident shared expert (intermediate I_sh) or NULL

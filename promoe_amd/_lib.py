@@ -59,6 +59,9 @@ _sig("moe_topk_dispatch", [vp, i32, i32, i32, i32, i32] + [vp] * 10 + [i32, vp, 
 _sig("moe_gate_route_ws_bytes", [i32, i32], i64)
 _sig("moe_gate_topk_dispatch", [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 10 +
      [i32, vp, vp, vp, i32, vp, i32, i32, vp, vp])
+_sig("moe_decode_batch_int4_gate_fits", [i32] * 7, i32)
+_sig("moe_decode_batch_int4_gate", [vp, i32, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 12 +
+     [i32] + [vp] * 8 + [i32, i32, vp])
 _sig("moe_noalloc_scratch_bytes", [], i64)
 _sig("moe_decode_token_int4_noalloc", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp])
 _sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])

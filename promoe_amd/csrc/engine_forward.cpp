@@ -343,6 +343,14 @@ static int route_batch(const moe_layer_desc &d, LayerState *s, const void *x, in
                            max_units, host_units, host_n, host_seq, seq_val, st);
 }
 
+// a decode batch whose w13 launch computes the gate logits and routes by itself (int4, 2 to 8 tokens)
+static bool batch_routes_in_w13(const moe_layer_desc &d, const LayerState *s, int T, int E, int k, int n_gate_rows) {
+  static const bool on = [] { const char *e = getenv("MOE_BATCH_ROUTE"); return !e || atoi(e) != 0; }();
+  return on && d.fmt == MOE_FMT_INT4_G128 && !use_prefill(d, T) &&
+         moe_decode_batch_int4_gate_fits(T, E, k, d.H, d.I, d.I_sh, n_gate_rows) &&
+         moe_gate_route_ws_bytes(T, n_gate_rows) <= (int64_t)s->gate_ws_bytes;
+}
+
 extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, void *y) {
   if (!eng) { moe_set_error("null engine"); return MOE_EINVAL; }
   if (!eng->fatal.empty()) { moe_set_error("engine is in a failed state: %s", eng->fatal.c_str()); return MOE_ESTATE; }
@@ -580,6 +588,31 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   }
   bool routed_by_tail = false, w13_publishes = false;
   int tail_seq = 0, host_seq = 0;  // host_seq != 0: the unit list comes to units_host with this value in *opt_seq
+  if (all_resident && batch_routes_in_w13(d, s, T, E, k, n_gate_rows)) {
+    // 2 to 8 tokens, nothing for the host to decide: the w13 launch sums the gate rows, routes by itself and hands
+    // the unit list to the host through the pending slot's pinned memory; then w2 and the combine (three launches)
+    LayerState::Pending &p = s->pend[s->pend_head];
+    if (p.busy && (rc = moe_forward_harvest(eng, true))) return rc;
+    s->pend_head = (s->pend_head + 1) % LayerState::kPending;
+    const int seq = ++s->seq_counter;
+    const uint64_t *table = nullptr;
+    if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+    if ((rc = moe_flush_table(eng, layer, st))) return rc;
+    s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
+    if ((rc = moe_decode_batch_int4_gate(x, T, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, ldl, E,
+                                         k, d.route_mode, d.H, d.I, d.I_sh, table, d.I_sh > 0 ? d.shared : nullptr, s->idx,
+                                         s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
+                                         s->units, s->n_active, s->active_ids, max_units, s->h_r, s->h_s, s->part_r,
+                                         s->part_s, s->err_host + layer, p.units, p.n_active, p.seq, seq, 3, st)))
+      return rc;
+    p.layer = layer; p.max_units = max_units; p.busy = true; p.by_seq = true; p.seq_expected = seq;
+    const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
+    if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k,
+                                 1, st)))
+      return rc;
+    if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    return moe_layer_done(eng, layer);
+  }
   if (all_resident && T <= 32 && E <= 256 && k <= 32 && T * k <= 512) {
     // decode batch, nothing for the host to decide: logits, then top-k + dispatch in one launch that
     // also hands the unit list to the host through the next pending slot's pinned memory

@@ -753,6 +753,9 @@ struct GemvArgs {
   int pairs;                    // T k of the step (0: unknown)
   int row_split;                // w2 launches of more than 32 tokens: a unit of more than 32 rows has two workgroups
                                 // per group of block pairs, rows 0..31 and 32.., and so has the shared expert
+  // w13 launches of a decode batch that sum the gate rows and route by themselves (k_gemv_int4_mfma<.., ROUTE>):
+  // 8-byte words per copy of the hand-over area, row stride of the logits in memory
+  int g_copy_words, g_ldl;
 };
 
 // Gate logits handed over inside a launch.  A logit travels as one 8-byte word (value, sequence number of the
@@ -1206,6 +1209,227 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
   if (a.r_E <= 64) return gemv_resolve_route_n<1>(a, lane, w, bx);
   if (a.r_E <= 128) return gemv_resolve_route_n<2>(a, lane, w, bx);
   return gemv_resolve_route_n<4>(a, lane, w, bx);
+}
+
+// ---------------------------------------------------------------------------
+// Decode batches of 2 to 8 tokens whose w13 launch sums the gate rows and routes by itself (the step is then
+// three launches: this one, w2, combine).  Grid: the gate workgroups (a token and four gate rows each, a wave per
+// row, once per part of the chip: see gate_rows_stamped), ONE workgroup that publishes the routing for the later
+// launches and the host (the routing workgroup of k_gate_route), the shared expert's workgroups, then one set of
+// workgroups per unit slot (min(E, T k) slots).  A workgroup of slot u derives the routing itself: wave w takes
+// the tokens w, w + 4 (polls their logit words in the copy of its part of the chip, k rounds of wave-wide
+// maxima: the selection and tie rule of topk_token) and leaves every token's experts as a bit mask in LDS; after
+// one barrier every wave counts, per expert (a lane per expert and 64-wide column), the tokens that chose it,
+// finds the u-th expert in use (units are in expert order), its rows' first position (the counts of all experts
+// below it, from ballots of the count's bits) and the tokens of the unit as a bit mask (a token holds an expert
+// at most once, so a unit's rows are its tokens in token order).  Every workgroup works from the same words with
+// the same rounds, so all of them and the publisher agree.
+// ---------------------------------------------------------------------------
+#define RB_MAXT 8
+static __device__ __forceinline__ void gate_rows_batch(const GemvArgs &a, const int lane, const int w, const int q) {
+  const int Erows = a.g_rows, H = a.cls[1].K;
+  const int item = q >> 3;
+  const int nrb = (Erows + 3) >> 2;
+  const int t = item / nrb, e = (item - t * nrb) * 4 + w;
+  if (e >= Erows) return;
+  const bool biased = a.g_bias && e < a.g_nbias;
+  const float bias_e = biased ? a.g_bias[e] : 0.f;
+  asm volatile("" :: "v"(bias_e));  // requested in front of the row
+  const float acc = gate_row_sum(a.cls[1].act + (size_t)t * H, a.g_w + (size_t)e * H, H, lane);
+  const float val = biased ? acc + bias_e : acc;
+  const u32x2_t word = {__float_as_uint(val), (u32)a.g_seq};
+  const int wi = t * Erows + e;
+  if (lane == 0)
+    __builtin_amdgcn_raw_buffer_store_b64(word, make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words,
+                                                          (u32)a.g_copy_words * 8u), wi * 8, 0, 1 /* sc0 */);
+  if ((q & 7) == 0) {
+    const unsigned long long word64 = ((unsigned long long)word.y << 32) | word.x;
+    if (lane == 1)
+      __hip_atomic_store(a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words + wi, word64, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) a.g_logits_out[(size_t)t * a.g_ldl + e] = val;
+  }
+}
+
+// LDS the publishing workgroup of such a launch takes from the launch's dynamic area
+#define RB_PUBLISH_LDS (2048 + 2048 + 1040 + 48 + RB_MAXT * GROUTE_MAX_ROWS * 4)
+static __device__ __forceinline__ void route_publish_batch(const GemvArgs &a, unsigned char *smem) {
+  int *s_idx = (int *)smem;                                            // [ROUTE_MAXP]
+  unsigned long long *s_mask = (unsigned long long *)(smem + 2048);    // [RB_MAXT .. ROUTE_MAXT][4]
+  int *s_off = (int *)(smem + 4096);                                   // [257]
+  int *s_wsum = (int *)(smem + 4096 + 1040), *s_wact = s_wsum + 4, *s_tot = s_wsum + 8;
+  float *s_logits = (float *)(smem + 4096 + 1040 + 48);                // [T][GROUTE_MAX_ROWS]
+  const int tid = threadIdx.x;
+  const int T = a.T, Erows = a.g_rows;
+  {
+    const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
+    const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
+    const int nw = T * Erows;
+    bool timeout = false;
+    for (int wi = tid; wi < nw; wi += 256) {
+      unsigned spins = 0;
+      u32x2_t word;
+      for (;;) {
+        if (spins < GATE_LOCAL_SPINS) {
+          word = __builtin_amdgcn_raw_buffer_load_b64(rl, wi * 8, 0, 16 /* sc1: past the first-level cache */);
+        } else {
+          const unsigned long long w64 = __hip_atomic_load(cg + wi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+        }
+        if ((int)word.y == a.g_seq) break;
+        if (++spins >= GATE_POLL_LIMIT) { timeout = true; break; }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      const int t = wi / Erows;
+      s_logits[t * GROUTE_MAX_ROWS + (wi - t * Erows)] = __uint_as_float(word.x);
+    }
+    if (timeout) moe_raise_err(a.err);
+  }
+  __syncthreads();
+  RouteArgs b;
+  b.x = nullptr; b.wg = nullptr; b.bias = nullptr;
+  b.logits = s_logits; b.T = T; b.H = a.cls[1].K; b.E = a.r_E; b.Erows = Erows; b.ldl = GROUTE_MAX_ROWS; b.k = a.r_k;
+  b.mode = a.r_mode; b.nbits = 0; b.max_units = a.p_max_units;
+  b.idx = a.r_idx; b.w = a.r_w; b.counts = a.r_counts; b.offsets = a.r_offsets; b.sorted_pair = a.r_sorted_pair;
+  b.pos_of_pair = a.r_pos_of_pair; b.sorted_tok = a.r_sorted_tok; b.units = a.r_units; b.n_active = a.r_n_active;
+  b.active_ids = a.r_active_ids; b.counter = nullptr;
+  b.host_units = a.r_host_units; b.host_n_active = a.p_host_n_active; b.host_seq = a.r_host_seq;
+  b.host_seq_val = a.r_host_seq_val; b.pad_ = 0;
+  b.n_bias = 0; b.g_seq = 0; b.g_copy_words = 0; b.g_parts = 0; b.g_stamp = nullptr; b.err = a.err;
+  route_tail<4, false>(b, s_idx, s_mask, s_off, s_wsum, s_wact, *s_tot);
+}
+
+// rr: the workgroup's index among those of the unit slots.  tokmask: the unit's tokens.
+template <int NR>
+static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const GemvArgs &a, const int lane, const int w,
+                                                                      const int rr, unsigned &tokmask) {
+  __shared__ unsigned long long s_sel[RB_MAXT][4];
+  GemvWork wk;
+  wk.c = a.cls[1];
+  const int E = a.r_E, k = a.r_k, T = a.T, Erows = a.g_rows;
+  const int u = rr / wk.c.nblk;
+  wk.b = rr - u * wk.c.nblk;
+  wk.half = 0;
+  const float NEG = -__builtin_inff();
+  unsigned long long ptrs[NR];  // slot addresses of the lane's experts, requested in front of the logits
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const int e = lane + 64 * r;
+    ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
+  }
+  const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
+  const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
+  for (int t = w; t < T; t += 4) {
+    float v[NR];
+    bool gate_timeout = false;
+    unsigned spins = 0;
+    for (;;) {
+      bool ok = true;
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const int e = lane + 64 * r;
+        v[r] = NEG;
+        if (e < E) {
+          u32x2_t word;
+          if (spins < GATE_LOCAL_SPINS) {
+            word = __builtin_amdgcn_raw_buffer_load_b64(rl, (t * Erows + e) * 8, 0, 16 /* sc1: past the first-level cache */);
+          } else {
+            const unsigned long long w64 = __hip_atomic_load(cg + t * Erows + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+          }
+          v[r] = __uint_as_float(word.x);
+          ok = ok && (int)word.y == a.g_seq;
+        }
+      }
+      if (__ballot(!ok) == 0ull) break;
+      if (++spins >= GATE_POLL_LIMIT) { gate_timeout = true; break; }  // (the launch then reports an error)
+      __builtin_amdgcn_s_sleep(2);
+    }
+    unsigned long long msel[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) msel[r] = 0ull;
+    for (int j = 0; j < k; ++j) {
+      float bv = v[0];
+#pragma unroll
+      for (int r = 1; r < NR; ++r) bv = fmaxf(bv, v[r]);
+      const float best = wave_max_f32(bv);
+      int wr = -1, wl = 0;
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const unsigned long long mr = __ballot(v[r] == best);
+        if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
+      }
+      if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+        if (r == wr) {
+          if (lane == wl) v[r] = NEG;
+          msel[r] |= 1ull << wl;
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < NR; ++r) s_sel[t][r] = gate_timeout ? 0ull : msel[r];
+      if (gate_timeout) moe_raise_err(a.err);
+    }
+  }
+  __syncthreads();
+  // per expert (this lane's, per column): its tokens
+  int cnt[NR];
+  unsigned mk[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) { cnt[r] = 0; mk[r] = 0u; }
+  for (int t = 0; t < T; ++t) {
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+      const unsigned bit = (unsigned)((s_sel[t][r] >> lane) & 1ull);
+      cnt[r] += (int)bit;
+      mk[r] |= bit << t;
+    }
+  }
+  int cum_act = 0, cum_rows = 0, m = 0, row0 = 0;
+  unsigned tm = 0u, lo = 0u, hi = 0u;
+  bool found = false;
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    const unsigned long long actm = __ballot(cnt[r] > 0);
+    const unsigned long long b0 = __ballot((cnt[r] & 1) != 0), b1 = __ballot((cnt[r] & 2) != 0),
+                             b2 = __ballot((cnt[r] & 4) != 0), b3 = __ballot((cnt[r] & 8) != 0);
+    const int na = __popcll(actm);
+    if (!found && u < cum_act + na) {
+      unsigned long long mm = actm;
+      for (int i = 0; i < u - cum_act; ++i) mm &= mm - 1;
+      const int src = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(mm));  // expert 64 r + src
+      const unsigned long long sb = (1ull << src) - 1ull;
+      row0 = cum_rows + __popcll(b0 & sb) + 2 * __popcll(b1 & sb) + 4 * __popcll(b2 & sb) + 8 * __popcll(b3 & sb);
+      m = __builtin_amdgcn_readlane(cnt[r], src);
+      tm = (unsigned)__builtin_amdgcn_readlane((int)mk[r], src);
+      lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)ptrs[r], src);
+      hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(ptrs[r] >> 32), src);
+      found = true;
+    }
+    cum_act += na;
+    cum_rows += __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2) + 8 * __popcll(b3);
+  }
+  wk.m = found ? m : 0;
+  wk.row0 = row0;
+  tokmask = tm;
+  wk.base = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+  return wk;
+}
+
+static __device__ __forceinline__ GemvWork gemv_resolve_route_batch(const GemvArgs &a, int lane, int w, int rr, unsigned &tokmask) {
+  if (a.r_E <= 64) return gemv_resolve_route_batch_n<1>(a, lane, w, rr, tokmask);
+  if (a.r_E <= 128) return gemv_resolve_route_batch_n<2>(a, lane, w, rr, tokmask);
+  return gemv_resolve_route_batch_n<4>(a, lane, w, rr, tokmask);
+}
+
+// the i-th token (i-th set bit) of a unit's token mask
+static __device__ __forceinline__ int nth_token(unsigned mask, const int i) {
+#pragma unroll
+  for (int q = 0; q < RB_MAXT - 1; ++q)
+    if (q < i) mask &= mask - 1u;
+  return mask ? __builtin_ctz(mask) : 0;
 }
 
 template <int TMAX, bool SWIGLU, int CH, bool DEVUNITS, bool Q4K = false>
@@ -1753,7 +1977,9 @@ static __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &x) {
   return __builtin_bit_cast(bf16x8_t, v);
 }
 
-template <bool SWIGLU, int CH, bool DEVUNITS>
+// ROUTE (w13 pass, device-side slot table): the launch sums the gate rows and routes by itself, see
+// gemv_resolve_route_batch_n; a unit's token rows then come from its token mask, not from a list in memory
+template <bool SWIGLU, int CH, bool DEVUNITS, bool ROUTE = false>
 __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW_R, const int RPW_S) {
   constexpr int NP = 1, NB = 2 * NP;  // block pairs / 16-row blocks per iteration
   constexpr int PF = 4;               // activation pieces in flight while staging
@@ -1763,13 +1989,29 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   const Q4Consts q4c = q4_consts();
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
-  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
+  const bool publishes = !ROUTE && SWIGLU && DEVUNITS && a.p_host_units != nullptr;
   if (publishes && blockIdx.x == 0) {
     gemv_publish_units(a);
     return;
   }
-  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
-  const GemvWork wk = gemv_resolve<DEVUNITS>(a, bx);
+  int bx = (int)blockIdx.x - (publishes ? 1 : 0);
+  unsigned tokmask = 0u;   // ROUTE: the tokens of a routed unit
+  bool masked = false;
+  GemvWork wk;
+  if constexpr (ROUTE) {
+    if (bx < a.g_nblk) { gate_rows_batch(a, lane, w, bx); return; }
+    bx -= a.g_nblk;
+    if (bx == 0) { route_publish_batch(a, smem); return; }
+    bx -= 1;
+    if (bx < a.n_sh_blocks) {
+      wk.c = a.cls[0]; wk.b = bx; wk.half = 0; wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
+    } else {
+      wk = gemv_resolve_route_batch(a, lane, w, bx - a.n_sh_blocks, tokmask);
+      masked = true;
+    }
+  } else {
+    wk = gemv_resolve<DEVUNITS>(a, bx);
+  }
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -1805,7 +2047,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
     const rsrc_t rz = make_rsrc(base + c.off_z + (size_t)rbA * G * 8, (u32)NB * G * 8u);
     // ---- straight-line load section ------------------------------------------------------
     const int row_first = row0 + t0;
-    const int arow0 = c.gather ? c.gather[row_first] : row_first;
+    const int arow0 = (ROUTE && masked) ? __builtin_amdgcn_readfirstlane(nth_token(tokmask, t0))
+                                        : (c.gather ? c.gather[row_first] : row_first);
     const uint4 xv0 = bload16(rx, (tid < vec_per_row ? tid : 0) * 16, arow0 * c.act_stride * 2);
     // scale dword e = (block, group, row pair j) and the zero dword that holds its two nibbles
     const int zoff = ((tid >> 3) * 2 + ((tid & 7) >> 2)) * 4;
@@ -1838,7 +2081,8 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
       const int total = mc * cpr;
       // row index of every token of this pass, one per lane (lanes >= mc repeat the last)
       const int grow = row_first + (lane < mc ? lane : mc - 1);
-      const int arow_l = c.gather ? c.gather[grow] : grow;
+      const int arow_l = (ROUTE && masked) ? nth_token(tokmask, t0 + (lane < mc ? lane : mc - 1))
+                                           : (c.gather ? c.gather[grow] : grow);
       for (int pb = 1; pb < total; pb += PF) {
         uint4 xb[PF];
 #pragma unroll
@@ -2832,20 +3076,28 @@ static size_t gemv_mfma_lds(int tb, int K, int nb) {
          (size_t)4 * nb * 256 * 4;
 }
 
+// Routed block pairs per workgroup of the whole-row matrix-core GEMV and what the shared expert's workgroups take
+// (see launch_gemv_mfma)
+static void gemv_mfma_rpw(const GemvArgs &a, int units, int *rpw_out, int *rpw_s_out) {
+  int rpw = 1;
+  while (rpw < 4 && units * a.cls[1].nblk / (rpw * 2) >= 1024 && a.cls[1].nblk % (rpw * 2) == 0) rpw *= 2;
+  int rpw_s = 1;
+  if (a.n_sh_blocks > 0 && a.cls[0].K <= a.cls[1].K)
+    while (rpw_s < rpw && a.cls[0].nblk % (rpw_s * 2) == 0) rpw_s *= 2;
+  *rpw_out = rpw; *rpw_s_out = rpw_s;
+}
+
 template <bool SW, int CH>
 static int launch_gemv_mfma(const GemvArgs &a_in, int grid_in, int tb, size_t lds, hipStream_t s) {
   GemvArgs a = a_in;
   const int units = a.cls[1].nblk > 0 ? (grid_in - a.n_sh_blocks) / a.cls[1].nblk : 0;
-  // routed block pairs per workgroup: enough workgroups to fill the chip twice, then fewer, larger ones
-  int rpw = 1;
-  while (rpw < 4 && units * a.cls[1].nblk / (rpw * 2) >= 1024 && a.cls[1].nblk % (rpw * 2) == 0) rpw *= 2;
-  // the shared expert's workgroups stage every token row.  With a reduction longer than the routed
+  // routed block pairs per workgroup: enough workgroups to fill the chip twice, then fewer, larger ones.
+  // The shared expert's workgroups stage every token row.  With a reduction longer than the routed
   // experts' (w2 of a wide shared expert) they are the long ones of the launch and keep one pair each:
   // four pairs each cost the 16-token step of a 2048 x 2816 shared expert about 8 us.  Otherwise they
   // take what the routed ones take (more, smaller workgroups only add staging traffic).
-  int rpw_s = 1;
-  if (a.n_sh_blocks > 0 && a.cls[0].K <= a.cls[1].K)
-    while (rpw_s < rpw && a.cls[0].nblk % (rpw_s * 2) == 0) rpw_s *= 2;
+  int rpw, rpw_s;
+  gemv_mfma_rpw(a, units, &rpw, &rpw_s);
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= rpw_s; a.n_sh_blocks /= rpw_s; }
   a.cls[1].nblk /= rpw;
   const int grid = a.n_sh_blocks + units * a.cls[1].nblk + (SW && a.units && a.p_host_units ? 1 : 0);
@@ -3089,6 +3341,105 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
     int rc = launch_gemv_t<false>(a, grid, T, I_sh > I ? I_sh : I, (max_units > 0 ? I : I_sh) / 128, s);
     if (rc) return rc;
   }
+  return MOE_OK;
+}
+
+template <int CH>
+static int launch_gemv_mfma_route(const GemvArgs &a_in, int units, int tb, size_t lds, hipStream_t s) {
+  GemvArgs a = a_in;
+  int rpw, rpw_s;
+  gemv_mfma_rpw(a, units, &rpw, &rpw_s);
+  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= rpw_s; a.n_sh_blocks /= rpw_s; }
+  a.cls[1].nblk /= rpw;
+  const int grid = a.g_nblk + 1 + a.n_sh_blocks + units * a.cls[1].nblk;
+  static bool attr_set = false;
+  if (lds > 64 * 1024 && !attr_set) {
+    if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gemv_int4_mfma<true, CH, true, true>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                               "hipFuncSetAttribute(k_gemv_int4_mfma, routing)"))
+      return rc;
+    attr_set = true;
+  }
+  moe_ktimer_begin(MOE_K_W13, s);
+  hipLaunchKernelGGL((k_gemv_int4_mfma<true, CH, true, true>), dim3(grid), dim3(256), lds, s, a, tb, rpw, rpw_s);
+  moe_ktimer_end(MOE_K_W13, s);
+  return moe_check_launch("k_gemv_int4_mfma<route>");
+}
+
+// whether moe_decode_batch_int4_gate takes a batch of T tokens of this shape
+extern "C" int moe_decode_batch_int4_gate_fits(int T, int E, int k, int H, int I, int I_sh, int n_gate_rows) {
+  if (T < 2 || T > RB_MAXT || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E || T * k > ROUTE_MAXP || H <= 0 || H % 128 ||
+      I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 || n_gate_rows < E || n_gate_rows > E + 1)
+    return 0;
+  int tb = 1;
+  while (tb < T) tb <<= 1;
+  return gemv_mfma_lds(tb, H, 2) <= 80 * 1024;  // two workgroups per compute unit (else the chunked form is the faster one)
+}
+
+extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate_w, const float *gate_bias,
+                                          int n_gate_rows, void *gate_ws, int gate_seq, float *logits, int ldl, int E,
+                                          int k, int mode, int H, int I, int I_sh, const uint64_t *expert_ptr,
+                                          const void *shared_ptr, int *idx, float *w, int *counts, int *offsets,
+                                          int *sorted_pair, int *pos_of_pair, int *sorted_tok, moe_unit *units,
+                                          int *n_active, int64_t *active_ids, int max_units, void *h_r, void *h_s,
+                                          float *part_r, float *part_s, int *err, moe_unit *units_host_out,
+                                          int *n_active_host_out, int *seq_host_out, int seq_value, int phases,
+                                          void *stream) {
+  if (!moe_decode_batch_int4_gate_fits(T, E, k, H, I, I_sh, n_gate_rows)) {
+    moe_set_error("moe_decode_batch_int4_gate: shape not taken (T=%d E=%d k=%d H=%d I=%d I_sh=%d rows=%d)", T, E, k, H, I,
+                  I_sh, n_gate_rows);
+    return MOE_EINVAL;
+  }
+  const int mu = E < T * k ? E : T * k;
+  if (!x || !gate_w || !gate_ws || gate_seq == 0 || !logits || ldl < n_gate_rows || !expert_ptr || !idx || !w || !counts ||
+      !offsets || !sorted_pair || !pos_of_pair || !sorted_tok || !units || !n_active || !active_ids || max_units != mu ||
+      !h_r || !part_r || !err || mode < 0 || mode > 2 || (shared_ptr && (!h_s || !part_s || I_sh == 0)) ||
+      (units_host_out && (!n_active_host_out || !seq_host_out))) {
+    moe_set_error("moe_decode_batch_int4_gate: bad argument (T=%d max_units=%d, %d expected)", T, max_units, mu);
+    return MOE_EINVAL;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (phases & 1) {
+    moe_int4_layout lr, ls;
+    memset(&lr, 0, sizeof lr); memset(&ls, 0, sizeof ls);
+    if (moe_int4_layout_make(H, I, &lr)) return MOE_EINVAL;
+    if (shared_ptr && moe_int4_layout_make(H, I_sh, &ls)) return MOE_EINVAL;
+    const bool sh = shared_ptr != nullptr;
+    GemvArgs a;
+    memset(&a, 0, sizeof a);
+    a.expert_ptr = (const unsigned long long *)expert_ptr;
+    a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err; a.pairs = T * k;
+    a.r_E = E; a.r_k = k; a.r_mode = mode; a.r_idx = idx; a.r_w = w; a.r_counts = counts; a.r_offsets = offsets;
+    a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok; a.r_units = units;
+    a.r_n_active = n_active; a.r_active_ids = (long long *)active_ids;
+    a.r_host_units = units_host_out; a.p_host_n_active = units_host_out ? n_active_host_out : nullptr;
+    a.r_host_seq = units_host_out ? seq_host_out : nullptr; a.r_host_seq_val = seq_value; a.p_max_units = max_units;
+    a.g_w = (const uint16_t *)gate_w; a.g_bias = gate_bias; a.g_stamp = (unsigned long long *)gate_ws;
+    a.g_logits_out = logits; a.g_ldl = ldl; a.g_rows = n_gate_rows; a.g_nbias = gate_bias ? E : 0; a.g_seq = gate_seq;
+    a.g_copy_words = T * n_gate_rows > GATE_COPY_WORDS ? T * n_gate_rows : GATE_COPY_WORDS;
+    a.g_nblk = GATE_PARTS * T * ((n_gate_rows + 3) / 4);
+    a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, H, I_sh, I_sh / 16, 0};
+    a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, H, I, I / 16, 0};
+    a.n_sh_blocks = sh ? I_sh / 16 : 0;
+    int tb = 1;
+    while (tb < T) tb <<= 1;
+    size_t lds = gemv_mfma_lds(tb, H, 2);
+    if (lds < RB_PUBLISH_LDS) lds = RB_PUBLISH_LDS;
+    const int gpw = (H / 128 + 3) / 4;
+    int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
+    if (ch < 1) ch = 1;
+    int rc;
+    switch (ch) {
+      case 1: rc = launch_gemv_mfma_route<1>(a, max_units, tb, lds, s); break;
+      case 2: rc = launch_gemv_mfma_route<2>(a, max_units, tb, lds, s); break;
+      case 3: rc = launch_gemv_mfma_route<3>(a, max_units, tb, lds, s); break;
+      default: rc = launch_gemv_mfma_route<4>(a, max_units, tb, lds, s); break;
+    }
+    if (rc) return rc;
+  }
+  if (phases & 2)  // w2 over the unit list the first launch published
+    return moe_experts_decode_int4(x, T, H, I, shared_ptr ? I_sh : 0, k, units, max_units, sorted_tok, expert_ptr, shared_ptr,
+                                   h_r, h_s, part_r, part_s, err, nullptr, nullptr, 2, stream);
   return MOE_OK;
 }
 

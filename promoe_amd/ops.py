@@ -205,6 +205,42 @@ class GateWorkspace:
         return self.seq
 
 
+def decode_batch_int4_gate_fits(T: int, E: int, k: int, H: int, I: int, I_sh: int, rows: int) -> bool:
+    return bool(lib.moe_decode_batch_int4_gate_fits(T, E, k, H, I, I_sh, rows))
+
+
+def decode_batch_int4_gate(x, wg, bias, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int,
+                           gws: "GateWorkspace", phases: int = 3):
+    """2 to 8 tokens: gate rows, routing and w13 in one launch (phase bit 0), w2 over the published unit list (bit 1).
+    wg may carry one extra row (shared gate, no bias).
+    Returns (logits [T, rows], idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
+    T = x.shape[0]
+    rows = wg.shape[0]
+    dev = x.device
+    P = T * k
+    logits = torch.empty(T, rows, dtype=torch.float32, device=dev)
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    w = torch.empty(T, k, dtype=torch.float32, device=dev)
+    d = Dispatch(T, k, E, min(E, P), dev)
+    h_r = torch.empty(P, I, dtype=torch.bfloat16, device=dev)
+    part_r = torch.empty(P, H, dtype=torch.float32, device=dev)
+    h_s = part_s = None
+    if shared is not None:
+        h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
+        part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    if gws.buf.numel() < int(lib.moe_gate_route_ws_bytes(T, rows)):
+        raise L.MoeError("gate workspace too small")
+    check(lib.moe_decode_batch_int4_gate(ptr(_dev(x)), T, ptr(_dev(wg)), ptr(bias), rows, ptr(gws.buf), gws.next_seq(),
+                                         ptr(logits), rows, E, k, mode, H, I, I_sh if shared is not None else 0,
+                                         ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
+                                         ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                         ptr(d.n_active), ptr(d.active_ids), d.max_units, ptr(h_r), ptr(h_s),
+                                         ptr(part_r), ptr(part_s), ptr(err), 0, 0, 0, 0, phases, cur_stream()),
+          "moe_decode_batch_int4_gate")
+    return logits, idx, w, d, part_r, part_s, err, h_r, h_s
+
+
 def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int, ws=None,
                       phases: int = 3, unit_ws=None, sg_logit=None, y=None, gate=None):
     """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s).

@@ -12,6 +12,7 @@ STUB(moe_dispatch_ws)
 STUB(moe_route_decode)
 STUB(moe_topk_dispatch)
 STUB(moe_gate_topk_dispatch)
+STUB(moe_decode_batch_int4_gate)
 STUB(moe_experts_decode_int4)
 STUB(moe_experts_decode_int4_publish)
 STUB(moe_decode_token_int4)
@@ -28,3 +29,4 @@ extern "C" int64_t moe_prefill_workspace_bytes(...) { return 0; }
 extern "C" int64_t moe_dispatch_workspace_bytes(...) { return 0; }
 extern "C" int64_t moe_gate_ws_bytes(...) { return 64; }
 extern "C" int64_t moe_gate_route_ws_bytes(...) { return 64; }
+extern "C" int moe_decode_batch_int4_gate_fits(...) { return 0; }

@@ -467,3 +467,53 @@ def test_gate_topk_dispatch_in_one_launch_equals_separate_kernels(cuda, T, E, k,
         for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active", "units", "active_ids"):
             assert torch.equal(getattr(d, name), getattr(d2, name)), name
     assert gws.seq == 3
+
+
+@pytest.mark.parametrize("T,H,I,E,k,mode,I_sh,zipf,gated", [
+    (4, 2048, 1408, 64, 6, 0, 2816, 1.2, False), (2, 2048, 1408, 64, 6, 0, 2816, 1.2, False),
+    (8, 2048, 1408, 64, 6, 1, 2816, 1.2, True), (3, 256, 384, 8, 2, 2, 256, None, True),
+    (7, 256, 256, 60, 4, 1, 512, 1.1, True), (5, 512, 128, 200, 8, 0, 0, None, False),
+    (4, 4096, 14336, 4, 2, 2, 0, None, False), (8, 1024, 128, 130, 3, 0, 128, 1.1, True),
+    (6, 384, 256, 256, 32, 0, 0, None, False)])
+def test_batch_decode_gate_rows_and_routing_in_the_w13_launch(cuda, T, H, I, E, k, mode, I_sh, zipf, gated):
+    """2 to 8 tokens: the w13 launch sums the gate rows, every unit's workgroups route by themselves and one
+    workgroup publishes the routing.  Logits, routing arrays, h rows and partial rows must equal those of the
+    gate + routing launch followed by the expert launches, bit for bit, on successive calls over one hand-over
+    workspace."""
+    from promoe_amd import ops
+    print(f"case batch_gate T={T} H={H} I={I} E={E} k={k} mode={mode} I_sh={I_sh}", flush=True)
+    layer = Int4Layer(H=H, I=I, E=E, I_sh=I_sh, seed=11, zipf=zipf, shared_gate=gated)
+    rows = E + (1 if gated else 0)
+    assert ops.decode_batch_int4_gate_fits(T, E, k, H, I, I_sh, rows)
+    slots = [torch.from_numpy(s).to(cuda) for s in layer.slots]
+    table = torch.tensor([s.data_ptr() for s in slots], dtype=torch.int64, device=cuda)
+    shared = torch.from_numpy(layer.shared_img).to(cuda) if I_sh else None
+    wg_np = layer.wg if not gated else np.concatenate([layer.wg, layer.shared_gate[None, :]], axis=0)
+    wg = bf16_dev(wg_np, cuda)
+    bias_e = None if layer.bias is None else torch.from_numpy(layer.bias).to(cuda)
+    gws = ops.GateWorkspace(cuda, 8, 257)
+    gws_ref = ops.GateWorkspace(cuda, 8, 257)
+    P = T * k
+    for seed in range(4):
+        x = O.synth_acts(T, H, seed=seed + 70)
+        if seed == 3:   # constructed ties
+            wg = wg.clone(); wg[E // 2] = wg[1]; wg[E - 1] = wg[1]
+            if bias_e is not None:
+                bias_e = bias_e.clone(); bias_e[E // 2] = bias_e[1]; bias_e[E - 1] = bias_e[1]
+        xd = bf16_dev(x, cuda)
+        lg, idx, w, d, err0 = ops.gate_topk_dispatch(xd, wg, bias_e, E, k, mode, gws_ref)
+        part_r, part_s, err, h_r, h_s = ops.experts_decode_int4(xd, d, table, shared, H, I, I_sh)
+        lg2, idx2, w2, d2, part_r2, part_s2, err2, h_r2, h_s2 = ops.decode_batch_int4_gate(
+            xd, wg, bias_e, E, k, mode, table, shared, H, I, I_sh, gws)
+        torch.cuda.synchronize()
+        assert int(err0.item()) == 0 and int(err.item()) == 0 and int(err2.item()) == 0
+        assert torch.equal(lg.view(torch.int32), lg2.view(torch.int32))
+        assert torch.equal(idx, idx2) and torch.equal(w.view(torch.int32), w2.view(torch.int32))
+        for name in ("counts", "offsets", "sorted_pair", "pos_of_pair", "sorted_tok", "n_active", "units", "active_ids"):
+            assert torch.equal(getattr(d, name), getattr(d2, name)), name
+        assert torch.equal(h_r[:P].view(torch.int16), h_r2[:P].view(torch.int16))
+        assert torch.equal(part_r[:P].view(torch.int32), part_r2[:P].view(torch.int32))
+        if I_sh:
+            assert torch.equal(h_s.view(torch.int16), h_s2.view(torch.int16))
+            assert torch.equal(part_s.view(torch.int32), part_s2.view(torch.int32))
+    assert gws.seq == 4
