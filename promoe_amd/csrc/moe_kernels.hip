@@ -756,6 +756,11 @@ struct GemvArgs {
   // w13 launches of a decode batch that sum the gate rows and route by themselves (k_gemv_int4_mfma<.., ROUTE>):
   // 8-byte words per copy of the hand-over area, row stride of the logits in memory
   int g_copy_words, g_ldl;
+  // workgroups from this grid index on first look for the routing that an earlier workgroup on their part of the
+  // chip has left behind (they start when the first round of workgroups ends)
+  int g_cache_from;
+  int g_parts;   // 8: the gate rows are summed once per part of the chip (hand-over through that part's second-level
+                 // cache), 1: once, handed over at device scope
 };
 
 // Gate logits handed over inside a launch.  A logit travels as one 8-byte word (value, sequence number of the
@@ -1225,29 +1230,95 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route(const GemvArgs &a,
 // at most once, so a unit's rows are its tokens in token order).  Every workgroup works from the same words with
 // the same rounds, so all of them and the publisher agree.
 // ---------------------------------------------------------------------------
-#define RB_MAXT 8
-static __device__ __forceinline__ void gate_rows_batch(const GemvArgs &a, const int lane, const int w, const int q) {
-  const int Erows = a.g_rows, H = a.cls[1].K;
-  const int item = q >> 3;
+#define RB_MAXT 16
+#define RB_MAX_UNITS 256   // unit slots of such a launch: min(E, T k) <= 256
+// gate rows of a batch: a workgroup takes four gate rows (a wave per row) and TG = ceil(T / 4) tokens; the row is
+// read once and every token's sum is the fma chain of gate_row_partial over the same chunks, then the same
+// butterfly (so the bits are those of gate_row_sum); all loads of a wave go out before the first fma
+template <int NCH, int TG>
+static __device__ __forceinline__ void gate_rows_multi(const uint16_t *__restrict__ x, const uint16_t *__restrict__ wr,
+                                                       const int H, const int lane, const int t0, const int T,
+                                                       float (&out)[TG]) {
+  uint4 wq[NCH], xq[TG][NCH];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int k = c * 512 + 8 * lane;
+    wq[c] = *(const uint4 *)(wr + (k < H ? k : 0));
+  }
+#pragma unroll
+  for (int i = 0; i < TG; ++i) {
+    const int t = t0 + i < T ? t0 + i : T - 1;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      const int k = c * 512 + 8 * lane;
+      xq[i][c] = *(const uint4 *)(x + (size_t)t * H + (k < H ? k : 0));
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TG; ++i) {
+    float acc = 0.f;
+#pragma unroll
+    for (int c = 0; c < NCH; ++c) {
+      float t = acc;
+      t = fmaf(bf16lo(xq[i][c].x), bf16lo(wq[c].x), t);
+      t = fmaf(bf16hi(xq[i][c].x), bf16hi(wq[c].x), t);
+      t = fmaf(bf16lo(xq[i][c].y), bf16lo(wq[c].y), t);
+      t = fmaf(bf16hi(xq[i][c].y), bf16hi(wq[c].y), t);
+      t = fmaf(bf16lo(xq[i][c].z), bf16lo(wq[c].z), t);
+      t = fmaf(bf16hi(xq[i][c].z), bf16hi(wq[c].z), t);
+      t = fmaf(bf16lo(xq[i][c].w), bf16lo(wq[c].w), t);
+      t = fmaf(bf16hi(xq[i][c].w), bf16hi(wq[c].w), t);
+      acc = (c * 512 + 8 * lane < H) ? t : acc;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);
+    out[i] = acc;
+  }
+}
+
+template <int TG>
+static __device__ __forceinline__ void gate_rows_batch_tg(const GemvArgs &a, const int lane, const int w, const int q) {
+  const int Erows = a.g_rows, H = a.cls[1].K, T = a.T;
+  const bool per_part = a.g_parts == GATE_PARTS;
+  const int item = per_part ? q >> 3 : q;
   const int nrb = (Erows + 3) >> 2;
-  const int t = item / nrb, e = (item - t * nrb) * 4 + w;
+  const int tgi = item / nrb, e = (item - tgi * nrb) * 4 + w;
+  const int t0 = tgi * TG;
   if (e >= Erows) return;
   const bool biased = a.g_bias && e < a.g_nbias;
   const float bias_e = biased ? a.g_bias[e] : 0.f;
   asm volatile("" :: "v"(bias_e));  // requested in front of the row
-  const float acc = gate_row_sum(a.cls[1].act + (size_t)t * H, a.g_w + (size_t)e * H, H, lane);
-  const float val = biased ? acc + bias_e : acc;
-  const u32x2_t word = {__float_as_uint(val), (u32)a.g_seq};
-  const int wi = t * Erows + e;
-  if (lane == 0)
-    __builtin_amdgcn_raw_buffer_store_b64(word, make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words,
-                                                          (u32)a.g_copy_words * 8u), wi * 8, 0, 1 /* sc0 */);
-  if ((q & 7) == 0) {
-    const unsigned long long word64 = ((unsigned long long)word.y << 32) | word.x;
-    if (lane == 1)
-      __hip_atomic_store(a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words + wi, word64, __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
-    if (lane == 0) a.g_logits_out[(size_t)t * a.g_ldl + e] = val;
+  float acc[TG];
+  const uint16_t *wr = a.g_w + (size_t)e * H;
+  const int nch = (H + 511) >> 9;  // wave-uniform
+  switch (nch) {
+    case 1: gate_rows_multi<1, TG>(a.cls[1].act, wr, H, lane, t0, T, acc); break;
+    case 2: gate_rows_multi<2, TG>(a.cls[1].act, wr, H, lane, t0, T, acc); break;
+    case 4: gate_rows_multi<4, TG>(a.cls[1].act, wr, H, lane, t0, T, acc); break;
+    case 8:  // (TG = 2 runs in the whole-row kernel, whose waves keep under 128 registers; 8 x 8 vectors do not fit)
+      if constexpr (TG != 2 && TG != 8) { gate_rows_multi<8, TG>(a.cls[1].act, wr, H, lane, t0, T, acc); break; }
+    default:
+#pragma unroll
+      for (int i = 0; i < TG; ++i)
+        acc[i] = gate_row_sum(a.cls[1].act + (size_t)(t0 + i < T ? t0 + i : T - 1) * H, wr, H, lane);
+  }
+  const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
+#pragma unroll
+  for (int i = 0; i < TG; ++i) {
+    const int t = t0 + i;
+    if (t < T) {
+      const float val = biased ? acc[i] + bias_e : acc[i];
+      const u32x2_t word = {__float_as_uint(val), (u32)a.g_seq};
+      const int wi = t * Erows + e;
+      if (per_part && lane == 0) __builtin_amdgcn_raw_buffer_store_b64(word, rl, wi * 8, 0, 1 /* sc0 */);
+      if (!per_part || (q & 7) == 0) {
+        const unsigned long long word64 = ((unsigned long long)word.y << 32) | word.x;
+        if (lane == 1)
+          __hip_atomic_store(a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words + wi, word64, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) a.g_logits_out[(size_t)t * a.g_ldl + e] = val;
+      }
+    }
   }
 }
 
@@ -1265,12 +1336,13 @@ static __device__ __forceinline__ void route_publish_batch(const GemvArgs &a, un
     const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
     const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
     const int nw = T * Erows;
+    const unsigned local_spins = a.g_parts == GATE_PARTS ? GATE_LOCAL_SPINS : 0u;
     bool timeout = false;
     for (int wi = tid; wi < nw; wi += 256) {
       unsigned spins = 0;
       u32x2_t word;
       for (;;) {
-        if (spins < GATE_LOCAL_SPINS) {
+        if (spins < local_spins) {
           word = __builtin_amdgcn_raw_buffer_load_b64(rl, wi * 8, 0, 16 /* sc1: past the first-level cache */);
         } else {
           const unsigned long long w64 = __hip_atomic_load(cg + wi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1300,7 +1372,8 @@ static __device__ __forceinline__ void route_publish_batch(const GemvArgs &a, un
 }
 
 // rr: the workgroup's index among those of the unit slots.  tokmask: the unit's tokens.
-template <int NR>
+// TPW: tokens per wave (wave w takes the tokens w, w + 4, ...; their selection rounds are interleaved)
+template <int NR, int TPW>
 static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const GemvArgs &a, const int lane, const int w,
                                                                       const int rr, unsigned &tokmask) {
   __shared__ unsigned long long s_sel[RB_MAXT][4];
@@ -1311,6 +1384,31 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const Gemv
   wk.b = rr - u * wk.c.nblk;
   wk.half = 0;
   const float NEG = -__builtin_inff();
+  // Unit records of this part of the chip: four (value, launch number) words per unit slot (slot address low and
+  // high, rows << 16 | first row position, token mask), written through this part's second-level cache by every
+  // workgroup that has derived the routing.  A workgroup that starts late (grid index from g_cache_from on: the
+  // first round of workgroups is over by then) reads its slot's record instead of polling logits and selecting;
+  // if the record is not there it derives the routing like the others.  All writers write the same values.
+  const rsrc_t rrec = make_rsrc(a.g_stamp + (size_t)GATE_COPIES * a.g_copy_words + (size_t)xcc_id() * (RB_MAX_UNITS * 4),
+                                RB_MAX_UNITS * 32u);
+  if ((int)blockIdx.x >= a.g_cache_from) {
+    __shared__ unsigned s_rec[5];
+    if (w == 0) {
+      const u32x2_t word = __builtin_amdgcn_raw_buffer_load_b64(rrec, (u * 4 + (lane & 3)) * 8, 0, 16 /* sc1 */);
+      const bool ok = (int)word.y == a.g_seq;
+      const bool all = (__ballot(ok) & 0xfull) == 0xfull;
+      if (lane < 4) s_rec[lane] = word.x;
+      if (lane == 0) s_rec[4] = all ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_rec[4]) {
+      wk.m = (int)(s_rec[2] >> 16);
+      wk.row0 = (int)(s_rec[2] & 0xffffu);
+      tokmask = s_rec[3];
+      wk.base = (const unsigned char *)(((unsigned long long)s_rec[1] << 32) | s_rec[0]);
+      return wk;
+    }
+  }
   unsigned long long ptrs[NR];  // slot addresses of the lane's experts, requested in front of the logits
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
@@ -1319,72 +1417,94 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const Gemv
   }
   const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
   const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
-  for (int t = w; t < T; t += 4) {
-    float v[NR];
-    bool gate_timeout = false;
+  float v[TPW][NR];
+  bool gate_timeout = false;
+  {
+    const unsigned local_spins = a.g_parts == GATE_PARTS ? GATE_LOCAL_SPINS : 0u;
     unsigned spins = 0;
     for (;;) {
       bool ok = true;
 #pragma unroll
-      for (int r = 0; r < NR; ++r) {
-        const int e = lane + 64 * r;
-        v[r] = NEG;
-        if (e < E) {
-          u32x2_t word;
-          if (spins < GATE_LOCAL_SPINS) {
-            word = __builtin_amdgcn_raw_buffer_load_b64(rl, (t * Erows + e) * 8, 0, 16 /* sc1: past the first-level cache */);
-          } else {
-            const unsigned long long w64 = __hip_atomic_load(cg + t * Erows + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+      for (int i = 0; i < TPW; ++i) {
+        const int t = w + 4 * i;
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+          const int e = lane + 64 * r;
+          v[i][r] = NEG;
+          if (e < E && t < T) {
+            u32x2_t word;
+            if (spins < local_spins) {
+              word = __builtin_amdgcn_raw_buffer_load_b64(rl, (t * Erows + e) * 8, 0, 16 /* sc1: past the first-level cache */);
+            } else {
+              const unsigned long long w64 = __hip_atomic_load(cg + t * Erows + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              word.x = (u32)w64; word.y = (u32)(w64 >> 32);
+            }
+            v[i][r] = __uint_as_float(word.x);
+            ok = ok && (int)word.y == a.g_seq;
           }
-          v[r] = __uint_as_float(word.x);
-          ok = ok && (int)word.y == a.g_seq;
         }
       }
       if (__ballot(!ok) == 0ull) break;
       if (++spins >= GATE_POLL_LIMIT) { gate_timeout = true; break; }  // (the launch then reports an error)
       __builtin_amdgcn_s_sleep(2);
     }
-    unsigned long long msel[NR];
+  }
+  unsigned long long msel[TPW][NR];
 #pragma unroll
-    for (int r = 0; r < NR; ++r) msel[r] = 0ull;
-    for (int j = 0; j < k; ++j) {
-      float bv = v[0];
+  for (int i = 0; i < TPW; ++i)
 #pragma unroll
-      for (int r = 1; r < NR; ++r) bv = fmaxf(bv, v[r]);
+    for (int r = 0; r < NR; ++r) msel[i][r] = 0ull;
+  for (int j = 0; j < k; ++j) {
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+      float bv = v[i][0];
+#pragma unroll
+      for (int r = 1; r < NR; ++r) bv = fmaxf(bv, v[i][r]);
       const float best = wave_max_f32(bv);
       int wr = -1, wl = 0;
 #pragma unroll
       for (int r = 0; r < NR; ++r) {
-        const unsigned long long mr = __ballot(v[r] == best);
+        const unsigned long long mr = __ballot(v[i][r] == best);
         if (wr < 0 && mr) { wr = r; wl = (int)__builtin_ctzll(mr); }
       }
       if (wr < 0) { wr = 0; wl = j; }  // NaN logits match nothing: stay inside the expert range
 #pragma unroll
       for (int r = 0; r < NR; ++r)
         if (r == wr) {
-          if (lane == wl) v[r] = NEG;
-          msel[r] |= 1ull << wl;
+          if (lane == wl) v[i][r] = NEG;
+          msel[i][r] |= 1ull << wl;
         }
     }
-    if (lane == 0) {
+  }
+  __shared__ int s_timeout[4];
+  if (lane == 0) {
 #pragma unroll
-      for (int r = 0; r < NR; ++r) s_sel[t][r] = gate_timeout ? 0ull : msel[r];
-      if (gate_timeout) moe_raise_err(a.err);
+    for (int i = 0; i < TPW; ++i) {
+      const int t = w + 4 * i;
+      if (t < T) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) s_sel[t][r] = gate_timeout ? 0ull : msel[i][r];
+      }
     }
+    s_timeout[w] = gate_timeout ? 1 : 0;
+    if (gate_timeout) moe_raise_err(a.err);
   }
   __syncthreads();
+  const bool gate_timeout_any = (s_timeout[0] | s_timeout[1] | s_timeout[2] | s_timeout[3]) != 0;  // (no records then)
   // per expert (this lane's, per column): its tokens
   int cnt[NR];
   unsigned mk[NR];
 #pragma unroll
   for (int r = 0; r < NR; ++r) { cnt[r] = 0; mk[r] = 0u; }
-  for (int t = 0; t < T; ++t) {
 #pragma unroll
-    for (int r = 0; r < NR; ++r) {
-      const unsigned bit = (unsigned)((s_sel[t][r] >> lane) & 1ull);
-      cnt[r] += (int)bit;
-      mk[r] |= bit << t;
+  for (int t = 0; t < 4 * TPW; ++t) {
+    if (t < T) {
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+        const unsigned bit = (unsigned)((s_sel[t][r] >> lane) & 1ull);
+        cnt[r] += (int)bit;
+        mk[r] |= bit << t;
+      }
     }
   }
   int cum_act = 0, cum_rows = 0, m = 0, row0 = 0;
@@ -1394,22 +1514,42 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const Gemv
   for (int r = 0; r < NR; ++r) {
     const unsigned long long actm = __ballot(cnt[r] > 0);
     const unsigned long long b0 = __ballot((cnt[r] & 1) != 0), b1 = __ballot((cnt[r] & 2) != 0),
-                             b2 = __ballot((cnt[r] & 4) != 0), b3 = __ballot((cnt[r] & 8) != 0);
+                             b2 = __ballot((cnt[r] & 4) != 0), b3 = __ballot((cnt[r] & 8) != 0),
+                             b4 = __ballot((cnt[r] & 16) != 0);
     const int na = __popcll(actm);
     if (!found && u < cum_act + na) {
       unsigned long long mm = actm;
       for (int i = 0; i < u - cum_act; ++i) mm &= mm - 1;
       const int src = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(mm));  // expert 64 r + src
       const unsigned long long sb = (1ull << src) - 1ull;
-      row0 = cum_rows + __popcll(b0 & sb) + 2 * __popcll(b1 & sb) + 4 * __popcll(b2 & sb) + 8 * __popcll(b3 & sb);
+      row0 = cum_rows + __popcll(b0 & sb) + 2 * __popcll(b1 & sb) + 4 * __popcll(b2 & sb) + 8 * __popcll(b3 & sb) +
+             16 * __popcll(b4 & sb);
       m = __builtin_amdgcn_readlane(cnt[r], src);
       tm = (unsigned)__builtin_amdgcn_readlane((int)mk[r], src);
       lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)ptrs[r], src);
       hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(ptrs[r] >> 32), src);
       found = true;
     }
+    if (w == 0 && !gate_timeout_any && cnt[r] > 0) {  // this lane's expert is a unit: leave its record
+      const unsigned long long lb = (1ull << lane) - 1ull;
+      const int ui = cum_act + __popcll(actm & lb);
+      const int rw = cum_rows + __popcll(b0 & lb) + 2 * __popcll(b1 & lb) + 4 * __popcll(b2 & lb) + 8 * __popcll(b3 & lb) +
+                     16 * __popcll(b4 & lb);
+      if (ui < RB_MAX_UNITS) {
+        const u32 seq = (u32)a.g_seq;
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{(u32)ptrs[r], seq}, rrec, (ui * 4 + 0) * 8, 0, 1 /* sc0 */);
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{(u32)(ptrs[r] >> 32), seq}, rrec, (ui * 4 + 1) * 8, 0, 1);
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{((u32)cnt[r] << 16) | (u32)rw, seq}, rrec, (ui * 4 + 2) * 8, 0, 1);
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{mk[r], seq}, rrec, (ui * 4 + 3) * 8, 0, 1);
+      }
+    }
     cum_act += na;
-    cum_rows += __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2) + 8 * __popcll(b3);
+    cum_rows += __popcll(b0) + 2 * __popcll(b1) + 4 * __popcll(b2) + 8 * __popcll(b3) + 16 * __popcll(b4);
+  }
+  if (w == 0 && !gate_timeout_any) {  // the slots past the last unit: records of no rows
+    const int nslots = a.p_max_units < RB_MAX_UNITS ? a.p_max_units : RB_MAX_UNITS;
+    for (int ui = cum_act + (lane >> 2); ui < nslots; ui += 16)
+      __builtin_amdgcn_raw_buffer_store_b64(u32x2_t{0u, (u32)a.g_seq}, rrec, (ui * 4 + (lane & 3)) * 8, 0, 1 /* sc0 */);
   }
   wk.m = found ? m : 0;
   wk.row0 = row0;
@@ -1418,10 +1558,11 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const Gemv
   return wk;
 }
 
+// TPW: the launch's tokens per wave (1: up to 4 tokens, 2: up to 8, 4: up to 16); E up to 64 pays for one column
+template <int TPW>
 static __device__ __forceinline__ GemvWork gemv_resolve_route_batch(const GemvArgs &a, int lane, int w, int rr, unsigned &tokmask) {
-  if (a.r_E <= 64) return gemv_resolve_route_batch_n<1>(a, lane, w, rr, tokmask);
-  if (a.r_E <= 128) return gemv_resolve_route_batch_n<2>(a, lane, w, rr, tokmask);
-  return gemv_resolve_route_batch_n<4>(a, lane, w, rr, tokmask);
+  if (a.r_E <= 64) return gemv_resolve_route_batch_n<1, TPW>(a, lane, w, rr, tokmask);
+  return gemv_resolve_route_batch_n<4, TPW>(a, lane, w, rr, tokmask);
 }
 
 // the i-th token (i-th set bit) of a unit's token mask
@@ -1980,7 +2121,7 @@ static __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4 &x) {
 // ROUTE (w13 pass, device-side slot table): the launch sums the gate rows and routes by itself, see
 // gemv_resolve_route_batch_n; a unit's token rows then come from its token mask, not from a list in memory
 template <bool SWIGLU, int CH, bool DEVUNITS, bool ROUTE = false>
-__global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW_R, const int RPW_S) {
+__global__ __launch_bounds__(256, (ROUTE ? 4 : 2)) void k_gemv_int4_mfma(const GemvArgs a, const int TB, const int RPW_R, const int RPW_S) {
   constexpr int NP = 1, NB = 2 * NP;  // block pairs / 16-row blocks per iteration
   constexpr int PF = 4;               // activation pieces in flight while staging
   extern __shared__ __align__(16) unsigned char smem[];
@@ -1999,14 +2140,27 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
   bool masked = false;
   GemvWork wk;
   if constexpr (ROUTE) {
-    if (bx < a.g_nblk) { gate_rows_batch(a, lane, w, bx); return; }
+    if (bx < a.g_nblk) {
+#ifdef RB_NO_TG2
+      gate_rows_batch_tg<1>(a, lane, w, bx);
+#else
+      if (a.T <= 4) gate_rows_batch_tg<1>(a, lane, w, bx);
+      else gate_rows_batch_tg<2>(a, lane, w, bx);
+#endif
+      return;
+    }
     bx -= a.g_nblk;
     if (bx == 0) { route_publish_batch(a, smem); return; }
     bx -= 1;
     if (bx < a.n_sh_blocks) {
       wk.c = a.cls[0]; wk.b = bx; wk.half = 0; wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
     } else {
-      wk = gemv_resolve_route_batch(a, lane, w, bx - a.n_sh_blocks, tokmask);
+#ifdef RB_NO_TPW2
+      wk = gemv_resolve_route_batch<1>(a, lane, w, bx - a.n_sh_blocks, tokmask);
+#else
+      if (a.T <= 4) wk = gemv_resolve_route_batch<1>(a, lane, w, bx - a.n_sh_blocks, tokmask);
+      else wk = gemv_resolve_route_batch<2>(a, lane, w, bx - a.n_sh_blocks, tokmask);
+#endif
       masked = true;
     }
   } else {
@@ -2231,10 +2385,12 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma(const GemvArgs a, con
 
 // One pass of the chunked-K form: rows row_first .. row_first + mc - 1 (mc <= 16 NT) of one unit against the block
 // pair b of its matrix.  Every thread of the workgroup takes part (barriers inside).
-template <bool SWIGLU, int NT, int CG, int KS>
+// MASKED with tokmask != 0: the pass's rows are the tokens of that bit mask (a unit of a launch that routes by
+// itself, all of its rows in this one pass) instead of c.gather's
+template <bool SWIGLU, int NT, int CG, int KS, bool MASKED = false>
 static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char *smem, const rsrc_t rq, const rsrc_t rs,
                                                const rsrc_t rz, const rsrc_t rx, const int b, const int row_first,
-                                               const int mc, const Q4Consts &q4c) {
+                                               const int mc, const Q4Consts &q4c, const unsigned tokmask = 0u) {
   constexpr int NB = 2;                // 16-row blocks per wave
   constexpr int GW = CG / KS;          // groups per wave and chunk
   constexpr int WS = GW < 4 ? GW : 4;  // groups per weight step
@@ -2272,7 +2428,8 @@ static __device__ __forceinline__ void kc_pass(const GemvClass &c, unsigned char
   for (int i = 0; i < NPC; ++i) {
     const int row = (tid + 256 * i) / XV;
     const int gr = row_first + (row < mc ? row : mc - 1);
-    xoff[i] = row < mc ? (c.gather ? c.gather[gr] : gr) * c.act_stride * 2 : -1;
+    if (MASKED && tokmask != 0u) xoff[i] = row < mc ? nth_token(tokmask, row) * c.act_stride * 2 : -1;
+    else xoff[i] = row < mc ? (c.gather ? c.gather[gr] : gr) * c.act_stride * 2 : -1;
   }
   uint4 xr[NPC];
   u32 scr[NSD], zr[NSD];
@@ -2703,22 +2860,43 @@ static __device__ __forceinline__ void kc_pass_q4k(const GemvClass &c, unsigned 
 // where 16-row passes cost up to four.
 // q4_K: the shared expert's w2 class may be split (c.ksplit workgroups per group of block pairs, each over 1 / ksplit
 // of the reduction, partial rows to their own copy of the output: see k_gemv_int4).
-template <bool SWIGLU, bool DEVUNITS, int NTMAX, int KS, bool Q4K = false>
+// ROUTE (int4 w13 pass of at most 16 tokens): the launch sums the gate rows and routes by itself, as
+// k_gemv_int4_mfma<.., ROUTE> does (see gemv_resolve_route_batch_n)
+template <bool SWIGLU, bool DEVUNITS, int NTMAX, int KS, bool Q4K = false, bool ROUTE = false>
 __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) {
   constexpr int NB = 2;
+  static_assert(!ROUTE || (SWIGLU && DEVUNITS && NTMAX == 1 && !Q4K), "routing launches: int4 w13, 16-row passes");
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   KC_STAMP(0);
 
   // a publishing workgroup comes first in the grid: it is over long before the ones that stream weights
-  const bool publishes = SWIGLU && DEVUNITS && a.p_host_units != nullptr;
+  const bool publishes = !ROUTE && SWIGLU && DEVUNITS && a.p_host_units != nullptr;
   if (publishes && blockIdx.x == 0) {
     gemv_publish_units(a);
     return;
   }
-  const int bx = (int)blockIdx.x - (publishes ? 1 : 0);
-  const GemvWork wk = gemv_resolve<DEVUNITS, (NTMAX > 1)>(a, bx, lane);
+  int bx = (int)blockIdx.x - (publishes ? 1 : 0);
+  unsigned tokmask = 0u;   // ROUTE: the tokens of a routed unit
+  GemvWork wk;
+  if constexpr (ROUTE) {
+    if (bx < a.g_nblk) {
+      if (a.T <= 8) gate_rows_batch_tg<4>(a, lane, w, bx);
+      else gate_rows_batch_tg<8>(a, lane, w, bx);
+      return;
+    }
+    bx -= a.g_nblk;
+    if (bx == 0) { route_publish_batch(a, smem); return; }
+    bx -= 1;
+    if (bx < a.n_sh_blocks) {
+      wk.c = a.cls[0]; wk.b = bx; wk.half = 0; wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
+    } else {
+      wk = gemv_resolve_route_batch<4>(a, lane, w, bx - a.n_sh_blocks, tokmask);
+    }
+  } else {
+    wk = gemv_resolve<DEVUNITS, (NTMAX > 1)>(a, bx, lane);
+  }
   const GemvClass &c = wk.c;
   const int m = wk.m, row0 = wk.row0;
   const unsigned char *base = wk.base;
@@ -2765,7 +2943,7 @@ __global__ __launch_bounds__(256, 2) void k_gemv_int4_mfma_kc(const GemvArgs a) 
     } else {
       const int mc = left < 16 ? left : 16;
       if constexpr (Q4K) kc_pass_q4k<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, Gt, G, b, orow0, row0 + t0, mc, dqc);
-      else kc_pass<SWIGLU, 1, 8, KS>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c);
+      else kc_pass<SWIGLU, 1, 8, KS, ROUTE>(c, smem, rq, rs, rz, rx, b, row0 + t0, mc, q4c, tokmask);
       t0 += 16;
     }
     if (t0 < r_hi) __syncthreads();  // the next pass restages chunk buffer 0
@@ -3352,10 +3530,15 @@ static int launch_gemv_mfma_route(const GemvArgs &a_in, int units, int tb, size_
   if (a.n_sh_blocks > 0) { a.cls[0].nblk /= rpw_s; a.n_sh_blocks /= rpw_s; }
   a.cls[1].nblk /= rpw;
   const int grid = a.g_nblk + 1 + a.n_sh_blocks + units * a.cls[1].nblk;
+  {  // workgroups the chip holds at once (four per compute unit by registers), and the gate workgroups' places again
+    int per_cu = (int)((160 * 1024) / (lds + 4096));
+    per_cu = per_cu > 4 ? 4 : (per_cu < 1 ? 1 : per_cu);
+    a.g_cache_from = 256 * per_cu + a.g_nblk;
+  }
   static bool attr_set = false;
   if (lds > 64 * 1024 && !attr_set) {
     if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gemv_int4_mfma<true, CH, true, true>,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024),
                                "hipFuncSetAttribute(k_gemv_int4_mfma, routing)"))
       return rc;
     attr_set = true;
@@ -3366,14 +3549,50 @@ static int launch_gemv_mfma_route(const GemvArgs &a_in, int units, int tb, size_
   return moe_check_launch("k_gemv_int4_mfma<route>");
 }
 
+template <int KS>
+static int launch_gemv_mfma_kc_route(const GemvArgs &a_in, int units, hipStream_t s) {
+  constexpr int PW = 4 / KS;
+  GemvArgs a = a_in;
+  if ((a.n_sh_blocks > 0 && a.cls[0].nblk % 4) || a.cls[1].nblk % 4) {
+    moe_set_error("k_gemv_int4_mfma_kc: block pairs per unit not a multiple of 4");
+    return MOE_EINVAL;
+  }
+  if (a.n_sh_blocks > 0) { a.cls[0].nblk /= PW; a.n_sh_blocks /= PW; }
+  a.cls[1].nblk /= PW;
+  a.unit_slots = 0;
+  const int grid = a.g_nblk + 1 + a.n_sh_blocks + units * a.cls[1].nblk;
+  a.g_cache_from = 256 * 2 + a.g_nblk;  // two workgroups per compute unit at a time
+  const size_t lds = gemv_mfma_kc_lds(1, 8);
+  static_assert(RB_PUBLISH_LDS <= 64 * 1024, "the publishing workgroup's LDS");
+  static bool attr_set = false;
+  if (!attr_set) {
+    // (the kernel also has a few hundred bytes of static LDS: dynamic + static must stay within 160 KB)
+    if (int rc = moe_check_hip(hipFuncSetAttribute((const void *)k_gemv_int4_mfma_kc<true, true, 1, KS, false, true>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024),
+                               "hipFuncSetAttribute(k_gemv_int4_mfma_kc, routing)"))
+      return rc;
+    attr_set = true;
+  }
+  moe_ktimer_begin(MOE_K_W13, s);
+  hipLaunchKernelGGL((k_gemv_int4_mfma_kc<true, true, 1, KS, false, true>), dim3(grid), dim3(256), lds, s, a);
+  moe_ktimer_end(MOE_K_W13, s);
+  return moe_check_launch("k_gemv_int4_mfma_kc<route>");
+}
+
+// whole-row form (up to 8 tokens whose rows leave room for two workgroups per compute unit) or chunked-K form
+static bool batch_route_whole_rows(int T, int H) {
+  if (T > 8) return false;
+  int tb = 1;
+  while (tb < T) tb <<= 1;
+  return gemv_mfma_lds(tb, H, 2) <= 80 * 1024;
+}
+
 // whether moe_decode_batch_int4_gate takes a batch of T tokens of this shape
 extern "C" int moe_decode_batch_int4_gate_fits(int T, int E, int k, int H, int I, int I_sh, int n_gate_rows) {
   if (T < 2 || T > RB_MAXT || E <= 0 || E > 256 || k <= 0 || k > 32 || k > E || T * k > ROUTE_MAXP || H <= 0 || H % 128 ||
       I <= 0 || I % 128 || I_sh < 0 || I_sh % 128 || n_gate_rows < E || n_gate_rows > E + 1)
     return 0;
-  int tb = 1;
-  while (tb < T) tb <<= 1;
-  return gemv_mfma_lds(tb, H, 2) <= 80 * 1024;  // two workgroups per compute unit (else the chunked form is the faster one)
+  return 1;
 }
 
 extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate_w, const float *gate_bias,
@@ -3417,23 +3636,32 @@ extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate
     a.g_w = (const uint16_t *)gate_w; a.g_bias = gate_bias; a.g_stamp = (unsigned long long *)gate_ws;
     a.g_logits_out = logits; a.g_ldl = ldl; a.g_rows = n_gate_rows; a.g_nbias = gate_bias ? E : 0; a.g_seq = gate_seq;
     a.g_copy_words = T * n_gate_rows > GATE_COPY_WORDS ? T * n_gate_rows : GATE_COPY_WORDS;
-    a.g_nblk = GATE_PARTS * T * ((n_gate_rows + 3) / 4);
     a.cls[0] = GemvClass{(const uint16_t *)x, nullptr, h_s, ls.off13_q, ls.off13_s, ls.off13_z, H, H / 128, H, I_sh, I_sh / 16, 0};
     a.cls[1] = GemvClass{(const uint16_t *)x, nullptr, h_r, lr.off13_q, lr.off13_s, lr.off13_z, H, H / 128, H, I, I / 16, 0};
     a.n_sh_blocks = sh ? I_sh / 16 : 0;
-    int tb = 1;
-    while (tb < T) tb <<= 1;
-    size_t lds = gemv_mfma_lds(tb, H, 2);
-    if (lds < RB_PUBLISH_LDS) lds = RB_PUBLISH_LDS;
-    const int gpw = (H / 128 + 3) / 4;
-    int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
-    if (ch < 1) ch = 1;
+    const bool whole = batch_route_whole_rows(T, H);
+    const int tg = !whole ? (T <= 8 ? 4 : 8) : (T <= 4 ? 1 : 2);   // tokens per gate workgroup: what the kernel instantiates
+    static const int parts_env = [] { const char *e = getenv("MOE_BATCH_PARTS"); return e ? atoi(e) : 0; }();
+    a.g_parts = parts_env == 1 ? 1 : (parts_env == 8 ? GATE_PARTS : GATE_PARTS);
+    a.g_nblk = a.g_parts * ((T + tg - 1) / tg) * ((n_gate_rows + 3) / 4);
     int rc;
-    switch (ch) {
-      case 1: rc = launch_gemv_mfma_route<1>(a, max_units, tb, lds, s); break;
-      case 2: rc = launch_gemv_mfma_route<2>(a, max_units, tb, lds, s); break;
-      case 3: rc = launch_gemv_mfma_route<3>(a, max_units, tb, lds, s); break;
-      default: rc = launch_gemv_mfma_route<4>(a, max_units, tb, lds, s); break;
+    if (!whole) {
+      rc = (a.n_sh_blocks + max_units * (I / 16)) / 4 >= 384 ? launch_gemv_mfma_kc_route<1>(a, max_units, s)
+                                                             : launch_gemv_mfma_kc_route<2>(a, max_units, s);
+    } else {
+      int tb = 1;
+      while (tb < T) tb <<= 1;
+      size_t lds = gemv_mfma_lds(tb, H, 2);
+      if (lds < RB_PUBLISH_LDS) lds = RB_PUBLISH_LDS;
+      const int gpw = (H / 128 + 3) / 4;
+      int ch = gpw >= 4 ? ((gpw % 4 == 0) ? 4 : (gpw % 3 == 0 ? 3 : 4)) : gpw;
+      if (ch < 1) ch = 1;
+      switch (ch) {
+        case 1: rc = launch_gemv_mfma_route<1>(a, max_units, tb, lds, s); break;
+        case 2: rc = launch_gemv_mfma_route<2>(a, max_units, tb, lds, s); break;
+        case 3: rc = launch_gemv_mfma_route<3>(a, max_units, tb, lds, s); break;
+        default: rc = launch_gemv_mfma_route<4>(a, max_units, tb, lds, s); break;
+      }
     }
     if (rc) return rc;
   }
@@ -3795,7 +4023,8 @@ extern "C" int moe_topk_dispatch(const float *logits, int T, int E, int ldl, int
 extern "C" int64_t moe_gate_route_ws_bytes(int T, int Erows) {
   if (T < 1 || Erows < 1) return 0;
   const int64_t words = (int64_t)T * Erows > GATE_COPY_WORDS ? (int64_t)T * Erows : GATE_COPY_WORDS;
-  return (int64_t)GATE_COPIES * words * 8;
+  // the logit words of every copy, then the unit records of every part (moe_decode_batch_int4_gate)
+  return (int64_t)GATE_COPIES * words * 8 + (int64_t)GATE_PARTS * RB_MAX_UNITS * 32;
 }
 
 extern "C" int moe_gate_topk_dispatch(const void *x, const void *wg, const float *bias, int n_bias, float *logits, int T,
