@@ -290,6 +290,33 @@ __global__ __launch_bounds__(256, 1) void k_prefill_gemm(const PfArgs a) {
 #undef PF_LOOPS
   // epilogue.  acc element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l%32
   const int col = 32 * w + (lane & 31);
+  if constexpr (SWIGLU) {
+    // The h tile (rows x 128 bf16) goes through LDS, so that it leaves in 16-byte stores that cover whole 256-byte
+    // rows: straight from the accumulators a lane stores 2 bytes at a time (128 store instructions per lane, each
+    // covering two 64-byte pieces of two rows).  The activation ring is free once every wave has left the main loop
+    // and the transfers still on their way into it (the slabs requested past the end) have landed.
+    constexpr int HS = 2 * PF_BNH + 16;  // padded row stride in bytes
+    static_assert((size_t)PF_BM * HS <= (size_t)PF4_RING * PF4_SLAB * 2, "the h tile fits the activation ring");
+    unsigned char *hs = (unsigned char *)As;
+    PF_VMCNT(0);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < nb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+          *(__bf16 *)(hs + row * HS + col * 2) = (__bf16)pf_silu_mul(acc[i][0][e], acc[i][1][e]);
+        }
+      }
+    __syncthreads();
+    const int chunk = tid & 15;
+    for (int row = tid >> 4; row < tile.rows; row += 16) {
+      const uint4 v = *(const uint4 *)(hs + row * HS + chunk * 16);
+      *(uint4 *)((__bf16 *)c.out + (size_t)(tile.row0 + row) * c.out_stride + n0 + 8 * chunk) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
