@@ -273,10 +273,20 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
     token_path = T == 1 and not q4k
     unit_ws = torch.zeros(32 * k, dtype=torch.uint8, device=dev)
     ws_tok = None
+    # 2 to 16 tokens, int4: likewise (gate rows and routing inside the w13 launch, then w2, then the combine)
+    batch_path = (not q4k) and T >= 2 and ops.decode_batch_int4_gate_fits(T, E, k, H, I, I_sh, rows)
+    gate_ws = ops.GateWorkspace(dev, max(T, 1), rows) if batch_path else None
+    ws_b = None
 
     def step(i, phases=3, route=True):
-        nonlocal ws, ws_tok
+        nonlocal ws, ws_tok, ws_b
         l, x = i % layers, xs[i % len(xs)]
+        if batch_path:
+            ws_b = ops.decode_batch_int4_gate(x, gws[l], biases[l], E, k, mode, tables[l], shs[l], H, I, I_sh, gate_ws,
+                                              phases=phases, ws=ws_b)
+            if phases == 3:
+                ops.combine(ws_b[4], ws_b[5], ws_b[2], ws_b[3].pos_of_pair, ws_b[0][:, E] if gated else None, T, H, k, out=y)
+            return
         if token_path and phases == 3:
             ops.gate_logits(x, gws[l], biases[l], out=logits)
             ws_tok = ops.decode_token_int4(x, logits, E, k, mode, tables[l], shs[l], H, I, I_sh, ws=ws_tok, phases=5,
@@ -305,7 +315,7 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
 
     for i in range(4 * layers):
         step(i)
-        nact.append(int((ws_tok[2] if token_path else d).n_active.cpu()[0]))
+        nact.append(int((ws_tok[2] if token_path else (ws_b[3] if batch_path else d)).n_active.cpu()[0]))
     if token_path:   # the one-token path against the separate kernels on the same input
         y_tok = y.float().clone()
         token_path = False
@@ -313,13 +323,14 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
         token_path = True
         assert int(ws_tok[5].cpu()[0]) == 0
         assert float((y_tok - y.float()).abs().max()) <= 1e-2 * float(y.float().abs().max())
-    assert int(ws[2].cpu()[0]) == 0
+    assert int((ws_b[6] if batch_path else ws[2]).cpu()[0]) == 0
     t_layer = timed(step, steps)
     # the w13 + SwiGLU GEMV alone, back to back, with the routing of the last full step kept
     for i in range(2 * layers):
         step(i, phases=1, route=False)
     torch.cuda.synchronize()
-    w13_us_leg, w13_method = launches_timed(torch, lambda n: [step(i, phases=1, route=False) for i in range(n)] and None, steps)
+    w13_us_leg, w13_method = launches_timed(torch, lambda n: [step(i, phases=1, route=False) for i in range(n)] and None, steps,
+                                            replay_once=batch_path)
     t_w13 = w13_us_leg * 1e-6
     D = float(np.mean(nact))
     D_last = nact[-1]
@@ -327,11 +338,15 @@ def decode_leg(torch, name, fmt, T, H, E, I, k, I_sh, gated, mode, layers, zipf,
     ls = lay(H, I_sh) if I_sh else {"total_bytes": 0, "off2_q": 0}
     step_bytes = D * lr["total_bytes"] + ls["total_bytes"] + rows * H * 2 + 2 * T * H * 2
     w13_bytes = D_last * lr["off2_q"] + ls["off2_q"] + 2 * T * H
+    if batch_path:   # the launch also reads the gate matrix and its bias
+        w13_bytes += rows * H * 2 + E * 4
     ach = w13_bytes / t_w13 / 1e9
     return {"workload": name, "tokens": T, "layers_in_rotation": layers, "tokens_per_s": T / t_layer,
             "us_per_layer": t_layer * 1e6, "distinct_routed_experts_per_step": D,
             "algorithmic_bytes_per_step": step_bytes, "layer_GBps": step_bytes / t_layer / 1e9,
-            "roofline": {"bound": "hbm", "kernel": ("k_prefill_int4 (w13 + SwiGLU)" if tiles else
+            "roofline": {"bound": "hbm", "kernel": ("k_gemv_int4_mfma%s<route> (gate rows + routing + w13 + SwiGLU in one launch)"
+                                                    % ("" if T <= 8 and H <= 2048 else "_kc")) if batch_path else
+                                                   ("k_prefill_int4 (w13 + SwiGLU)" if tiles else
                                                     "k_gemv_int4%s (w13 + SwiGLU)" % (("_mfma_kc<q4_K>" if T > 1 else "<q4_K>") if q4k else ("_mfma_kc" if (T > 16 or H > 2048) and T > 1 else ("_mfma" if T > 1 else "")))),
                          "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
                          "algorithmic_bytes_per_launch": w13_bytes, "avg_launch_us": t_w13 * 1e6,
@@ -470,11 +485,19 @@ def main():
     gate_ws = ops.GateWorkspace(dev)
     ws_tok = None
 
+    # 2 to 16 tokens: likewise (the w13 launch of a batch sums the gate rows and routes by itself)
+    batch_fused = T >= 2 and ops.decode_batch_int4_gate_fits(T, E, k, H, I, I_sh, E)
+    gate_ws_b = ops.GateWorkspace(dev, T, E + 1) if batch_fused else None
+    ws_b = None
+
     def w13_only(n):
-        nonlocal ws_tok
+        nonlocal ws_tok, ws_b
         for i in range(n):
             l = i % L_
-            if T == 1:
+            if batch_fused:
+                ws_b = ops.decode_batch_int4_gate(xs[i % len(xs)], stack.gate_w[l], stack.gate_bias[l], E, k, 0, _Tab(tables[l]),
+                                                  stack.shared[l], H, I, I_sh, gate_ws_b, phases=1, ws=ws_b)
+            elif T == 1:
                 ws_tok = ops.decode_token_int4(xs[i % len(xs)], logits_out, E, k, 0, _Tab(tables[l]), stack.shared[l], H, I,
                                                I_sh, ws=ws_tok, phases=1, gate=(stack.gate_w[l], stack.gate_bias[l], gate_ws))
             else:
@@ -482,16 +505,20 @@ def main():
     w13_only(2 * L_)
     torch.cuda.synchronize()
     n_k = 20 * L_
-    w13_us, w13_method = launches_timed(torch, w13_only, n_k, replay_once=(T == 1))
-    assert int((ws_tok[5] if T == 1 else ws[2]).cpu()[0]) == 0
+    w13_us, w13_method = launches_timed(torch, w13_only, n_k, replay_once=(T == 1 or batch_fused))
+    assert int((ws_tok[5] if T == 1 else (ws_b[6] if batch_fused else ws[2])).cpu()[0]) == 0
     D_k = float(np.mean([int(r.n_active.cpu()[0]) for r in routed]))
-    gate_bytes = (E * H * 2 + E * 4) if T == 1 else 0          # gate rows + bias, read by the same launch at T = 1
+    if batch_fused:   # (the launches above route xs[i % 8] themselves: take the last one's count)
+        D_k = float(int(ws_b[3].n_active.cpu()[0]))
+    gate_bytes = (E * H * 2 + E * 4) if (T == 1 or batch_fused) else 0   # gate rows + bias, read by the same launch
     w13_bytes_k = D_k * lay_r["off2_q"] + lay_s["off2_q"] + 2 * T * H + gate_bytes
     achieved = w13_bytes_k / (w13_us * 1e-6) / 1e9
     # the same kernel inside the timed steps (between the w2 + combine launches of the neighbouring steps), from
     # the committed rocprofv3 kernel trace of this command; null when the kernel sources changed since
     in_path_us = recorded_decode("decode_w13_in_path_avg_us", "decode_deepseek_int4_T1_kernel_trace.md") if (T == 1 and L_ == 27) else None
-    roofline = {"bound": "hbm", "kernel": ("k_w13_token (gate rows + routing + w13 + SwiGLU in one launch)" if T == 1 else "k_gemv_int4_mfma (w13 + SwiGLU)"),
+    roofline = {"bound": "hbm", "kernel": ("k_w13_token (gate rows + routing + w13 + SwiGLU in one launch)" if T == 1 else
+                                           ("k_gemv_int4_mfma%s<route> (gate rows + routing + w13 + SwiGLU in one launch)" % ("" if T <= 8 else "_kc")
+                                            if batch_fused else "k_gemv_int4_mfma (w13 + SwiGLU)")),
                 "achieved": achieved,
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs of this kernel at this
@@ -508,7 +535,7 @@ def main():
     layer = {"algorithmic_bytes_per_step": layer_bytes, "us_per_step": step_us,
              "wall_GBps": layer_bytes / (dt / a.steps) / 1e9,
              "frac_of_hbm_peak": layer_bytes / (dt / a.steps) / 1e9 / HBM_PEAK_GBS,
-             "launches_per_step": 2 if T == 1 else 5,
+             "launches_per_step": 2 if T == 1 else (3 if batch_fused else 4),
              "w2_combine_avg_us_in_timed_steps": recorded_decode("decode_w2c_in_path_avg_us", "decode_deepseek_int4_T1_kernel_trace.md") if (T == 1 and L_ == 27) else None}
 
     sweep = {}

@@ -2141,12 +2141,8 @@ __global__ __launch_bounds__(256, (ROUTE ? 4 : 2)) void k_gemv_int4_mfma(const G
   GemvWork wk;
   if constexpr (ROUTE) {
     if (bx < a.g_nblk) {
-#ifdef RB_NO_TG2
-      gate_rows_batch_tg<1>(a, lane, w, bx);
-#else
       if (a.T <= 4) gate_rows_batch_tg<1>(a, lane, w, bx);
       else gate_rows_batch_tg<2>(a, lane, w, bx);
-#endif
       return;
     }
     bx -= a.g_nblk;
@@ -2155,12 +2151,8 @@ __global__ __launch_bounds__(256, (ROUTE ? 4 : 2)) void k_gemv_int4_mfma(const G
     if (bx < a.n_sh_blocks) {
       wk.c = a.cls[0]; wk.b = bx; wk.half = 0; wk.m = a.T; wk.row0 = 0; wk.base = a.shared_base;
     } else {
-#ifdef RB_NO_TPW2
-      wk = gemv_resolve_route_batch<1>(a, lane, w, bx - a.n_sh_blocks, tokmask);
-#else
       if (a.T <= 4) wk = gemv_resolve_route_batch<1>(a, lane, w, bx - a.n_sh_blocks, tokmask);
       else wk = gemv_resolve_route_batch<2>(a, lane, w, bx - a.n_sh_blocks, tokmask);
-#endif
       masked = true;
     }
   } else {
@@ -3641,8 +3633,7 @@ extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate
     a.n_sh_blocks = sh ? I_sh / 16 : 0;
     const bool whole = batch_route_whole_rows(T, H);
     const int tg = !whole ? (T <= 8 ? 4 : 8) : (T <= 4 ? 1 : 2);   // tokens per gate workgroup: what the kernel instantiates
-    static const int parts_env = [] { const char *e = getenv("MOE_BATCH_PARTS"); return e ? atoi(e) : 0; }();
-    a.g_parts = parts_env == 1 ? 1 : (parts_env == 8 ? GATE_PARTS : GATE_PARTS);
+    a.g_parts = GATE_PARTS;
     a.g_nblk = a.g_parts * ((T + tg - 1) / tg) * ((n_gate_rows + 3) / 4);
     int rc;
     if (!whole) {

@@ -210,25 +210,28 @@ def decode_batch_int4_gate_fits(T: int, E: int, k: int, H: int, I: int, I_sh: in
 
 
 def decode_batch_int4_gate(x, wg, bias, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int,
-                           gws: "GateWorkspace", phases: int = 3):
-    """2 to 8 tokens: gate rows, routing and w13 in one launch (phase bit 0), w2 over the published unit list (bit 1).
-    wg may carry one extra row (shared gate, no bias).
+                           gws: "GateWorkspace", phases: int = 3, ws=None):
+    """2 to 16 tokens: gate rows, routing and w13 in one launch (phase bit 0), w2 over the published unit list (bit 1).
+    wg may carry one extra row (shared gate, no bias); ws: the tuple an earlier call returned (nothing is allocated).
     Returns (logits [T, rows], idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
     T = x.shape[0]
     rows = wg.shape[0]
     dev = x.device
     P = T * k
-    logits = torch.empty(T, rows, dtype=torch.float32, device=dev)
-    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
-    w = torch.empty(T, k, dtype=torch.float32, device=dev)
-    d = Dispatch(T, k, E, min(E, P), dev)
-    h_r = torch.empty(P, I, dtype=torch.bfloat16, device=dev)
-    part_r = torch.empty(P, H, dtype=torch.float32, device=dev)
-    h_s = part_s = None
-    if shared is not None:
-        h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
-        part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
-    err = torch.zeros(1, dtype=torch.int32, device=dev)
+    if ws is not None:
+        logits, idx, w, d, part_r, part_s, err, h_r, h_s = ws
+    else:
+        logits = torch.empty(T, rows, dtype=torch.float32, device=dev)
+        idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+        w = torch.empty(T, k, dtype=torch.float32, device=dev)
+        d = Dispatch(T, k, E, min(E, P), dev)
+        h_r = torch.empty(P, I, dtype=torch.bfloat16, device=dev)
+        part_r = torch.empty(P, H, dtype=torch.float32, device=dev)
+        h_s = part_s = None
+        if shared is not None:
+            h_s = torch.empty(T, I_sh, dtype=torch.bfloat16, device=dev)
+            part_s = torch.empty(T, H, dtype=torch.float32, device=dev)
+        err = torch.zeros(1, dtype=torch.int32, device=dev)
     if gws.buf.numel() < int(lib.moe_gate_route_ws_bytes(T, rows)):
         raise L.MoeError("gate workspace too small")
     check(lib.moe_decode_batch_int4_gate(ptr(_dev(x)), T, ptr(_dev(wg)), ptr(bias), rows, ptr(gws.buf), gws.next_seq(),
