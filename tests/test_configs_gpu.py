@@ -121,6 +121,35 @@ def test_c1_deepseek_layer_T128_all_resident(cuda, deepseek_layers):
     pm.close()
 
 
+def test_c2_decode_batches_all_resident_three_launches(cuda, deepseek_layers):
+    """The DeepSeek-shaped layer with every expert resident, batches of 2 to 16 tokens (and 1, 17 and 32 around
+    them): moe_forward takes the w13 launch that sums the gate rows and routes by itself (whole-row form up to 8
+    tokens, chunked-K form from 9), then w2 and the combine.  Routing bit-exact against the oracle, outputs within
+    the tolerance of the path, the asynchronously accounted hits equal to the experts the oracle activates."""
+    print("case C2 decode batches, all resident", flush=True)
+    layer, k = deepseek_layers[1], 6
+    pm = build_engine([layer], k, cuda, max_tokens=32, cache_rate=1.0, cache_policy="lru")
+    pm.acquire_layer(0, np.arange(64, dtype=np.int64))
+    pm.release_layer(0)
+    c0 = pm.counters()
+    n_act = 0
+    for T in (4, 16, 2, 8, 12, 3, 9, 1, 17, 32, 5, 16, 4):
+        x = O.synth_acts(T, 2048, seed=1500 + T)
+        y = pm.forward(0, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
+        torch.cuda.synchronize()
+        ref = ref_forward_lazy(layer, x, k, 0)
+        assert np.array_equal(pm.last_routing_idx(T, k), ref["idx"]), T
+        err = rel_err(y, ref["out"])
+        print(f"  T={T} max-rel-err {err:.3e}", flush=True)
+        assert err <= TOL, (T, err)
+        n_act += len(np.unique(ref["idx"]))
+        layer.drop_cache()
+    pm.drain()
+    c1 = pm.counters()
+    assert c1["miss"] == c0["miss"] and c1["hit"] - c0["hit"] == n_act
+    pm.close()
+
+
 def test_c4_mixtral_layers_through_cache(cuda):
     """Two Mixtral-shaped layers (the second one holds the first one's experts in another order), cache rate
     0.5 = 4 of 8 experts per layer in 91.5 MB slots, top-2 then softmax; T = 1 and 64."""
