@@ -175,11 +175,15 @@ int moe_gate_topk_dispatch(const void *x_bf16, const void *wg_bf16, const float 
  * moe_topk_dispatch, bit for bit, and the optional host copy).  Results equal moe_gate_topk_dispatch followed by
  * moe_experts_decode_int4, bit for bit.  phases: bit 0 = that launch, bit 1 = the w2 launch over the published
  * unit list.  max_units must be min(E, T k); gate_ws / gate_seq as in moe_gate_topk_dispatch
- * (moe_gate_route_ws_bytes(T, n_gate_rows) bytes).  moe_decode_batch_int4_gate_fits says whether a shape is taken. */
+ * (moe_gate_route_ws_bytes(T, n_gate_rows) bytes).  moe_decode_batch_int4_gate_fits says whether a shape is taken.
+ *   expert_ptr_host (optional, E <= 64): a HOST copy of the slot table.  Both launches then carry the table in
+ *   their arguments and do not read expert_ptr, so a caller whose table changed since the last launch needs no
+ *   copy in the stream in front of this one (a cache that has just loaded an expert).  NULL: expert_ptr is read. */
 int moe_decode_batch_int4_gate_fits(int T, int E, int k, int H, int I, int I_sh, int n_gate_rows);
 int moe_decode_batch_int4_gate(const void *x_bf16, int T, const void *gate_w_bf16, const float *gate_bias,
                                int n_gate_rows, void *gate_ws, int gate_seq, float *logits, int ldl, int E, int k,
-                               int mode, int H, int I, int I_sh, const uint64_t *expert_ptr, const void *shared_ptr,
+                               int mode, int H, int I, int I_sh, const uint64_t *expert_ptr,
+                               const uint64_t *expert_ptr_host, const void *shared_ptr,
                                int *idx, float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids, int max_units,
                                void *h_r, void *h_s, float *part_r, float *part_s, int *err,
@@ -230,9 +234,12 @@ int moe_experts_decode_int4_publish(const void *x_bf16, int T, int H, int I, int
  * phases: bit 0 = routing + w13 + SwiGLU, bit 1 = w2 into partial rows (needs the units of an
  * earlier bit-0 call), bit 2 = w2 and the weighted combine in ONE launch, straight into y_bf16 [H]
  * (needs unit_ws of 32*k bytes; shared_gate_logit = the shared expert's gate logit or NULL; every
- * selected expert resident).  Bits 1 and 2 exclude each other. */
+ * selected expert resident).  Bits 1 and 2 exclude each other.
+ * expert_ptr_host (optional, E <= 64): a HOST copy of the slot table; the launch of phase bit 0 then carries the
+ * table in its arguments and does not read expert_ptr (no copy of a changed table in front of the launch). */
 int moe_decode_token_int4(const void *x_bf16, const float *logits, int E, int k, int mode, int H, int I,
-                          int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx, float *w,
+                          int I_sh, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host,
+                          const void *shared_ptr, int *idx, float *w,
                           int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                           moe_unit *units, int *n_active, int64_t *active_ids, void *h_r, void *h_s,
                           float *part_r, float *part_s, int *err, void *unit_ws, moe_unit *units_host_out,
@@ -263,7 +270,8 @@ int moe_decode_token_late_expert_int4(const void *x_bf16, int H, int I, uint64_t
 int64_t moe_gate_ws_bytes(void);
 int moe_decode_token_int4_gate(const void *x_bf16, const void *gate_w, const float *gate_bias, int n_gate_rows,
                                void *gate_ws, int gate_seq, float *logits, int E, int k, int mode, int H, int I,
-                               int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx, float *w,
+                               int I_sh, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host,
+                               const void *shared_ptr, int *idx, float *w,
                                int *counts, int *offsets, int *sorted_pair, int *pos_of_pair, int *sorted_tok,
                                moe_unit *units, int *n_active, int64_t *active_ids, void *h_r, void *h_s,
                                float *part_r, float *part_s, int *err, void *unit_ws, moe_unit *units_host_out,

@@ -60,14 +60,14 @@ _sig("moe_gate_route_ws_bytes", [i32, i32], i64)
 _sig("moe_gate_topk_dispatch", [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 10 +
      [i32, vp, vp, vp, i32, vp, i32, i32, vp, vp])
 _sig("moe_decode_batch_int4_gate_fits", [i32] * 7, i32)
-_sig("moe_decode_batch_int4_gate", [vp, i32, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 12 +
+_sig("moe_decode_batch_int4_gate", [vp, i32, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, i32] + [vp] * 13 +
      [i32] + [vp] * 8 + [i32, i32, vp])
 _sig("moe_noalloc_scratch_bytes", [], i64)
 _sig("moe_decode_token_int4_noalloc", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, vp])
-_sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])
+_sig("moe_decode_token_int4", [vp, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp] + [vp] * 15 + [vp, vp, vp, i32, i32, vp, vp, vp])
 _sig("moe_gate_ws_bytes", [], i64)
 _sig("moe_decode_token_late_expert_int4", [vp, i32, i32, u64, i32, vp, vp, vp, vp])
-_sig("moe_decode_token_int4_gate", [vp, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp, vp] + [vp] * 15 +
+_sig("moe_decode_token_int4_gate", [vp, vp, vp, i32, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp, vp, vp] + [vp] * 15 +
      [vp, vp, vp, i32, i32, vp, vp, vp])
 _sig("moe_predictor_windows", [vp, vp, vp])
 _sig("moe_predictor_set_model", [vp, i32, i32, vp, vp, i32])

@@ -847,6 +847,22 @@ int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resi
   return MOE_OK;
 }
 
+// The guarded snapshot without the copy to the device: for launches that carry the table in their arguments.  The
+// device table stays marked as it was, so a later launch that reads it still gets its flush.
+int moe_snapshot_table_guarded(moe_engine *eng, int layer, uint64_t *table_out, char *resident_out) {
+  ENG_GUARD(eng);
+  if (int rc = check_le(eng, layer, 0)) return rc;
+  if (!eng->slots_ready) { moe_set_error("slots not initialised"); return MOE_ESTATE; }
+  std::lock_guard<std::mutex> lk(eng->mu);
+  const size_t o = (size_t)layer * eng->cfg.num_expert;
+  for (int e = 0; e < eng->cfg.num_expert; ++e) {
+    table_out[e] = eng->h_table[o + e];
+    resident_out[e] = table_out[e] != 0;
+  }
+  eng->group_of(layer).guard++;
+  return MOE_OK;
+}
+
 void moe_guard_release(moe_engine *eng, int layer) {
   {
     std::lock_guard<std::mutex> lk(eng->mu);

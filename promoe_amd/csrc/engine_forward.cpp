@@ -37,6 +37,7 @@ struct LayerState {
   // sees them without a copy: one per layer for launches in which that must not happen (checked at the next
   // call and when the engine drains), one for launches that are allowed to meet non-resident experts
   int *err_host = nullptr, *err_loose = nullptr;
+  int *err_loose_dev = nullptr;  // device word for launches whose every workgroup of a skipped unit raises it
   // error words of the w2 + combine launches that go out before the host knows the routing, and what the host
   // expects of each once it does: 1 = must stay zero (every selected expert was resident at launch), 2 = may be
   // set (an expert was missing; that launch's output is recomputed), 0 = none outstanding.  Two words per layer,
@@ -47,6 +48,7 @@ struct LayerState {
   int *err_spec = nullptr;
   std::vector<char> spec_state;
   std::vector<unsigned> spec_turn;
+  std::vector<unsigned char> late_last;   // per layer: experts the last turn had to wait for
   int num_layer = 0;
   std::vector<void *> dev_allocs, host_allocs;
   hipEvent_t ev = nullptr;
@@ -168,6 +170,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   rc |= dalloc(s, &s->pos_of_pair, P);
   rc |= dalloc(s, &s->sorted_tok, P);
   rc |= dalloc(s, &s->n_active, 1);
+  rc |= dalloc(s, &s->err_loose_dev, 1);
   rc |= dalloc(s, &s->unit_ws, (size_t)32 * std::max(k, 1));
   s->gate_ws_bytes = (size_t)std::max<int64_t>(moe_gate_ws_bytes(), moe_gate_route_ws_bytes(std::min(T, 32), E + 1));
   rc |= dalloc(s, &s->gate_ws, s->gate_ws_bytes);
@@ -211,6 +214,7 @@ extern "C" int moe_forward_prepare(moe_engine *eng, int max_tokens) {
   memset(s->err_spec, 0, sizeof(int) * 2 * eng->cfg.num_layer);
   s->spec_state.assign((size_t)2 * eng->cfg.num_layer, 0);
   s->spec_turn.assign(eng->cfg.num_layer, 0);
+  s->late_last.assign(eng->cfg.num_layer, 0);
   HIPC(hipMemset(s->gate_ws, 0, s->gate_ws_bytes));
   if (s->disp_ws) HIPC(hipMemset(s->disp_ws, 0, 64));
   *s->opt_seq = 0;
@@ -307,6 +311,13 @@ static int shared_pieces(const moe_layer_desc &d, int T, const LayerState *s) {
 
 // what the one-token w2 + combine kernel asks of a layer (its waves stage what they need themselves, so the
 // widths of the experts do not matter; a lane per unit holds the unit's address)
+// launches that take a host copy of the slot table carry at most this many entries in their arguments
+static constexpr int kTableByValueMax = 64;
+static bool table_by_value(int E) {   // MOE_TABLE_BY_VALUE=0: always refresh and read the device table
+  static const bool on = [] { const char *e = getenv("MOE_TABLE_BY_VALUE"); return !e || atoi(e) != 0; }();
+  return on && E <= kTableByValueMax;
+}
+
 static bool w2c_fits(const moe_layer_desc &d, int k) { return d.H % 16 == 0 && k < 64; }
 
 
@@ -403,7 +414,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const bool w2c = w2c_fits(d, k);  // w2 and the combine in one launch
     s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
     if ((rc = moe_decode_token_int4_gate(x, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, E, k,
-                                         d.route_mode, d.H, d.I, d.I_sh, table,
+                                         d.route_mode, d.H, d.I, d.I_sh, table, nullptr,
                                          d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                          s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                          s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws, p.units, p.seq, seq,
@@ -442,7 +453,15 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
     // what the kernel will find resident: exactly these experts get computed by it
     std::vector<char> resident_at_launch(E);
-    if ((rc = moe_flush_table_guarded(eng, layer, st, resident_at_launch.data()))) return rc;
+    // Up to 64 experts the launches below carry the slot table in their arguments (the routing launch) or take
+    // resolved units (the others): the device table is not read, and its refresh after a miss, a copy in the stream
+    // in front of the routing launch, is not made (it held the routing back from the host, and with it the demand
+    // copy of the next miss, by 5 to 7 us).
+    uint64_t tab_now[kTableByValueMax];
+    const uint64_t *tab_host = table_by_value(E) ? tab_now : nullptr;
+    if ((rc = tab_host ? moe_snapshot_table_guarded(eng, layer, tab_now, resident_at_launch.data())
+                       : moe_flush_table_guarded(eng, layer, st, resident_at_launch.data())))
+      return rc;
     struct GuardRelease {  // on every way out, errors included
       moe_engine *eng; int layer; bool armed;
       void release() { if (armed) { armed = false; moe_guard_release(eng, layer); } }
@@ -450,7 +469,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     } guard{eng, layer, true};
     const int seq = ++s->seq_counter;
     if (pred_fused) {
-      rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+      rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table, tab_host,
                                  d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                  s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                  s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
@@ -458,7 +477,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     } else {
       s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
       rc = moe_decode_token_int4_gate(x, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, E, k,
-                                      d.route_mode, d.H, d.I, d.I_sh, table,
+                                      d.route_mode, d.H, d.I, d.I_sh, table, tab_host,
                                       d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                       s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                       s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws, s->units_host, s->opt_seq, seq, 1,
@@ -480,7 +499,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
         return engine_fail(eng, "a kernel of layer %d met a selected expert without a slot: its output is wrong", layer);
       s->spec_state[sw] = 0;
       s->err_spec[sw] = 0;
-      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table, nullptr,
                                       d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                       s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                       s->h_r, s->h_s, s->part_r, s->part_s, s->err_spec + sw, s->unit_ws,
@@ -537,7 +556,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       late_w13_only = later.size() + now_ids.size() <= eng->group_of(layer).full_len;
     }
     if (!w2c && !late_w13_only &&
-        (rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+        (rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table, nullptr,
                                     d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                     s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                     s->h_r, s->h_s, s->part_r, s->part_s, s->err_loose, s->unit_ws,
@@ -572,7 +591,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
     }
     if (late_w13_only) {
-      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table,
+      if ((rc = moe_decode_token_int4(x, s->logits, E, k, d.route_mode, d.H, d.I, d.I_sh, table, nullptr,
                                       d.I_sh > 0 ? d.shared : nullptr, s->idx, s->topk_w, s->counts, s->offsets,
                                       s->sorted_pair, s->pos_of_pair, s->sorted_tok, s->units, s->n_active, s->active_ids,
                                       s->h_r, s->h_s, s->part_r, s->part_s, s->err_host + layer, s->unit_ws,
@@ -600,7 +619,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_flush_table(eng, layer, st))) return rc;
     s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
     if ((rc = moe_decode_batch_int4_gate(x, T, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, ldl, E,
-                                         k, d.route_mode, d.H, d.I, d.I_sh, table, d.I_sh > 0 ? d.shared : nullptr, s->idx,
+                                         k, d.route_mode, d.H, d.I, d.I_sh, table, nullptr, d.I_sh > 0 ? d.shared : nullptr, s->idx,
                                          s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
                                          s->units, s->n_active, s->active_ids, max_units, s->h_r, s->h_s, s->part_r,
                                          s->part_s, s->err_host + layer, p.units, p.n_active, p.seq, seq, 3, st)))
@@ -609,6 +628,108 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     const float *sg0 = d.shared_gated ? s->logits + E : nullptr;
     if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sg0, ldl, y, T, d.H, k,
                                  1, st)))
+      return rc;
+    if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
+    return moe_layer_done(eng, layer);
+  }
+  static const bool batch_spec_on = [] { const char *e = getenv("MOE_BATCH_SPEC"); return !e || atoi(e) != 0; }();
+  // (more than 8 tokens: only while the layer's last turn missed at most one expert; with several misses a step the
+  // time is in the copies, which start no earlier this way, and the recomputed units cost more than the wait saved:
+  // 16 tokens at cache rate 0.375 370 -> 379 us per step, at 0.97 85 -> 77)
+  if (!all_resident && batch_spec_on && eng->cfg.early_preempt && eng->cfg.reorder_experts &&
+      (T <= 8 || s->late_last[layer] <= 1) && batch_routes_in_w13(d, s, T, E, k, n_gate_rows)) {
+    // 2 to 16 tokens that may meet non-resident experts: as for one token, the expert launches go out BEFORE the host
+    // knows the routing.  The self-routing w13 launch and the w2 launch behind it compute what is resident (a unit
+    // whose table entry is 0 is skipped and raises the loose error word) and hand the unit list to the host, which
+    // runs the cache hooks in the reference's order while the GPU works; the units that were not resident follow as
+    // their copies land, then the combine.  The GPU used to idle from the end of the routing launch until the host had
+    // seen the routing, run the hooks and launched (about 8 us per step).  The slot group is guarded from the table
+    // snapshot until the hooks have marked the hits, as in the one-token path.
+    const uint64_t *table = nullptr;
+    if ((rc = moe_expert_ptr_table(eng, layer, &table))) return rc;
+    std::vector<char> resident_at_launch(E);
+    uint64_t tab_now[kTableByValueMax];   // (the launches carry the table in their arguments: no refresh of the device table)
+    const uint64_t *tab_host = table_by_value(E) ? tab_now : nullptr;
+    if ((rc = tab_host ? moe_snapshot_table_guarded(eng, layer, tab_now, resident_at_launch.data())
+                       : moe_flush_table_guarded(eng, layer, st, resident_at_launch.data())))
+      return rc;
+    struct GuardRelease {  // on every way out, errors included
+      moe_engine *eng; int layer; bool armed;
+      void release() { if (armed) { armed = false; moe_guard_release(eng, layer); } }
+      ~GuardRelease() { release(); }
+    } guard{eng, layer, true};
+    const int seq = ++s->seq_counter;
+    s->gate_seq = s->gate_seq < 0x7fffffff ? s->gate_seq + 1 : 1;
+    if ((rc = moe_decode_batch_int4_gate(x, T, d.gate_w, d.gate_bias, n_gate_rows, s->gate_ws, s->gate_seq, s->logits, ldl, E,
+                                         k, d.route_mode, d.H, d.I, d.I_sh, table, tab_host, d.I_sh > 0 ? d.shared : nullptr, s->idx,
+                                         s->topk_w, s->counts, s->offsets, s->sorted_pair, s->pos_of_pair, s->sorted_tok,
+                                         s->units, s->n_active, s->active_ids, max_units, s->h_r, s->h_s, s->part_r,
+                                         s->part_s, s->err_loose_dev, s->units_host, s->n_active_host, s->opt_seq, seq, 3, st)))
+      return rc;
+    {  // the routing arrives a few microseconds after the launch starts
+      volatile int *sq = s->opt_seq;
+      const auto t0 = std::chrono::steady_clock::now();
+      unsigned spins = 0;
+      while (*sq != seq) {
+        if ((++spins & 1023u) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
+          HIPC(hipStreamSynchronize(st));
+          if (*sq != seq) { moe_set_error("routing of layer %d never reached the host", layer); return MOE_EHIP; }
+        }
+      }
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    }
+    const int n_act = std::min(*s->n_active_host, max_units);
+    std::vector<int64_t> ids(n_act);
+    std::unordered_map<int, moe_unit> unit_of;
+    for (int u = 0; u < n_act; ++u) { ids[u] = s->units_host[u].expert; unit_of[s->units_host[u].expert] = s->units_host[u]; }
+    if ((rc = moe_report_one_layer(eng, layer, ids.data(), n_act))) return rc;
+    std::vector<int64_t> later, now_ids;
+    {
+      std::lock_guard<std::mutex> lk(eng->mu);
+      for (int i = 0; i < n_act; ++i) {
+        // resident at launch and still there (now `launching`): computed already; anything else (missed, or evicted
+        // by a prefetch between the snapshot and the hooks) is computed when it is usable
+        Expert *ex = eng->ex(layer, (int)ids[i]);
+        if (resident_at_launch[(int)ids[i]] && ex->status.load() == kLaunching && ex->num_ready == eng->cfg.num_per_expert_param &&
+            eng->h_table[(size_t)layer * E + ids[i]] != 0)
+          now_ids.push_back(ids[i]);
+        else
+          later.push_back(ids[i]);
+      }
+      eng->ctr.ready += (uint64_t)now_ids.size();
+    }
+    s->late_last[layer] = (unsigned char)std::min<size_t>(later.size(), 255);
+    guard.release();
+    // launching -> using.  No event in the stream where that is safe: the experts count as in use until the sequence
+    // word of a LATER launch arrives.  A batch can route to more experts than the layer has slots, and then a demand
+    // copy of this very step picks one of these experts as its victim: it would stand for the 100 us the fetch thread
+    // gives the word before it falls back to an event (16 tokens at cache rate 0.375: 373 -> 381-389 us per step), so
+    // such a step releases against an event recorded now.  (With the routed experts no more than the slots, the
+    // victims of this step's copies are experts it did not touch: they are the least recently used.)
+    if (!now_ids.empty()) {
+      size_t slots_of_layer;
+      {
+        std::lock_guard<std::mutex> lk(eng->mu);
+        slots_of_layer = eng->group_of(layer).full_len;
+      }
+      rc = (size_t)n_act <= slots_of_layer && eng->cfg.per_layer_cache
+               ? moe_release_experts_seq(eng, layer, now_ids.data(), (int64_t)now_ids.size(), s->opt_seq, seq + 1)
+               : moe_release_experts(eng, layer, now_ids.data(), (int64_t)now_ids.size());
+      if (rc) return rc;
+    }
+    s->sub_cursor = 0;
+    for (int64_t id : later) {
+      if ((rc = moe_wait_expert(eng, layer, (int)id))) return rc;
+      moe_unit *slot_h = s->units_sub_host + s->sub_cursor;
+      *slot_h = unit_of[(int)id];
+      // (one unit by value: its slot address travels in the kernel arguments, the device table is not read)
+      if ((rc = run_units(eng, d, s, x, T, s->units_sub + s->sub_cursor, slot_h, 1, false, layer, table, st))) return rc;
+      s->sub_cursor++;
+      if ((rc = moe_expert_launched(eng, layer, (int)id))) return rc;
+    }
+    const float *sgo = d.shared_gated ? s->logits + E : nullptr;
+    if ((rc = moe_combine_splits(s->part_r, d.I_sh > 0 ? s->part_s : nullptr, s->topk_w, s->pos_of_pair, sgo, ldl, y, T, d.H, k, 1,
+                                 st)))
       return rc;
     if (layer + 1 == eng->cfg.num_layer && (rc = moe_report_layer_logits(eng, layer + 1, y, 1, T, d.H))) return rc;
     return moe_layer_done(eng, layer);
@@ -717,11 +838,13 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     }
     eng->ctr.ready += (uint64_t)n_now;
   }
-  if ((rc = moe_flush_table(eng, layer, st))) return rc;
+  s->late_last[layer] = (unsigned char)std::min<size_t>(later.size(), 255);
   // int4 decode launches of up to 64 units take the units and their slot addresses in the kernel arguments
   // (run_units hands over the host copies): the device copy of a sub-list is then never read, and its
-  // host-to-device copy would only put 4 us into the stream in front of the launch
+  // host-to-device copy would only put 4 us into the stream in front of the launch.  The same holds for the
+  // refresh of the device table after a miss, which such a launch does not read either.
   const bool by_value = d.fmt == MOE_FMT_INT4_G128 && !use_prefill(d, T);
+  if (!(by_value && n_now <= 64) && (rc = moe_flush_table(eng, layer, st))) return rc;
   const moe_unit *units_now = s->units;
   if (!later.empty() || n_now != n_act) {
     if (n_now && !(by_value && n_now <= 64))

@@ -237,6 +237,7 @@ int moe_report_layer_logits_bookkeeping(moe_engine *eng, int layer, int S);
 // slot table of `layer` to the device (if changed) and the same residency as a byte vector, taken in one
 // critical section together with raising the group's guard; moe_guard_release lowers it again
 int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resident_out);
+int moe_snapshot_table_guarded(moe_engine *eng, int layer, uint64_t *table_out, char *resident_out);
 void moe_guard_release(moe_engine *eng, int layer);
 int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int64_t n, int blocking, bool over_copy);
 // every expert that waits for a sequence word becomes ready (the caller has drained the compute stream)

@@ -727,8 +727,15 @@ struct GemvArgs {
   const unsigned char *shared_base;
   int n_sh_blocks, T;
   int *err;
-  KUnit ku[GEMV_MAX_KUNITS];             // units resolved on the host, passed by value: the
+  union {
+    KUnit ku[GEMV_MAX_KUNITS];           // units resolved on the host, passed by value: the
                                          // weight loads then depend on no global load
+    // tab_n > 0 (launches that take their units from device memory and so leave ku unused): the slot table of
+    // experts 0 .. tab_n - 1 by value.  The device table is then not read, and no copy that refreshes it has to
+    // stand in the stream in front of the launch.
+    unsigned long long tab[GEMV_MAX_KUNITS];
+  };
+  int tab_n, tab_pad;
   // one-token launches that route inside the kernel (ROUTE): inputs and the routing outputs
   const float *r_logits;
   int r_E, r_k, r_mode, r_pad;
@@ -926,6 +933,21 @@ static __device__ __forceinline__ void gemv_publish_units(const GemvArgs &a) {
   if (tid == 0) __hip_atomic_store(a.p_host_seq, a.p_seq_val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// Slot address of expert e: from the kernel arguments when the launch carries the table, else from the device table.
+static __device__ __forceinline__ unsigned long long slot_of(const GemvArgs &a, const int e) {
+  return a.tab_n > 0 ? (e < a.tab_n ? a.tab[e] : 0ull) : a.expert_ptr[e];
+}
+
+// Host side: the table by value when the caller has a host copy and it fits, else the device table.
+static void gemv_set_table(GemvArgs &a, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host, int E) {
+  a.expert_ptr = (const unsigned long long *)expert_ptr;
+  a.tab_n = 0;
+  if (expert_ptr_host && E > 0 && E <= GEMV_MAX_KUNITS) {
+    for (int e = 0; e < E; ++e) a.tab[e] = expert_ptr_host[e];
+    a.tab_n = E;
+  }
+}
+
 // bx: the workgroup's index among the working ones (launches with a publishing workgroup put that one first)
 // BY_ROWS (device-built unit list of at most 64 slots, a.unit_slots > 0): position u of the grid takes the unit of
 // rank u when the units are ordered by the passes they need (more than 32 rows, 17 to 32, 1 to 16, none; list
@@ -983,12 +1005,12 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
           const int ue = __builtin_amdgcn_readlane((int)ul.x, src);
           wk.m = __builtin_amdgcn_readlane(ml, src);
           wk.row0 = __builtin_amdgcn_readlane((int)ul.z, src);
-          wk.base = wk.m > 0 ? (const unsigned char *)a.expert_ptr[ue] : nullptr;
+          wk.base = wk.m > 0 ? (const unsigned char *)slot_of(a, ue) : nullptr;
         }
       } else {
         const moe_unit ud = a.units[u];
         wk.m = ud.m; wk.row0 = ud.row0;
-        wk.base = ud.m > 0 ? (const unsigned char *)a.expert_ptr[ud.expert] : nullptr;
+        wk.base = ud.m > 0 ? (const unsigned char *)slot_of(a, ud.expert) : nullptr;
       }
     }
   } else {
@@ -1056,7 +1078,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
   for (int r = 0; r < NR; ++r) {
     const int e = lane + 64 * r;
     v[r] = (e < E && a.g_nblk == 0) ? a.r_logits[e] : NEG;
-    ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
+    ptrs[r] = (e < E) ? slot_of(a, e) : 0ull;
   }
   bool gate_timeout = false;
   if (a.g_nblk) {
@@ -1190,7 +1212,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_n(const GemvArgs &
       moe_unit un; un.expert = my_e; un.m = 1; un.row0 = pos; un.pad = 0;
       a.r_units[pos] = un;
       a.r_active_ids[pos] = my_e;
-      if (a.r_kunits) { KUnit kd; kd.base = a.expert_ptr[my_e]; kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; a.r_unit_w[pos] = wgt; }
+      if (a.r_kunits) { KUnit kd; kd.base = slot_of(a, my_e); kd.m = 1; kd.row0 = pos; a.r_kunits[pos] = kd; a.r_unit_w[pos] = wgt; }
     }
 #pragma unroll
     for (int r = 0; r < NR; ++r) {
@@ -1413,7 +1435,7 @@ static __device__ __forceinline__ GemvWork gemv_resolve_route_batch_n(const Gemv
 #pragma unroll
   for (int r = 0; r < NR; ++r) {
     const int e = lane + 64 * r;
-    ptrs[r] = (e < E) ? a.expert_ptr[e] : 0ull;
+    ptrs[r] = (e < E) ? slot_of(a, e) : 0ull;
   }
   const rsrc_t rl = make_rsrc(a.g_stamp + (size_t)xcc_id() * a.g_copy_words, (u32)a.g_copy_words * 8u);
   const unsigned long long *cg = a.g_stamp + (size_t)GATE_PARTS * a.g_copy_words;
@@ -3444,6 +3466,16 @@ extern "C" int moe_experts_decode_int4(const void *x, int T, int H, int I, int I
                                          nullptr, nullptr, nullptr, 0, stream);
 }
 
+// tab_host/tab_E: a host copy of the slot table to put into the arguments of launches that take the device unit list
+static int experts_decode_int4_impl(const void *x, int T, int H, int I, int I_sh, int k,
+                                    const moe_unit *units, int max_units, const int *sorted_tok,
+                                    const uint64_t *expert_ptr, const void *shared_ptr,
+                                    void *h_r, void *h_s, float *part_r, float *part_s,
+                                    int *err, const moe_unit *units_host,
+                                    const uint64_t *expert_ptr_host, int phases,
+                                    const int *n_active, moe_unit *units_host_out, int *n_active_host_out,
+                                    int *seq_host_out, int seq_value, const uint64_t *tab_host, int tab_E, void *stream);
+
 extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int I, int I_sh, int k,
                                                const moe_unit *units, int max_units, const int *sorted_tok,
                                                const uint64_t *expert_ptr, const void *shared_ptr,
@@ -3452,6 +3484,19 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
                                                const uint64_t *expert_ptr_host, int phases,
                                                const int *n_active, moe_unit *units_host_out, int *n_active_host_out,
                                                int *seq_host_out, int seq_value, void *stream) {
+  return experts_decode_int4_impl(x, T, H, I, I_sh, k, units, max_units, sorted_tok, expert_ptr, shared_ptr, h_r, h_s, part_r,
+                                  part_s, err, units_host, expert_ptr_host, phases, n_active, units_host_out,
+                                  n_active_host_out, seq_host_out, seq_value, nullptr, 0, stream);
+}
+
+static int experts_decode_int4_impl(const void *x, int T, int H, int I, int I_sh, int k,
+                                    const moe_unit *units, int max_units, const int *sorted_tok,
+                                    const uint64_t *expert_ptr, const void *shared_ptr,
+                                    void *h_r, void *h_s, float *part_r, float *part_s,
+                                    int *err, const moe_unit *units_host,
+                                    const uint64_t *expert_ptr_host, int phases,
+                                    const int *n_active, moe_unit *units_host_out, int *n_active_host_out,
+                                    int *seq_host_out, int seq_value, const uint64_t *tab_host, int tab_E, void *stream) {
   if (units_host_out && (T < 2 || !units || units_host || !n_active || !n_active_host_out || !seq_host_out ||
                          !(phases & 1) || max_units <= 0)) {
     moe_set_error("moe_experts_decode_int4_publish: publishing needs T >= 2, the device unit list, its length and "
@@ -3476,6 +3521,7 @@ extern "C" int moe_experts_decode_int4_publish(const void *x, int T, int H, int 
   a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
   a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err;
   a.pairs = k > 0 ? T * k : 0;
+  if (units && !units_host && tab_host) gemv_set_table(a, expert_ptr, tab_host, tab_E);
   if (units_host && expert_ptr_host && max_units <= GEMV_MAX_KUNITS) {
     a.units = nullptr;
     for (int u = 0; u < max_units; ++u) {
@@ -3590,6 +3636,7 @@ extern "C" int moe_decode_batch_int4_gate_fits(int T, int E, int k, int H, int I
 extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate_w, const float *gate_bias,
                                           int n_gate_rows, void *gate_ws, int gate_seq, float *logits, int ldl, int E,
                                           int k, int mode, int H, int I, int I_sh, const uint64_t *expert_ptr,
+                                          const uint64_t *expert_ptr_host,
                                           const void *shared_ptr, int *idx, float *w, int *counts, int *offsets,
                                           int *sorted_pair, int *pos_of_pair, int *sorted_tok, moe_unit *units,
                                           int *n_active, int64_t *active_ids, int max_units, void *h_r, void *h_s,
@@ -3618,7 +3665,7 @@ extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate
     const bool sh = shared_ptr != nullptr;
     GemvArgs a;
     memset(&a, 0, sizeof a);
-    a.expert_ptr = (const unsigned long long *)expert_ptr;
+    gemv_set_table(a, expert_ptr, expert_ptr_host, E);
     a.shared_base = (const unsigned char *)shared_ptr; a.T = T; a.err = err; a.pairs = T * k;
     a.r_E = E; a.r_k = k; a.r_mode = mode; a.r_idx = idx; a.r_w = w; a.r_counts = counts; a.r_offsets = offsets;
     a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok; a.r_units = units;
@@ -3657,8 +3704,9 @@ extern "C" int moe_decode_batch_int4_gate(const void *x, int T, const void *gate
     if (rc) return rc;
   }
   if (phases & 2)  // w2 over the unit list the first launch published
-    return moe_experts_decode_int4(x, T, H, I, shared_ptr ? I_sh : 0, k, units, max_units, sorted_tok, expert_ptr, shared_ptr,
-                                   h_r, h_s, part_r, part_s, err, nullptr, nullptr, 2, stream);
+    return experts_decode_int4_impl(x, T, H, I, shared_ptr ? I_sh : 0, k, units, max_units, sorted_tok, expert_ptr, shared_ptr,
+                                    h_r, h_s, part_r, part_s, err, nullptr, nullptr, 2, nullptr, nullptr, nullptr, nullptr, 0,
+                                    expert_ptr_host, E, stream);
   return MOE_OK;
 }
 
@@ -3692,7 +3740,8 @@ static int launch_gemv_route(const GemvArgs &a, int grid, size_t lds, hipStream_
 // gate_w != NULL: the launch of phase bit 0 computes the gate logits itself (moe_decode_token_int4_gate)
 static int decode_token_int4_impl(const void *gate_w, const float *gate_bias, int n_gate_rows, void *gate_ws,
                                   int gate_seq, const void *x, const float *logits, int E, int k, int mode, int H, int I,
-                                     int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                     int I_sh, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host,
+                                     const void *shared_ptr, int *idx,
                                      float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
@@ -3718,7 +3767,7 @@ static int decode_token_int4_impl(const void *gate_w, const float *gate_bias, in
   hipStream_t s = (hipStream_t)stream;
   GemvArgs a;
   memset(&a, 0, sizeof a);
-  a.units = units; a.expert_ptr = (const unsigned long long *)expert_ptr;
+  a.units = units; gemv_set_table(a, expert_ptr, expert_ptr_host, E);
   a.shared_base = (const unsigned char *)shared_ptr; a.T = 1; a.err = err;
   a.r_logits = logits; a.r_E = E; a.r_k = k; a.r_mode = mode; a.r_idx = idx; a.r_w = w; a.r_counts = counts;
   a.r_offsets = offsets; a.r_sorted_pair = sorted_pair; a.r_pos_of_pair = pos_of_pair; a.r_sorted_tok = sorted_tok;
@@ -3790,13 +3839,15 @@ static int decode_token_int4_impl(const void *gate_w, const float *gate_bias, in
 }
 
 extern "C" int moe_decode_token_int4(const void *x, const float *logits, int E, int k, int mode, int H, int I,
-                                     int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                     int I_sh, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host,
+                                     const void *shared_ptr, int *idx,
                                      float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                      int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                      void *h_r, void *h_s, float *part_r, float *part_s, int *err,
                                      void *unit_ws, moe_unit *units_host_out, int *seq_host_out, int seq_value,
                                      int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
-  return decode_token_int4_impl(nullptr, nullptr, 0, nullptr, 0, x, logits, E, k, mode, H, I, I_sh, expert_ptr, shared_ptr,
+  return decode_token_int4_impl(nullptr, nullptr, 0, nullptr, 0, x, logits, E, k, mode, H, I, I_sh, expert_ptr,
+                                expert_ptr_host, shared_ptr,
                                 idx, w, counts, offsets, sorted_pair, pos_of_pair, sorted_tok, units, n_active, active_ids,
                                 h_r, h_s, part_r, part_s, err, unit_ws, units_host_out, seq_host_out, seq_value, phases,
                                 shared_gate_logit, y_bf16, stream);
@@ -3806,7 +3857,8 @@ extern "C" int64_t moe_gate_ws_bytes(void) { return (int64_t)GATE_COPIES * GATE_
 
 extern "C" int moe_decode_token_int4_gate(const void *x, const void *gate_w, const float *gate_bias, int n_gate_rows,
                                           void *gate_ws, int gate_seq, float *logits, int E, int k, int mode, int H,
-                                          int I, int I_sh, const uint64_t *expert_ptr, const void *shared_ptr, int *idx,
+                                          int I, int I_sh, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host,
+                                          const void *shared_ptr, int *idx,
                                           float *w, int *counts, int *offsets, int *sorted_pair, int *pos_of_pair,
                                           int *sorted_tok, moe_unit *units, int *n_active, int64_t *active_ids,
                                           void *h_r, void *h_s, float *part_r, float *part_s, int *err,
@@ -3814,8 +3866,8 @@ extern "C" int moe_decode_token_int4_gate(const void *x, const void *gate_w, con
                                           int phases, const float *shared_gate_logit, void *y_bf16, void *stream) {
   if (!gate_w) { moe_set_error("moe_decode_token_int4_gate: no gate matrix"); return MOE_EINVAL; }
   return decode_token_int4_impl(gate_w, gate_bias, n_gate_rows, gate_ws, gate_seq, x, logits, E, k, mode, H, I, I_sh,
-                                expert_ptr, shared_ptr, idx, w, counts, offsets, sorted_pair, pos_of_pair, sorted_tok,
-                                units, n_active, active_ids, h_r, h_s, part_r, part_s, err, unit_ws, units_host_out,
+                                expert_ptr, expert_ptr_host, shared_ptr, idx, w, counts, offsets, sorted_pair, pos_of_pair,
+                                sorted_tok, units, n_active, active_ids, h_r, h_s, part_r, part_s, err, unit_ws, units_host_out,
                                 seq_host_out, seq_value, phases, shared_gate_logit, y_bf16, stream);
 }
 
@@ -3874,7 +3926,7 @@ extern "C" int moe_decode_token_int4_noalloc(const void *x, const float *logits,
   uint16_t *h_s = ws->h + (((size_t)k * I + 7) & ~(size_t)7);
   // phases 5 never touches the partial-row buffers; the entry point it shares wants them non-null
   float *unused_part = (float *)ws->h;
-  return moe_decode_token_int4(x, logits, E, k, mode, H, I, I_sh, expert_ptr, shared_ptr, ws->idx, ws->w, ws->counts,
+  return moe_decode_token_int4(x, logits, E, k, mode, H, I, I_sh, expert_ptr, nullptr, shared_ptr, ws->idx, ws->w, ws->counts,
                                ws->offsets, ws->sorted_pair, ws->pos_of_pair, ws->sorted_tok, ws->units, &ws->n_active,
                                (int64_t *)ws->active_ids, h_r, shared_ptr ? h_s : nullptr, unused_part,
                                shared_ptr ? unused_part : nullptr, err, ws->unit_ws, nullptr, nullptr, 0, 5,

@@ -210,8 +210,10 @@ def decode_batch_int4_gate_fits(T: int, E: int, k: int, H: int, I: int, I_sh: in
 
 
 def decode_batch_int4_gate(x, wg, bias, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int,
-                           gws: "GateWorkspace", phases: int = 3, ws=None):
+                           gws: "GateWorkspace", phases: int = 3, ws=None, expert_ptr_host=None):
     """2 to 16 tokens: gate rows, routing and w13 in one launch (phase bit 0), w2 over the published unit list (bit 1).
+    expert_ptr_host: a CPU int64 tensor holding the slot table (E <= 64): both launches take the table from their
+    arguments instead of reading expert_ptr.
     wg may carry one extra row (shared gate, no bias); ws: the tuple an earlier call returned (nothing is allocated).
     Returns (logits [T, rows], idx, w, Dispatch, part_r, part_s, err, h_r, h_s)."""
     T = x.shape[0]
@@ -236,8 +238,8 @@ def decode_batch_int4_gate(x, wg, bias, E: int, k: int, mode: int, expert_ptr, s
         raise L.MoeError("gate workspace too small")
     check(lib.moe_decode_batch_int4_gate(ptr(_dev(x)), T, ptr(_dev(wg)), ptr(bias), rows, ptr(gws.buf), gws.next_seq(),
                                          ptr(logits), rows, E, k, mode, H, I, I_sh if shared is not None else 0,
-                                         ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
-                                         ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                         ptr(expert_ptr), ptr(expert_ptr_host), ptr(shared), ptr(idx), ptr(w), ptr(d.counts),
+                                         ptr(d.offsets), ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
                                          ptr(d.n_active), ptr(d.active_ids), d.max_units, ptr(h_r), ptr(h_s),
                                          ptr(part_r), ptr(part_s), ptr(err), 0, 0, 0, 0, phases, cur_stream()),
           "moe_decode_batch_int4_gate")
@@ -245,8 +247,10 @@ def decode_batch_int4_gate(x, wg, bias, E: int, k: int, mode: int, expert_ptr, s
 
 
 def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, H: int, I: int, I_sh: int, ws=None,
-                      phases: int = 3, unit_ws=None, sg_logit=None, y=None, gate=None):
+                      phases: int = 3, unit_ws=None, sg_logit=None, y=None, gate=None, expert_ptr_host=None):
     """One token: routing inside the w13 kernel.  Returns (idx, w, Dispatch, part_r, part_s, err, h_r, h_s).
+    expert_ptr_host: a CPU int64 tensor holding the slot table (E <= 64): the routing launch takes the table from its
+    arguments instead of reading expert_ptr.
     gate = (gate_w [rows, H] bf16, bias [E] or None, GateWorkspace): the launch computes the gate logits too and
     `logits` (rows fp32) is an output."""
     dev = x.device
@@ -267,16 +271,16 @@ def decode_token_int4(x, logits, E: int, k: int, mode: int, expert_ptr, shared, 
         gw, gb, gws = gate
         check(lib.moe_decode_token_int4_gate(ptr(_dev(x)), ptr(gw), ptr(gb), gw.shape[0], ptr(gws.buf), gws.next_seq(),
                                              ptr(logits), E, k, mode, H, I, I_sh if shared is not None else 0,
-                                             ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
-                                             ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                             ptr(expert_ptr), ptr(expert_ptr_host), ptr(shared), ptr(idx), ptr(w), ptr(d.counts),
+                                             ptr(d.offsets), ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
                                              ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r),
                                              ptr(part_s), ptr(err), ptr(unit_ws), 0, 0, 0, phases, ptr(sg_logit), ptr(y),
                                              cur_stream()),
               "moe_decode_token_int4_gate")
         return idx, w, d, part_r, part_s, err, h_r, h_s
     check(lib.moe_decode_token_int4(ptr(_dev(x)), ptr(logits), E, k, mode, H, I, I_sh if shared is not None else 0,
-                                    ptr(expert_ptr), ptr(shared), ptr(idx), ptr(w), ptr(d.counts), ptr(d.offsets),
-                                    ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
+                                    ptr(expert_ptr), ptr(expert_ptr_host), ptr(shared), ptr(idx), ptr(w), ptr(d.counts),
+                                    ptr(d.offsets), ptr(d.sorted_pair), ptr(d.pos_of_pair), ptr(d.sorted_tok), ptr(d.units),
                                     ptr(d.n_active), ptr(d.active_ids), ptr(h_r), ptr(h_s), ptr(part_r), ptr(part_s),
                                     ptr(err), ptr(unit_ws), 0, 0, 0, phases, ptr(sg_logit), ptr(y), cur_stream()),
           "moe_decode_token_int4")
