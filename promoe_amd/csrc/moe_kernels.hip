@@ -937,6 +937,15 @@ static __device__ __forceinline__ void gemv_publish_units(const GemvArgs &a) {
 static __device__ __forceinline__ unsigned long long slot_of(const GemvArgs &a, const int e) {
   return a.tab_n > 0 ? (e < a.tab_n ? a.tab[e] : 0ull) : a.expert_ptr[e];
 }
+// The same for an expert id that is the same in every lane: the address comes back in scalar registers, so that the
+// buffer descriptors made from it need no loop over the lanes' values (an indexed read of the argument block is a
+// vector load to the compiler, and everything derived from it counts as different per lane).
+static __device__ __forceinline__ unsigned long long slot_of_uniform(const GemvArgs &a, const int e) {
+  const unsigned long long v = slot_of(a, e);
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(v >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
 
 // Host side: the table by value when the caller has a host copy and it fits, else the device table.
 static void gemv_set_table(GemvArgs &a, const uint64_t *expert_ptr, const uint64_t *expert_ptr_host, int E) {
@@ -1005,12 +1014,12 @@ static __device__ __forceinline__ GemvWork gemv_resolve(const GemvArgs &a, const
           const int ue = __builtin_amdgcn_readlane((int)ul.x, src);
           wk.m = __builtin_amdgcn_readlane(ml, src);
           wk.row0 = __builtin_amdgcn_readlane((int)ul.z, src);
-          wk.base = wk.m > 0 ? (const unsigned char *)slot_of(a, ue) : nullptr;
+          wk.base = wk.m > 0 ? (const unsigned char *)slot_of_uniform(a, ue) : nullptr;
         }
       } else {
         const moe_unit ud = a.units[u];
         wk.m = ud.m; wk.row0 = ud.row0;
-        wk.base = ud.m > 0 ? (const unsigned char *)slot_of(a, ud.expert) : nullptr;
+        wk.base = ud.m > 0 ? (const unsigned char *)slot_of_uniform(a, ud.expert) : nullptr;
       }
     }
   } else {

@@ -229,20 +229,23 @@ def test_patched_module_mirror_matches_oracle(cuda, fused):
     pm.close()
 
 
-def test_forward_single_token_starts_before_the_host_knows_the_routing(cuda):
-    """Demand fetching only (no prefetch producer): a one-token forward launches the self-routing
-    expert kernel on whatever is resident, learns the routing from pinned memory and serves the
-    misses afterwards.  Outputs, residency and counters must still follow the reference logic."""
-    print("case engine_forward optimistic", flush=True)
-    Lyr, E, k = 3, 16, 4
+@pytest.mark.parametrize("E,batch,steps", [(16, 3, 12), (80, 3, 30), (16, 12, 12), (24, 16, 10)])
+def test_forward_single_token_starts_before_the_host_knows_the_routing(cuda, E, batch, steps):
+    """Demand fetching only (no prefetch producer): a forward of one token (or of a decode batch of up to 16) launches
+    the self-routing expert kernel on whatever is resident, learns the routing from pinned memory and serves the
+    misses afterwards.  Outputs, residency and counters must still follow the reference logic.  Up to 64 experts
+    the launches carry the slot table in their arguments; with 80 they read the device table, refreshed in the
+    stream after every miss."""
+    print(f"case engine_forward optimistic E={E} batch={batch}", flush=True)
+    Lyr, k = 3, 4
     layers = [Int4Layer(H=256, I=384, E=E, I_sh=256, seed=50 + l, zipf=1.2) for l in range(Lyr)]
     cfg = dict(cache_rate=0.375, cache_policy="lru", num_predict_expert_per_layer=0, reorder_experts=True,
                early_preempt=True)
     pm = build_engine(layers, k, cuda, **cfg)
     sim = CO.CacheSim(Lyr, E, 6, k, cache_rate=0.375, policy="lru", num_predict=0, reorder=True, early_preempt=True)
     worst = 0.0
-    for step in range(12):
-        T = 1 if step % 5 else 3          # mostly single tokens, a few small batches in between
+    for step in range(steps):
+        T = 1 if step % 5 and batch < 8 else batch    # mostly single tokens with a few small batches in between, or batches only
         for l in range(Lyr):
             x = O.synth_acts(T, 256, seed=400 + step * Lyr + l)
             y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
