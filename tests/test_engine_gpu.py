@@ -372,11 +372,12 @@ def test_trained_predictor_models_beat_demand_fetching_on_held_out_steps(cuda, t
     assert c1["miss"] < c0["miss"]
 
 
-def test_one_token_path_under_wrong_prefetches(cuda):
+@pytest.mark.parametrize("T", [1, 3, 12])
+def test_one_token_path_under_wrong_prefetches(cuda, T):
     """A predictor with random models keeps evicting experts the tokens are about to use, while the one-token
-    path launches its kernels on table snapshots: the outputs must stay the oracle's (the slot-group guard and
-    the late classification of evicted experts are what this exercises)."""
-    print("case engine_wrong_prefetch", flush=True)
+    path (and that of a decode batch of up to 16 tokens) launches its kernels on table snapshots: the outputs must
+    stay the oracle's (the slot-group guard and the late classification of evicted experts are what this exercises)."""
+    print(f"case engine_wrong_prefetch T={T}", flush=True)
     Lyr, E, k, H = 3, 16, 4, 256
     layers = [Int4Layer(H=H, I=128, E=E, I_sh=128, seed=60 + l, zipf=1.1) for l in range(Lyr)]
     pm = build_engine(layers, k, cuda, cache_rate=0.3, cache_policy="lru", num_predict_expert_per_layer=k,
@@ -389,7 +390,9 @@ def test_one_token_path_under_wrong_prefetches(cuda):
     worst = 0.0
     for t in range(30):
         for l in range(Lyr):
-            x = O.synth_acts(1, H, seed=900 + t * Lyr + l)
+            # (the predictor acts on one-token steps only, as the reference's does: batches alternate with them and
+            # meet what their prefetches left behind)
+            x = O.synth_acts(T if t % 2 else 1, H, seed=900 + t * Lyr + l)
             y = pm.forward(l, torch.from_numpy(x).to(torch.bfloat16).to(cuda))
             torch.cuda.synchronize()
             ref = ref_forward(layers[l], x, k, 0)
