@@ -525,19 +525,19 @@ static void resolve_using(moe_engine *eng, Expert *v, std::unique_lock<std::mute
                std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(100)) {}
         eng->seq_pollers.fetch_sub(1, std::memory_order_acq_rel);  // sp is not read again
         if (!reached) {
-          lk.lock();
+          moe_spin_lock(lk);
           if (!eng->proof_event) eng->proof_event = eng->be->event_create();
           void *pe = eng->proof_event;
           if (pe) eng->be->event_record(pe, eng->be->compute_stream());
           lk.unlock();
           if (pe) eng->be->event_sync(pe);
         }
-        lk.lock();
+        moe_spin_lock(lk);
         if (v->status.load() == kUsing && v->seq_ptr == sp && v->seq_need == need) { v->seq_ptr = nullptr; v->status = kReady; }
         continue;
       }
       void *ev = v->event;
-      if (ev) { lk.unlock(); eng->be->event_sync(ev); lk.lock(); }
+      if (ev) { lk.unlock(); eng->be->event_sync(ev); moe_spin_lock(lk); }
       if (v->status.load() == kUsing) v->status = kReady;
       continue;
     }
@@ -547,7 +547,8 @@ static void resolve_using(moe_engine *eng, Expert *v, std::unique_lock<std::mute
 }
 
 static void fetch_thread_main(moe_engine *eng) {
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   while (!eng->exiting) {
     CopyTask t;
     if (!eng->fatal.empty() || !pop_next_task(eng, t)) {
@@ -565,7 +566,7 @@ static void fetch_thread_main(moe_engine *eng) {
 #endif
           if ((spins & 63u) == 63u && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(500)) break;
         }
-        lk.lock();
+        moe_spin_lock(lk);
       }
       if (eng->task_epoch.load(std::memory_order_acquire) == ep && !eng->exiting) eng->cv_work.wait(lk);
       continue;
@@ -591,7 +592,7 @@ static void fetch_thread_main(moe_engine *eng) {
 #if defined(__x86_64__)
           for (int i = 0; i < 32; ++i) __builtin_ia32_pause();
 #endif
-          lk.lock();
+          moe_spin_lock(lk);
         } else {
           eng->cv_state.wait_for(lk, std::chrono::microseconds(50));
         }
@@ -621,7 +622,7 @@ static void fetch_thread_main(moe_engine *eng) {
       c = c2;
     }
     if (rc == 0) rc = eng->be->copy_sync();
-    lk.lock();
+    moe_spin_lock(lk);
     if (rc != 0) engine_fail(eng, "host->slot copy failed: %s", moe_last_error());
     eng->ctr.h2d_bytes += bytes;
     eng->ctr.h2d_copies += (uint64_t)(stop - start);
@@ -807,7 +808,7 @@ extern "C" int moe_expert_param_ptr(moe_engine *eng, int layer, int expert, int 
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, expert)) return rc;
   if (!out || param_id < 0 || param_id >= eng->cfg.num_per_expert_param) { moe_set_error("bad param_id"); return MOE_EINVAL; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   Expert *e = eng->ex(layer, expert);
   *out = e->slot < 0 ? nullptr : (char *)eng->pool_base + (size_t)e->slot * eng->slot_stride + eng->chunk_off[param_id];
   return MOE_OK;
@@ -825,7 +826,7 @@ extern "C" int moe_flush_table(moe_engine *eng, int layer, void *stream) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
   if (!eng->slots_ready) { moe_set_error("slots not initialised"); return MOE_ESTATE; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   if (!eng->table_dirty[layer]) return MOE_OK;
   eng->table_dirty[layer] = 0;
   const size_t o = (size_t)layer * eng->cfg.num_expert;
@@ -836,7 +837,7 @@ int moe_flush_table_guarded(moe_engine *eng, int layer, void *stream, char *resi
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
   if (!eng->slots_ready) { moe_set_error("slots not initialised"); return MOE_ESTATE; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   const size_t o = (size_t)layer * eng->cfg.num_expert;
   if (eng->table_dirty[layer]) {
     eng->table_dirty[layer] = 0;
@@ -853,7 +854,7 @@ int moe_snapshot_table_guarded(moe_engine *eng, int layer, uint64_t *table_out, 
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
   if (!eng->slots_ready) { moe_set_error("slots not initialised"); return MOE_ESTATE; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   const size_t o = (size_t)layer * eng->cfg.num_expert;
   for (int e = 0; e < eng->cfg.num_expert; ++e) {
     table_out[e] = eng->h_table[o + e];
@@ -865,7 +866,7 @@ int moe_snapshot_table_guarded(moe_engine *eng, int layer, uint64_t *table_out, 
 
 void moe_guard_release(moe_engine *eng, int layer) {
   {
-    std::lock_guard<std::mutex> lk(eng->mu);
+    SpinGuard lk(eng->mu);
     Group &g = eng->group_of(layer);
     if (g.guard > 0) g.guard--;
   }
@@ -874,7 +875,7 @@ void moe_guard_release(moe_engine *eng, int layer) {
 
 extern "C" int moe_expert_status(moe_engine *eng, int layer, int expert) {
   if (!eng || check_le(eng, layer, expert)) return MOE_EINVAL;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   Expert *e = eng->ex(layer, expert);
   if (e->status.load() == kUsing && (e->seq_ptr ? e->seq_reached() : (!e->event || eng->be->event_done(e->event)))) {
     e->seq_ptr = nullptr;
@@ -884,12 +885,12 @@ extern "C" int moe_expert_status(moe_engine *eng, int layer, int expert) {
 }
 extern "C" int moe_is_in_cache(moe_engine *eng, int layer, int expert) {
   if (!eng || check_le(eng, layer, expert)) return MOE_EINVAL;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   return in_cache(eng, eng->ex(layer, expert)) ? 1 : 0;
 }
 extern "C" int moe_expert_num_ready(moe_engine *eng, int layer, int expert) {
   if (!eng || check_le(eng, layer, expert)) return MOE_EINVAL;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   return eng->ex(layer, expert)->num_ready;
 }
 
@@ -899,7 +900,7 @@ extern "C" int moe_expert_num_ready(moe_engine *eng, int layer, int expert) {
 int moe_report_layer_logits_bookkeeping(moe_engine *eng, int layer, int S) {
   ENG_GUARD(eng);
   if (layer < 0 || layer > eng->cfg.num_layer) { moe_set_error("bad layer %d", layer); return MOE_EINVAL; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   if (layer == 0) eng->s_seqlen.push_back((uint64_t)S);  // prefetcher.cpp:452-455
   return MOE_OK;
 }
@@ -938,7 +939,8 @@ extern "C" int moe_report_one_layer(moe_engine *eng, int layer, int64_t *ids, in
   if (int rc = check_le(eng, layer, 0)) return rc;
   if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_report_one_layer: bad ids"); return MOE_EINVAL; }
   if (!eng->launched) { moe_set_error("engine not launched"); return MOE_ESTATE; }
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   return report_one_layer_locked(eng, layer, ids, n, lk);
 }
 
@@ -969,7 +971,7 @@ static int wait_expert_locked(moe_engine *eng, Expert *e, std::unique_lock<std::
     std::this_thread::yield();
 #endif
   }
-  lk.lock();
+  moe_spin_lock(lk);
   eng->cv_state.wait(lk, [&] { return e->status.load() == kLaunching || eng->exiting || !eng->fatal.empty(); });
   eng->ctr.wait_us += (uint64_t)std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count();
   if (!eng->fatal.empty()) { moe_set_error("engine failed while waiting: %s", eng->fatal.c_str()); return MOE_ESTATE; }
@@ -980,7 +982,8 @@ extern "C" int moe_wait_expert(moe_engine *eng, int layer, int expert) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, expert)) return rc;
   if (!eng->launched) { moe_set_error("engine not launched"); return MOE_ESTATE; }
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   if (!eng->cfg.early_preempt) {  // PreemptOneExpertTask (prefetcher.cpp:225-233)
     if (int rc = preempt_one_expert(eng, layer, expert)) return rc;
     eng->cv_work.notify_all();
@@ -991,7 +994,8 @@ extern "C" int moe_wait_expert(moe_engine *eng, int layer, int expert) {
 extern "C" int moe_expert_launched(moe_engine *eng, int layer, int expert) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, expert)) return rc;
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   Expert *e = eng->ex(layer, expert);
   ENG_CHECK(eng, e->status.load() == kLaunching, "transfer launching->using, but expert %d.%d is in state %d", layer,
             expert, e->status.load());
@@ -1022,7 +1026,7 @@ static void push_forward_series(moe_engine *eng) {
 extern "C" int moe_layer_done(moe_engine *eng, int layer) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   if (!eng->cfg.early_preempt) { eng->budget++; eng->cv_sem.notify_all(); }
   if (layer == eng->cfg.num_layer - 1) push_forward_series(eng);
   return MOE_OK;
@@ -1034,7 +1038,8 @@ extern "C" int moe_acquire_layer(moe_engine *eng, int layer, int64_t *ids, int64
   if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_acquire_layer: bad ids"); return MOE_EINVAL; }
   if (!eng->launched) { moe_set_error("engine not launched"); return MOE_ESTATE; }
   {
-    std::unique_lock<std::mutex> lk(eng->mu);
+    std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
     if (int rc = report_one_layer_locked(eng, layer, ids, n, lk)) return rc;
     for (int64_t i = 0; i < n; ++i) {
       if (!eng->cfg.early_preempt) {
@@ -1051,7 +1056,7 @@ extern "C" int moe_release_experts(moe_engine *eng, int layer, const int64_t *id
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
   if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_release_experts: bad ids"); return MOE_EINVAL; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   void *ev = nullptr;
   for (int64_t i = 0; i < n; ++i) {
     if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
@@ -1074,7 +1079,7 @@ extern "C" int moe_release_experts(moe_engine *eng, int layer, const int64_t *id
 int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int64_t n, const volatile int *seq_ptr, int seq_need) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   for (int64_t i = 0; i < n; ++i) {
     if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
     Expert *x = eng->ex(layer, (int)ids[i]);
@@ -1092,7 +1097,7 @@ int moe_release_experts_seq(moe_engine *eng, int layer, const int64_t *ids, int6
 extern "C" int moe_release_layer(moe_engine *eng, int layer) {
   ENG_GUARD(eng);
   if (int rc = check_le(eng, layer, 0)) return rc;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   void *ev = nullptr;
   for (int e = 0; e < eng->cfg.num_expert; ++e) {
     Expert *x = eng->ex(layer, e);
@@ -1127,7 +1132,8 @@ int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int6
   if (int rc = check_le(eng, layer, 0)) return rc;
   if ((n > 0 && !ids) || n < 0) { moe_set_error("moe_prefetch_layer: bad ids"); return MOE_EINVAL; }
   if (!eng->launched) { moe_set_error("engine not launched"); return MOE_ESTATE; }
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   for (int64_t i = 0; i < n; ++i)
     if (ids[i] < 0 || ids[i] >= eng->cfg.num_expert) { moe_set_error("expert id out of range"); return MOE_EINVAL; }
   // run-ahead budget (worker.cpp:41-53)
@@ -1174,7 +1180,7 @@ int moe_prefetch_layer_over(moe_engine *eng, int layer, const int64_t *ids, int6
 
 extern "C" int moe_attach_predictor(moe_engine *eng, int attached) {
   ENG_GUARD(eng);
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   eng->predictor_attached = attached != 0;
   return MOE_OK;
 }
@@ -1184,7 +1190,7 @@ extern "C" int moe_update_priority(moe_engine *eng, const float *p, int n_layers
   const int L = eng->cfg.num_layer, E = eng->cfg.num_expert;
   if (!p || n_layers <= 0 || starting_layer < 0 || starting_layer + n_layers > L) { moe_set_error("moe_update_priority: bad range"); return MOE_EINVAL; }
   if (eng->cfg.cache_policy != "nn") { moe_set_error("moe_update_priority: policy is %s, not nn", eng->cfg.cache_policy.c_str()); return MOE_ESTATE; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   std::copy(p, p + (size_t)n_layers * E, eng->priority.begin() + (size_t)starting_layer * E);
   eng->max_priority = *std::max_element(eng->priority.begin(), eng->priority.end());
   std::set<Group *> gs;
@@ -1204,7 +1210,7 @@ extern "C" int moe_oracle_load(moe_engine *eng, const int64_t *entry_metas, int6
     return MOE_EINVAL;
   }
   const int L = eng->cfg.num_layer, E = eng->cfg.num_expert;
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   std::vector<int64_t> reply_len(n_seq, 0);
   for (int64_t i = 0; i < n_entries; ++i) {
     const int64_t s = entry_metas[2 * i];
@@ -1249,7 +1255,7 @@ extern "C" int moe_oracle_load(moe_engine *eng, const int64_t *entry_metas, int6
 
 extern "C" int moe_set_seq(moe_engine *eng, uint64_t seq_id) {
   ENG_GUARD(eng);
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   for (auto &g : eng->groups)
     if (int rc = g.policy->set_cur_seq(seq_id)) return rc;
   return MOE_OK;
@@ -1258,7 +1264,8 @@ extern "C" int moe_set_seq(moe_engine *eng, uint64_t seq_id) {
 extern "C" int moe_drain(moe_engine *eng) {
   ENG_GUARD(eng);
   if (!eng->launched) return MOE_OK;
-  std::unique_lock<std::mutex> lk(eng->mu);
+  std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
   eng->cv_work.notify_all();
   eng->cv_state.wait(lk, [&] {
     if (eng->exiting || !eng->fatal.empty()) return true;
@@ -1272,7 +1279,7 @@ extern "C" int moe_drain(moe_engine *eng) {
 }
 
 void engine_drop_seq_releases(moe_engine *eng) {
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   for (auto &x : eng->experts)
     if (x->seq_ptr) {
       x->seq_ptr = nullptr;
@@ -1289,7 +1296,7 @@ extern "C" int moe_streams(moe_engine *eng, void **compute, void **copy) {
 }
 
 int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n) {
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   for (int i = 0; i < n; ++i) {
     if (units[i].expert < 0 || units[i].expert >= eng->cfg.num_expert) continue;
     Expert *e = eng->ex(layer, units[i].expert);
@@ -1304,7 +1311,7 @@ int engine_account_hits(moe_engine *eng, int layer, const moe_unit *units, int n
 extern "C" int moe_get_counters(moe_engine *eng, moe_counters *out) {
   if (!eng || !out) { moe_set_error("moe_get_counters: null"); return MOE_EINVAL; }
   if (eng->fw) moe_forward_harvest(eng, true);
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   *out = eng->ctr;
   return MOE_OK;
 }
@@ -1313,7 +1320,7 @@ extern "C" int moe_get_counters(moe_engine *eng, moe_counters *out) {
 // after skipping the first `skip` prompts.
 extern "C" int moe_report(moe_engine *eng, int skip, char *buf, int buflen) {
   if (!eng || !buf || buflen <= 0) { moe_set_error("moe_report: bad argument"); return MOE_EINVAL; }
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   const size_t n = std::min(eng->s_hit.size(), eng->s_seqlen.size());
   size_t start = n;
   int seen = 0;

@@ -394,7 +394,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   // unit list; the routing comes back asynchronously and the hits are accounted when it lands.
   bool all_resident = false;
   {
-    std::lock_guard<std::mutex> lk(eng->mu);
+    SpinGuard lk(eng->mu);
     // (with a predictor attached the hooks' budget / progress bookkeeping has to run: no short cut)
     all_resident = eng->cfg.per_layer_cache && eng->cfg.early_preempt && (int)eng->group_of(layer).full_len == E &&
                    eng->layer_complete[layer] == E && !eng->predictor_attached;
@@ -525,7 +525,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_report_one_layer(eng, layer, ids.data(), n_act))) return rc;
     std::vector<int64_t> later, now_ids;
     {
-      std::lock_guard<std::mutex> lk(eng->mu);
+      SpinGuard lk(eng->mu);
       for (int i = 0; i < n_act; ++i) {
         // resident at launch and still there (now `launching`: nobody overwrites it): computed already.
         // A missed expert whose copy has landed meanwhile is `launching` too, but still has to be computed;
@@ -552,7 +552,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (spec_w2c) s->spec_state[sw] = later.empty() ? 1 : 2;
     bool late_w13_only = false;
     if (!w2c && spec_w2c) {
-      std::lock_guard<std::mutex> lk(eng->mu);
+      SpinGuard lk(eng->mu);
       late_w13_only = later.size() + now_ids.size() <= eng->group_of(layer).full_len;
     }
     if (!w2c && !late_w13_only &&
@@ -573,7 +573,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
       if (late_w13_only) {
         uint64_t addr = 0;
         {
-          std::lock_guard<std::mutex> lk(eng->mu);
+          SpinGuard lk(eng->mu);
           addr = eng->h_table[(size_t)layer * E + id];
         }
         if ((rc = moe_decode_token_late_expert_int4(x, d.H, d.I, addr, unit_of[(int)id].row0, s->h_r, s->unit_ws,
@@ -685,7 +685,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if ((rc = moe_report_one_layer(eng, layer, ids.data(), n_act))) return rc;
     std::vector<int64_t> later, now_ids;
     {
-      std::lock_guard<std::mutex> lk(eng->mu);
+      SpinGuard lk(eng->mu);
       for (int i = 0; i < n_act; ++i) {
         // resident at launch and still there (now `launching`): computed already; anything else (missed, or evicted
         // by a prefetch between the snapshot and the hooks) is computed when it is usable
@@ -709,7 +709,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
     if (!now_ids.empty()) {
       size_t slots_of_layer;
       {
-        std::lock_guard<std::mutex> lk(eng->mu);
+        SpinGuard lk(eng->mu);
         slots_of_layer = eng->group_of(layer).full_len;
       }
       rc = (size_t)n_act <= slots_of_layer && eng->cfg.per_layer_cache
@@ -830,7 +830,7 @@ extern "C" int moe_forward(moe_engine *eng, int layer, const void *x, int T, voi
   s->sub_cursor = 0;
   moe_unit *sub_h = s->units_sub_host;
   {
-    std::lock_guard<std::mutex> lk(eng->mu);
+    SpinGuard lk(eng->mu);
     for (int i = 0; i < n_act; ++i) {
       Expert *e = eng->ex(layer, (int)ids[i]);
       if (eng->cfg.early_preempt && e->status.load() == kLaunching) { sub_h[n_now++] = unit_of[(int)ids[i]]; now_ids.push_back(ids[i]); }

@@ -8,6 +8,7 @@
 #include <list>
 #include <map>
 #include <memory>
+#include <cstdlib>
 #include <mutex>
 #include <string>
 #include <thread>
@@ -134,6 +135,40 @@ struct Group {
   // > 0 while a kernel runs on a snapshot of the slot table whose selection the host does not know yet:
   // evictions go on, but no copy into a slot of this group starts (fetch thread waits)
   int guard = 0;
+};
+
+// The engine's mutex is held for a microsecond or so at a time, by three threads (the caller's, the fetch thread, the
+// predictor's).  A thread that finds it taken and sleeps on it pays the kernel's wake-up, 5 us and more, and leaves
+// the mutex in its contended state, where every unlock is a system call.  So everybody tries for a while before
+// sleeping.  MOE_LOCK_SPINS=0: sleep at once.
+static inline int moe_lock_spins() {
+  static const int n = [] { const char *e = getenv("MOE_LOCK_SPINS"); return e ? atoi(e) : 2000; }();
+  return n;
+}
+static inline void moe_spin_lock(std::mutex &m) {
+  for (int i = 0, n = moe_lock_spins(); i < n; ++i) {
+    if (m.try_lock()) return;
+#if defined(__x86_64__)
+    __builtin_ia32_pause();
+#endif
+  }
+  m.lock();
+}
+static inline void moe_spin_lock(std::unique_lock<std::mutex> &lk) {
+  for (int i = 0, n = moe_lock_spins(); i < n; ++i) {
+    if (lk.try_lock()) return;
+#if defined(__x86_64__)
+    __builtin_ia32_pause();
+#endif
+  }
+  lk.lock();
+}
+struct SpinGuard {
+  std::mutex &m;
+  explicit SpinGuard(std::mutex &mu) : m(mu) { moe_spin_lock(m); }
+  ~SpinGuard() { m.unlock(); }
+  SpinGuard(const SpinGuard &) = delete;
+  SpinGuard &operator=(const SpinGuard &) = delete;
 };
 
 struct CopyTask {

@@ -185,7 +185,7 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
         // scored against - the ranking as a whole looks good whenever the popular experts are resident.
         std::vector<int64_t> would_copy;
         {
-          std::lock_guard<std::mutex> lk(eng->mu);
+          SpinGuard lk(eng->mu);
           for (int64_t e : ids)
             if (!eng->resident.count(eng->ex(dst, (int)e))) would_copy.push_back(e);
         }
@@ -195,7 +195,8 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
       }
       {  // a copy of this layer still in flight is a leftover of the layer's previous turn and normally over
          // in a moment: give it that moment, so that the new tasks do not queue behind it for nothing
-        std::unique_lock<std::mutex> lk(eng->mu);
+        std::unique_lock<std::mutex> lk(eng->mu, std::defer_lock);
+  moe_spin_lock(lk);
         const auto t0 = std::chrono::steady_clock::now();
         while (!eng->exiting && eng->current.e && eng->current.e->layer == dst &&
                std::chrono::steady_clock::now() - t0 < std::chrono::microseconds(500))
@@ -207,7 +208,7 @@ static void predictor_loop(moe_engine *eng, PredictorState *p) {
       if (rc == MOE_ESTATE && eng->exiting) return;
       if (rc != MOE_OK) {  // keep the layer's progress in step so that report_one_layer does not wait for ever
         predictor_fail(eng, p, "prefetch_layer");
-        std::lock_guard<std::mutex> lk(eng->mu);
+        SpinGuard lk(eng->mu);
         eng->progress++;
         eng->cv_sem.notify_all();
       }
@@ -273,7 +274,7 @@ extern "C" int moe_predictor_start(moe_engine *eng) {
   }
   p->started = true;
   p->th = std::thread(predictor_loop, eng, p);
-  std::lock_guard<std::mutex> lk(eng->mu);
+  SpinGuard lk(eng->mu);
   eng->predictor_attached = true;
   return MOE_OK;
 }
